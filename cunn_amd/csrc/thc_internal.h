@@ -1,0 +1,147 @@
+// Internal C++ side of the THC shim: error plumbing, tensor metadata helpers
+// and stream-ordered temporaries used by the THNN_Cuda* wrappers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "../../include/THCUNN.h"
+
+struct THCState {
+  int device;
+  hipStream_t stream;
+};
+
+namespace thc {
+
+// ---- errors ---------------------------------------------------------------
+// THError / THArgCheck unwind to the extern "C" boundary as a C++ exception;
+// the boundary hands the text to the installed TH handler and returns.
+struct Error {
+  std::string msg;
+  int arg;  // 0: THError, >0: THArgCheck argument number
+};
+
+[[noreturn]] void error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+[[noreturn]] void argError(int arg, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void dispatchError(const Error &e);  // calls the installed handler
+
+#define THC_ARG_CHECK(cond, arg, ...) \
+  do {                                \
+    if (!(cond)) ::thc::argError(arg, __VA_ARGS__); \
+  } while (0)
+
+#define THC_HIP_CHECK(expr)                                                         \
+  do {                                                                              \
+    hipError_t err__ = (expr);                                                      \
+    if (err__ != hipSuccess)                                                        \
+      ::thc::error("HIP runtime error: %s (%s) at %s:%d", hipGetErrorString(err__), \
+                   #expr, __FILE__, __LINE__);                                      \
+  } while (0)
+
+// Wraps the body of every extern "C" entry point.
+#define THNN_ENTER try {
+#define THNN_LEAVE                    \
+  }                                   \
+  catch (const ::thc::Error &e__) {   \
+    ::thc::Error copy__ = e__;        \
+    ::thc::dispatchError(copy__);     \
+  }
+
+// ---- type-erased tensor view of THCudaTensor / THCudaLongTensor ------------
+struct Storage {
+  void *data;
+  ptrdiff_t size;
+  int refcount;
+  char flag;
+  void *allocator;
+  void *allocatorContext;
+  Storage *view;
+  int device;
+};
+struct Tensor {
+  long *size;
+  long *stride;
+  int nDimension;
+  Storage *storage;
+  ptrdiff_t storageOffset;
+  int refcount;
+  char flag;
+};
+static_assert(sizeof(Tensor) == sizeof(THCudaTensor), "layout");
+static_assert(sizeof(Storage) == sizeof(THCudaStorage), "layout");
+
+inline Tensor *erase(THCudaTensor *t) { return reinterpret_cast<Tensor *>(t); }
+inline const Tensor *erase(const THCudaTensor *t) { return reinterpret_cast<const Tensor *>(t); }
+inline Tensor *erase(THCudaLongTensor *t) { return reinterpret_cast<Tensor *>(t); }
+inline const Tensor *erase(const THCudaLongTensor *t) { return reinterpret_cast<const Tensor *>(t); }
+
+Tensor *tensorNew();
+void tensorFree(Tensor *t);
+void tensorRetain(Tensor *t);
+// TH resizeNd semantics: a tensor that already has these sizes is left alone
+// (strides included); otherwise sizes are set, strides made contiguous and the
+// storage grown (never shrunk) to hold storageOffset + numel elements.
+void tensorResize(THCState *state, Tensor *t, int nd, const long *size, size_t elemSize);
+void tensorSetView(Tensor *t, Storage *s, ptrdiff_t offset, int nd, const long *size, const long *stride);
+ptrdiff_t numel(const Tensor *t);
+bool isContiguous(const Tensor *t);
+bool sameSize(const Tensor *a, const Tensor *b);
+std::string sizeDesc(const Tensor *t);  // "[64 x 128 x 56 x 56]" as THCTensor_(sizeDesc)
+
+inline void resize(THCState *s, THCudaTensor *t, std::initializer_list<long> dims) {
+  std::vector<long> v(dims);
+  tensorResize(s, erase(t), (int)v.size(), v.data(), sizeof(float));
+}
+inline void resize(THCState *s, THCudaLongTensor *t, std::initializer_list<long> dims) {
+  std::vector<long> v(dims);
+  tensorResize(s, erase(t), (int)v.size(), v.data(), sizeof(long));
+}
+inline float *data(const THCudaTensor *t) {
+  return t->storage ? t->storage->data + t->storageOffset : nullptr;
+}
+inline long *data(const THCudaLongTensor *t) {
+  return t->storage ? t->storage->data + t->storageOffset : nullptr;
+}
+
+// strided gather src(size,stride) -> dst contiguous (or the reverse scatter)
+void stridedCopy(hipStream_t stream, const Tensor *t, void *contig, size_t elemSize, bool toContig);
+
+// Stream-ordered temporary: memory is returned to the pool after the work
+// queued so far on `stream` has drained, with no host synchronisation.
+class Temp {
+ public:
+  Temp() = default;
+  Temp(hipStream_t stream, size_t bytes);
+  Temp(Temp &&o) noexcept : p_(o.p_), stream_(o.stream_) { o.p_ = nullptr; }
+  Temp &operator=(Temp &&o) noexcept;
+  Temp(const Temp &) = delete;
+  Temp &operator=(const Temp &) = delete;
+  ~Temp();
+  void *get() const { return p_; }
+
+ private:
+  void *p_ = nullptr;
+  hipStream_t stream_ = nullptr;
+};
+
+// THCTensor_(newContiguous): the tensor's own data when it is contiguous,
+// otherwise a packed stream-ordered copy that lives as long as this object.
+class Contiguous {
+ public:
+  Contiguous(THCState *state, const THCudaTensor *t);
+  const float *ptr() const { return ptr_; }
+
+ private:
+  const float *ptr_;
+  Temp tmp_;
+};
+
+// THCUNN_check_dim_size (lib/THCUNN/common.h:69-75)
+void checkDimSize(const Tensor *t, const char *name, int dim, int dimSize, long size);
+
+}  // namespace thc

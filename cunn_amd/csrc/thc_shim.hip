@@ -1,0 +1,436 @@
+// THC shim: state, storages/tensors on hipMalloc, error hooks, strided copies.
+// This is the part of cutorch the THNN_Cuda* wrappers lean on
+// (THCTensor_(resizeNd/newContiguous/free/data/fill), THCState_getCurrentStream,
+// THError/THArgCheck); cutorch itself is not part of the reference tree.
+#include "thc_internal.h"
+
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+
+namespace thc {
+
+// ---------------------------------------------------------------- errors ----
+static void defaultErrorHandler(const char *msg, void *) {
+  fprintf(stderr, "$ Error: %s\n", msg);
+  abort();
+}
+static void defaultArgErrorHandler(int arg, const char *msg, void *) {
+  fprintf(stderr, "$ Invalid argument %d: %s\n", arg, msg ? msg : "");
+  abort();
+}
+static THErrorHandlerFunction g_errHandler = defaultErrorHandler;
+static void *g_errData = nullptr;
+static THArgErrorHandlerFunction g_argHandler = defaultArgErrorHandler;
+static void *g_argData = nullptr;
+
+static std::string vformat(const char *fmt, va_list ap) {
+  char buf[2048];
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  return std::string(buf);
+}
+
+void error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  Error e{vformat(fmt, ap), 0};
+  va_end(ap);
+  throw e;
+}
+void argError(int arg, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  Error e{vformat(fmt, ap), arg};
+  va_end(ap);
+  throw e;
+}
+void dispatchError(const Error &e) {
+  if (e.arg > 0)
+    g_argHandler(e.arg, e.msg.c_str(), g_argData);
+  else
+    g_errHandler(e.msg.c_str(), g_errData);
+}
+
+// --------------------------------------------------------------- storage ----
+static Storage *storageNew(int device) {
+  Storage *s = (Storage *)calloc(1, sizeof(Storage));
+  s->refcount = 1;
+  s->flag = TH_STORAGE_REFCOUNTED | TH_STORAGE_RESIZABLE | TH_STORAGE_FREEMEM;
+  s->device = device;
+  return s;
+}
+static void storageFree(Storage *s) {
+  if (!s) return;
+  if (--s->refcount > 0) return;
+  if ((s->flag & TH_STORAGE_FREEMEM) && s->data) (void)hipFree(s->data);
+  free(s);
+}
+static void storageGrow(THCState *state, Storage *s, ptrdiff_t elems, size_t elemSize) {
+  if (elems <= s->size) return;
+  if (!(s->flag & TH_STORAGE_RESIZABLE)) error("Trying to resize storage that is not resizable");
+  void *p = nullptr;
+  THC_HIP_CHECK(hipMalloc(&p, (size_t)elems * elemSize));
+  if (s->data && s->size > 0) {
+    // THCStorage_resize keeps the old contents
+    THC_HIP_CHECK(hipMemcpyAsync(p, s->data, (size_t)s->size * elemSize, hipMemcpyDeviceToDevice,
+                                 state->stream));
+    THC_HIP_CHECK(hipStreamSynchronize(state->stream));
+    if (s->flag & TH_STORAGE_FREEMEM) THC_HIP_CHECK(hipFree(s->data));
+  }
+  s->data = p;
+  s->size = elems;
+  s->flag |= TH_STORAGE_FREEMEM;
+}
+
+// ---------------------------------------------------------------- tensor ----
+Tensor *tensorNew() {
+  Tensor *t = (Tensor *)calloc(1, sizeof(Tensor));
+  t->refcount = 1;
+  t->flag = TH_TENSOR_REFCOUNTED;
+  return t;
+}
+void tensorRetain(Tensor *t) {
+  if (t) ++t->refcount;
+}
+void tensorFree(Tensor *t) {
+  if (!t) return;
+  if (--t->refcount > 0) return;
+  free(t->size);
+  free(t->stride);
+  storageFree(t->storage);
+  free(t);
+}
+ptrdiff_t numel(const Tensor *t) {
+  if (!t || t->nDimension == 0) return 0;
+  ptrdiff_t n = 1;
+  for (int i = 0; i < t->nDimension; ++i) n *= t->size[i];
+  return n;
+}
+bool isContiguous(const Tensor *t) {
+  long z = 1;
+  for (int d = t->nDimension - 1; d >= 0; --d) {
+    if (t->size[d] != 1) {
+      if (t->stride[d] != z) return false;
+      z *= t->size[d];
+    }
+  }
+  return true;
+}
+bool sameSize(const Tensor *a, const Tensor *b) {
+  if (a->nDimension != b->nDimension) return false;
+  for (int i = 0; i < a->nDimension; ++i)
+    if (a->size[i] != b->size[i]) return false;
+  return true;
+}
+std::string sizeDesc(const Tensor *t) {
+  std::string s = "[";
+  for (int i = 0; i < t->nDimension; ++i) {
+    s += std::to_string(t->size[i]);
+    if (i + 1 < t->nDimension) s += " x ";
+  }
+  return s + "]";
+}
+static void setDims(Tensor *t, int nd, const long *size, const long *stride) {
+  if (nd != t->nDimension) {
+    t->size = (long *)realloc(t->size, sizeof(long) * (nd > 0 ? nd : 1));
+    t->stride = (long *)realloc(t->stride, sizeof(long) * (nd > 0 ? nd : 1));
+    t->nDimension = nd;
+  }
+  long z = 1;
+  for (int d = nd - 1; d >= 0; --d) {
+    t->size[d] = size[d];
+    if (stride && stride[d] >= 0) {
+      t->stride[d] = stride[d];
+    } else {
+      t->stride[d] = z;
+    }
+    z *= size[d];
+  }
+}
+void tensorResize(THCState *state, Tensor *t, int nd, const long *size, size_t elemSize) {
+  bool same = (nd == t->nDimension);
+  for (int d = 0; same && d < nd; ++d) same = (size[d] == t->size[d]);
+  if (same) return;
+  setDims(t, nd, size, nullptr);
+  ptrdiff_t n = numel(t);
+  if (n > 0) {
+    if (!t->storage) t->storage = storageNew(state->device);
+    storageGrow(state, t->storage, n + t->storageOffset, elemSize);
+  }
+}
+void tensorSetView(Tensor *t, Storage *s, ptrdiff_t offset, int nd, const long *size, const long *stride) {
+  if (t->storage != s) {
+    storageFree(t->storage);
+    t->storage = s;
+    if (s) ++s->refcount;
+  }
+  t->storageOffset = offset;
+  setDims(t, nd, size, stride);
+}
+void checkDimSize(const Tensor *t, const char *name, int dim, int dimSize, long size) {
+  if (t->nDimension != dim || t->size[dimSize] != size) {
+    error("Need %s of dimension %d and %s.size[%d] == %ld but got %s to be of shape: %s", name, dim,
+          name, dimSize, size, name, sizeDesc(t).c_str());
+  }
+}
+
+// ----------------------------------------------------------- strided copy ----
+constexpr int kMaxDims = 8;
+struct StridedDesc {
+  long size[kMaxDims];
+  long stride[kMaxDims];
+  int nd;
+  long total;
+};
+
+template <typename T, bool TO_CONTIG>
+__global__ void __launch_bounds__(256) stridedCopyKernel(T *strided, T *contig, StridedDesc d) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < d.total;
+       i += (long)gridDim.x * blockDim.x) {
+    long rem = i, off = 0;
+    for (int k = d.nd - 1; k >= 0; --k) {
+      long q = rem / d.size[k];
+      off += (rem - q * d.size[k]) * d.stride[k];
+      rem = q;
+    }
+    if (TO_CONTIG)
+      contig[i] = strided[off];
+    else
+      strided[off] = contig[i];
+  }
+}
+
+void stridedCopy(hipStream_t stream, const Tensor *t, void *contig, size_t elemSize, bool toContig) {
+  if (t->nDimension > kMaxDims) error("tensors of more than %d dimensions are not supported", kMaxDims);
+  StridedDesc d;
+  d.nd = t->nDimension;
+  d.total = numel(t);
+  for (int i = 0; i < d.nd; ++i) {
+    d.size[i] = t->size[i];
+    d.stride[i] = t->stride[i];
+  }
+  if (d.total == 0) return;
+  long blocks = (d.total + 255) / 256;
+  if (blocks > 65535 * 16) blocks = 65535 * 16;
+  void *base = (char *)t->storage->data + (size_t)t->storageOffset * elemSize;
+  if (elemSize == 4) {
+    if (toContig)
+      stridedCopyKernel<uint32_t, true><<<(unsigned)blocks, 256, 0, stream>>>((uint32_t *)base, (uint32_t *)contig, d);
+    else
+      stridedCopyKernel<uint32_t, false><<<(unsigned)blocks, 256, 0, stream>>>((uint32_t *)base, (uint32_t *)contig, d);
+  } else {
+    if (toContig)
+      stridedCopyKernel<uint64_t, true><<<(unsigned)blocks, 256, 0, stream>>>((uint64_t *)base, (uint64_t *)contig, d);
+    else
+      stridedCopyKernel<uint64_t, false><<<(unsigned)blocks, 256, 0, stream>>>((uint64_t *)base, (uint64_t *)contig, d);
+  }
+  THC_HIP_CHECK(hipGetLastError());
+}
+
+// ------------------------------------------------------------ temporaries ----
+Temp::Temp(hipStream_t stream, size_t bytes) : stream_(stream) {
+  if (bytes == 0) return;
+  THC_HIP_CHECK(hipMallocAsync(&p_, bytes, stream));
+}
+Temp &Temp::operator=(Temp &&o) noexcept {
+  if (this != &o) {
+    if (p_) (void)hipFreeAsync(p_, stream_);
+    p_ = o.p_;
+    stream_ = o.stream_;
+    o.p_ = nullptr;
+  }
+  return *this;
+}
+Temp::~Temp() {
+  if (p_) (void)hipFreeAsync(p_, stream_);
+}
+
+Contiguous::Contiguous(THCState *state, const THCudaTensor *t) {
+  const Tensor *e = erase(t);
+  if (isContiguous(e)) {
+    ptr_ = data(t);
+    return;
+  }
+  tmp_ = Temp(state->stream, (size_t)numel(e) * sizeof(float));
+  stridedCopy(state->stream, e, tmp_.get(), sizeof(float), true);
+  ptr_ = (const float *)tmp_.get();
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) fillKernel(T *p, long n, T v) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+    p[i] = v;
+}
+
+// ------------------------------------------------------ generic C helpers ----
+static Tensor *newWithSize(THCState *state, int nd, const long *size, size_t elemSize) {
+  Tensor *t = tensorNew();
+  if (nd > 0) tensorResize(state, t, nd, size, elemSize);
+  return t;
+}
+static Tensor *newWithData(THCState *state, void *devPtr, ptrdiff_t capacity, ptrdiff_t offset, int nd,
+                           const long *size, const long *stride) {
+  Storage *s = (Storage *)calloc(1, sizeof(Storage));
+  s->refcount = 1;
+  s->flag = TH_STORAGE_REFCOUNTED;  // neither resizable nor owned
+  s->data = devPtr;
+  s->size = capacity;
+  s->device = state->device;
+  Tensor *t = tensorNew();
+  tensorSetView(t, s, offset, nd, size, stride);
+  storageFree(s);  // the tensor holds the only reference now
+  return t;
+}
+static void copyHost(THCState *state, Tensor *t, void *host, size_t elemSize, bool toHost) {
+  ptrdiff_t n = numel(t);
+  if (n == 0) return;
+  size_t bytes = (size_t)n * elemSize;
+  void *base = (char *)t->storage->data + (size_t)t->storageOffset * elemSize;
+  if (isContiguous(t)) {
+    if (toHost) {
+      THC_HIP_CHECK(hipStreamSynchronize(state->stream));
+      THC_HIP_CHECK(hipMemcpy(host, base, bytes, hipMemcpyDeviceToHost));
+    } else {
+      THC_HIP_CHECK(hipMemcpy(base, host, bytes, hipMemcpyHostToDevice));
+    }
+    return;
+  }
+  void *tmp = nullptr;
+  THC_HIP_CHECK(hipMalloc(&tmp, bytes));
+  if (toHost) {
+    stridedCopy(state->stream, t, tmp, elemSize, true);
+    THC_HIP_CHECK(hipStreamSynchronize(state->stream));
+    THC_HIP_CHECK(hipMemcpy(host, tmp, bytes, hipMemcpyDeviceToHost));
+  } else {
+    THC_HIP_CHECK(hipMemcpy(tmp, host, bytes, hipMemcpyHostToDevice));
+    stridedCopy(state->stream, t, tmp, elemSize, false);
+    THC_HIP_CHECK(hipStreamSynchronize(state->stream));
+  }
+  THC_HIP_CHECK(hipFree(tmp));
+}
+
+}  // namespace thc
+
+using namespace thc;
+
+// =============================================================== C API =======
+extern "C" {
+
+THCState *THCState_alloc(void) {
+  THCState *s = nullptr;
+  THNN_ENTER
+  s = (THCState *)calloc(1, sizeof(THCState));
+  THC_HIP_CHECK(hipGetDevice(&s->device));
+  s->stream = nullptr;  // the device's default stream
+  THNN_LEAVE
+  return s;
+}
+void THCState_free(THCState *state) { free(state); }
+void THCState_setCurrentStream(THCState *state, void *hipStream) { state->stream = (hipStream_t)hipStream; }
+void *THCState_getCurrentStream(THCState *state) { return (void *)state->stream; }
+void THCState_synchronize(THCState *state) {
+  THNN_ENTER
+  THC_HIP_CHECK(hipStreamSynchronize(state->stream));
+  THNN_LEAVE
+}
+
+void THSetErrorHandler(THErrorHandlerFunction handler, void *data) {
+  g_errHandler = handler ? handler : defaultErrorHandler;
+  g_errData = data;
+}
+void THSetArgErrorHandler(THArgErrorHandlerFunction handler, void *data) {
+  g_argHandler = handler ? handler : defaultArgErrorHandler;
+  g_argData = data;
+}
+
+// ---- float tensors
+THCudaTensor *THCudaTensor_new(THCState *) { return (THCudaTensor *)tensorNew(); }
+THCudaTensor *THCudaTensor_newWithSize(THCState *state, int nd, const long *size) {
+  Tensor *t = nullptr;
+  THNN_ENTER
+  t = newWithSize(state, nd, size, sizeof(float));
+  THNN_LEAVE
+  return (THCudaTensor *)t;
+}
+THCudaTensor *THCudaTensor_newWithData(THCState *state, float *devPtr, ptrdiff_t capacity, ptrdiff_t offset,
+                                       int nd, const long *size, const long *stride) {
+  return (THCudaTensor *)newWithData(state, devPtr, capacity, offset, nd, size, stride);
+}
+THCudaTensor *THCudaTensor_newView(THCState *, THCudaTensor *src, ptrdiff_t offset, int nd, const long *size,
+                                   const long *stride) {
+  Tensor *t = tensorNew();
+  tensorSetView(t, erase(src)->storage, offset, nd, size, stride);
+  return (THCudaTensor *)t;
+}
+void THCudaTensor_retain(THCState *, THCudaTensor *self) { tensorRetain(erase(self)); }
+void THCudaTensor_free(THCState *, THCudaTensor *self) { tensorFree(erase(self)); }
+void THCudaTensor_resizeNd(THCState *state, THCudaTensor *self, int nd, const long *size) {
+  THNN_ENTER
+  tensorResize(state, erase(self), nd, size, sizeof(float));
+  THNN_LEAVE
+}
+float *THCudaTensor_data(THCState *, const THCudaTensor *self) { return data(self); }
+int THCudaTensor_nDimension(THCState *, const THCudaTensor *self) { return self->nDimension; }
+long THCudaTensor_size(THCState *, const THCudaTensor *self, int dim) { return self->size[dim]; }
+long THCudaTensor_stride(THCState *, const THCudaTensor *self, int dim) { return self->stride[dim]; }
+ptrdiff_t THCudaTensor_nElement(THCState *, const THCudaTensor *self) { return numel(erase(self)); }
+int THCudaTensor_isContiguous(THCState *, const THCudaTensor *self) { return isContiguous(erase(self)); }
+void THCudaTensor_fill(THCState *state, THCudaTensor *self, float value) {
+  THNN_ENTER
+  Tensor *t = erase(self);
+  ptrdiff_t n = numel(t);
+  if (n == 0) return;
+  if (!isContiguous(t)) error("fill: contiguous tensor expected");
+  long blocks = (n + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  fillKernel<float><<<(unsigned)blocks, 256, 0, state->stream>>>(data(self), n, value);
+  THC_HIP_CHECK(hipGetLastError());
+  THNN_LEAVE
+}
+void THCudaTensor_copyFromHost(THCState *state, THCudaTensor *self, const float *src) {
+  THNN_ENTER
+  copyHost(state, erase(self), (void *)src, sizeof(float), false);
+  THNN_LEAVE
+}
+void THCudaTensor_copyToHost(THCState *state, THCudaTensor *self, float *dst) {
+  THNN_ENTER
+  copyHost(state, erase(self), dst, sizeof(float), true);
+  THNN_LEAVE
+}
+
+// ---- int64 tensors
+THCudaLongTensor *THCudaLongTensor_new(THCState *) { return (THCudaLongTensor *)tensorNew(); }
+THCudaLongTensor *THCudaLongTensor_newWithSize(THCState *state, int nd, const long *size) {
+  Tensor *t = nullptr;
+  THNN_ENTER
+  t = newWithSize(state, nd, size, sizeof(long));
+  THNN_LEAVE
+  return (THCudaLongTensor *)t;
+}
+THCudaLongTensor *THCudaLongTensor_newWithData(THCState *state, long *devPtr, ptrdiff_t capacity,
+                                               ptrdiff_t offset, int nd, const long *size,
+                                               const long *stride) {
+  return (THCudaLongTensor *)newWithData(state, devPtr, capacity, offset, nd, size, stride);
+}
+void THCudaLongTensor_free(THCState *, THCudaLongTensor *self) { tensorFree(erase(self)); }
+void THCudaLongTensor_resizeNd(THCState *state, THCudaLongTensor *self, int nd, const long *size) {
+  THNN_ENTER
+  tensorResize(state, erase(self), nd, size, sizeof(long));
+  THNN_LEAVE
+}
+long *THCudaLongTensor_data(THCState *, const THCudaLongTensor *self) { return data(self); }
+int THCudaLongTensor_nDimension(THCState *, const THCudaLongTensor *self) { return self->nDimension; }
+long THCudaLongTensor_size(THCState *, const THCudaLongTensor *self, int dim) { return self->size[dim]; }
+ptrdiff_t THCudaLongTensor_nElement(THCState *, const THCudaLongTensor *self) { return numel(erase(self)); }
+void THCudaLongTensor_copyFromHost(THCState *state, THCudaLongTensor *self, const long *src) {
+  THNN_ENTER
+  copyHost(state, erase(self), (void *)src, sizeof(long), false);
+  THNN_LEAVE
+}
+void THCudaLongTensor_copyToHost(THCState *state, THCudaLongTensor *self, long *dst) {
+  THNN_ENTER
+  copyHost(state, erase(self), dst, sizeof(long), true);
+  THNN_LEAVE
+}
+
+}  // extern "C"

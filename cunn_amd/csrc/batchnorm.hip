@@ -1,0 +1,500 @@
+// BatchNormalization (1-D/2-D/3-D share it: the input is viewed as N x C x L,
+// lib/THCUNN/generic/BatchNormalization.cu:8-32) for gfx950.
+//
+// The reference gives one workgroup a whole channel and walks the batch
+// serially three times (lib/THCUNN/BatchNormalization.cu:166-212). With 256 CUs
+// and typically a few hundred channels that leaves the chip idle, so here a
+// channel is cut into chunks (a few whole planes, or a segment of a large
+// plane) and every pass is a grid of C x chunks workgroups streaming 16-byte
+// loads:
+//   statistics:  per chunk (count, mean, M2) from shifted sums, reduced with a
+//                64-lane shuffle tree + LDS; chunks are merged with Chan's
+//                formula in double, in a fixed order, by every workgroup of
+//                the channel (no atomics, no extra launch, deterministic)
+//   apply:       y = gamma * (x - mean) * invStd + beta on the same chunking.
+// Backward mirrors it with the fused (sum gy, sum gy*(x-mean)) reduction of
+// lib/THCUNN/BatchNormalization.cu:214-283.
+#include <cmath>
+
+#include "device_utils.h"
+#include "launch_utils.h"
+#include "thc_internal.h"
+
+using namespace thc;
+
+namespace {
+
+struct BnGeom {
+  int N, C, L;
+  int planesPerChunk;  // whole planes a chunk covers (1 when planes are segmented)
+  int segsPerPlane;    // segments a plane is cut into
+  int segLen;          // elements per segment (multiple of 4 when vectorised)
+  int chunks;          // chunks per channel = ceil(N / planesPerChunk) * segsPerPlane
+};
+
+struct Chunk {
+  int n0, nN;  // planes [n0, n0 + nN)
+  int l0, lN;  // elements [l0, l0 + lN) of each plane
+};
+
+__device__ __forceinline__ Chunk chunkOf(const BnGeom &g, int chunk) {
+  int nb = chunk / g.segsPerPlane, sg = chunk - nb * g.segsPerPlane;
+  Chunk c;
+  c.n0 = nb * g.planesPerChunk;
+  c.nN = min(g.planesPerChunk, g.N - c.n0);
+  c.l0 = sg * g.segLen;
+  c.lN = min(g.segLen, g.L - c.l0);
+  return c;
+}
+
+// Visits every element of a chunk of channel `ch`: f(offset, width) is called
+// with the flat offset into the (N,C,L) tensor of `width` (4 or 1) consecutive
+// elements.
+template <bool VEC, typename F>
+__device__ __forceinline__ void forChunk(const BnGeom &g, int ch, const Chunk &c, F f) {
+  if (VEC) {
+    const int seg4 = c.lN >> 2;
+    const int total = c.nN * seg4;
+    for (int i = threadIdx.x; i < total; i += blockDim.x) {
+      int n = i / seg4, l4 = i - n * seg4;
+      f(((long)(c.n0 + n) * g.C + ch) * g.L + c.l0 + (l4 << 2));
+    }
+  } else {
+    const int total = c.nN * c.lN;
+    for (int i = threadIdx.x; i < total; i += blockDim.x) {
+      int n = i / c.lN, l = i - n * c.lN;
+      f(((long)(c.n0 + n) * g.C + ch) * g.L + c.l0 + l);
+    }
+  }
+}
+
+template <int NV>
+__device__ __forceinline__ void blockSum(float (&v)[NV], float (*red)[NV]) {
+  const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    v[k] = dev::waveSum(v[k]);
+    if (lane == 0) red[wave][k] = v[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < dev::kBlock / dev::kWave; ++w) s += red[w][k];
+    v[k] = s;
+  }
+}
+
+// ------------------------------------------------------ forward statistics ----
+// partial[(ch * chunks + chunk) * 3 + {0,1,2}] = count, mean, M2 of the chunk
+template <bool VEC>
+__global__ void __launch_bounds__(dev::kBlock)
+bnStatsKernel(const float *__restrict__ x, float *__restrict__ partial, BnGeom g) {
+  __shared__ float red[dev::kBlock / dev::kWave][2];
+  const int ch = blockIdx.x / g.chunks, chunk = blockIdx.x - ch * g.chunks;
+  const Chunk c = chunkOf(g, chunk);
+  // sums are taken about the chunk's first element so that E[d^2] - E[d]^2 does
+  // not cancel when |mean| >> sigma
+  const float shift = x[((long)c.n0 * g.C + ch) * g.L + c.l0];
+  float v[2] = {0.f, 0.f};
+  forChunk<VEC>(g, ch, c, [&](long off) {
+    if (VEC) {
+      float4 q = *reinterpret_cast<const float4 *>(x + off);
+      float d0 = q.x - shift, d1 = q.y - shift, d2 = q.z - shift, d3 = q.w - shift;
+      v[0] += (d0 + d1) + (d2 + d3);
+      v[1] += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+    } else {
+      float d = x[off] - shift;
+      v[0] += d;
+      v[1] += d * d;
+    }
+  });
+  blockSum<2>(v, red);
+  if (threadIdx.x == 0) {
+    float cnt = (float)c.nN * (float)c.lN;
+    float *p = partial + ((long)ch * g.chunks + chunk) * 3;
+    p[0] = cnt;
+    p[1] = shift + v[0] / cnt;
+    p[2] = fmaxf(v[1] - v[0] * v[0] / cnt, 0.f);
+  }
+}
+
+// Chan et al. pairwise merge of (n, mean, M2), lanes of wave 0 stride the chunk
+// list, then a shuffle tree; every lane ends with the channel totals.
+__device__ __forceinline__ void mergeStats(const float *__restrict__ p, int chunks, double &n, double &mean,
+                                           double &m2) {
+  const int lane = threadIdx.x % dev::kWave;
+  n = 0.0, mean = 0.0, m2 = 0.0;
+  for (int k = lane; k < chunks; k += dev::kWave) {
+    double nb = p[k * 3], mb = p[k * 3 + 1], qb = p[k * 3 + 2];
+    double tot = n + nb, d = mb - mean;
+    mean += d * (nb / tot);
+    m2 += qb + d * d * (n * nb / tot);
+    n = tot;
+  }
+#pragma unroll
+  for (int o = dev::kWave / 2; o > 0; o >>= 1) {
+    double nb = __shfl_xor(n, o, dev::kWave), mb = __shfl_xor(mean, o, dev::kWave),
+           qb = __shfl_xor(m2, o, dev::kWave);
+    double tot = n + nb;
+    if (tot > 0.0) {
+      // symmetric form so that both partners compute bit-identical results
+      double ma = mean, d = mb - ma;
+      mean = (ma * n + mb * nb) / tot;
+      m2 = m2 + qb + d * d * (n * nb / tot);
+      n = tot;
+    }
+  }
+}
+
+// ------------------------------------------------------------ forward apply ----
+// TRAIN: merges the chunk statistics, publishes saveMean/saveStd/running stats
+// (chunk 0 only) and normalises; otherwise uses the running statistics.
+template <bool TRAIN, bool VEC>
+__global__ void __launch_bounds__(dev::kBlock)
+bnApplyKernel(const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ partial,
+              const float *__restrict__ weight, const float *__restrict__ bias, float *__restrict__ runningMean,
+              float *__restrict__ runningVar, float *__restrict__ saveMean, float *__restrict__ saveStd, BnGeom g,
+              float momentum, float eps) {
+  __shared__ float bc[2];
+  const int ch = blockIdx.x / g.chunks, chunk = blockIdx.x - ch * g.chunks;
+  float mean, invStd;
+  if (TRAIN) {
+    if (threadIdx.x < dev::kWave) {
+      double n, m, m2;
+      mergeStats(partial + (long)ch * g.chunks * 3, g.chunks, n, m, m2);
+      if (threadIdx.x == 0) {
+        // lib/THCUNN/BatchNormalization.cu:181-200, in the Cuda type's float accreal
+        float meanF = (float)m, varN = (float)m2, norm = 1.f / (float)n;
+        float inv = 0.f;
+        if (varN != 0.f || eps != 0.f) inv = 1.f / sqrtf(varN * norm + eps);
+        bc[0] = meanF;
+        bc[1] = inv;
+        if (chunk == 0) {
+          float unbiased = varN / ((float)n - 1.f);
+          saveMean[ch] = meanF;
+          saveStd[ch] = inv;
+          runningMean[ch] = (1.f - momentum) * runningMean[ch] + momentum * meanF;
+          runningVar[ch] = (1.f - momentum) * runningVar[ch] + momentum * unbiased;
+        }
+      }
+    }
+    __syncthreads();
+    mean = bc[0];
+    invStd = bc[1];
+  } else {
+    mean = runningMean[ch];
+    invStd = 1.f / sqrtf(runningVar[ch] + eps);
+  }
+  const float gamma = weight ? weight[ch] : 1.f, beta = bias ? bias[ch] : 0.f;
+  const Chunk c = chunkOf(g, chunk);
+  forChunk<VEC>(g, ch, c, [&](long off) {
+    if (VEC) {
+      float4 q = *reinterpret_cast<const float4 *>(x + off), r;
+      r.x = gamma * (q.x - mean) * invStd + beta;
+      r.y = gamma * (q.y - mean) * invStd + beta;
+      r.z = gamma * (q.z - mean) * invStd + beta;
+      r.w = gamma * (q.w - mean) * invStd + beta;
+      *reinterpret_cast<float4 *>(y + off) = r;
+    } else {
+      y[off] = gamma * (x[off] - mean) * invStd + beta;
+    }
+  });
+}
+
+// ----------------------------------------------------------- backward sums ----
+// partial[(ch * chunks + chunk) * 2 + {0,1}] = sum gy, sum gy * (x - mean)
+template <bool VEC>
+__global__ void __launch_bounds__(dev::kBlock)
+bnGradSumsKernel(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ partial,
+                 const float *__restrict__ meanSrc, BnGeom g) {
+  __shared__ float red[dev::kBlock / dev::kWave][2];
+  const int ch = blockIdx.x / g.chunks, chunk = blockIdx.x - ch * g.chunks;
+  const Chunk c = chunkOf(g, chunk);
+  const float mean = meanSrc[ch];
+  float v[2] = {0.f, 0.f};
+  forChunk<VEC>(g, ch, c, [&](long off) {
+    if (VEC) {
+      float4 q = *reinterpret_cast<const float4 *>(x + off);
+      float4 d = *reinterpret_cast<const float4 *>(gy + off);
+      v[0] += (d.x + d.y) + (d.z + d.w);
+      v[1] += (d.x * (q.x - mean) + d.y * (q.y - mean)) + (d.z * (q.z - mean) + d.w * (q.w - mean));
+    } else {
+      float d = gy[off];
+      v[0] += d;
+      v[1] += d * (x[off] - mean);
+    }
+  });
+  blockSum<2>(v, red);
+  if (threadIdx.x == 0) {
+    float *p = partial + ((long)ch * g.chunks + chunk) * 2;
+    p[0] = v[0];
+    p[1] = v[1];
+  }
+}
+
+__device__ __forceinline__ void mergeSums(const float *__restrict__ p, int chunks, double &s0, double &s1) {
+  const int lane = threadIdx.x % dev::kWave;
+  s0 = 0.0, s1 = 0.0;
+  for (int k = lane; k < chunks; k += dev::kWave) {
+    s0 += p[k * 2];
+    s1 += p[k * 2 + 1];
+  }
+#pragma unroll
+  for (int o = dev::kWave / 2; o > 0; o >>= 1) {
+    s0 += __shfl_xor(s0, o, dev::kWave);
+    s1 += __shfl_xor(s1, o, dev::kWave);
+  }
+}
+
+// ---------------------------------------------------------- backward apply ----
+// lib/THCUNN/BatchNormalization.cu:253-282. HAVE_SUMS: partial holds the chunk
+// sums (needed for train-mode gradInput and for gradWeight/gradBias).
+template <bool TRAIN, bool VEC>
+__global__ void __launch_bounds__(dev::kBlock)
+bnBackwardKernel(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
+                 const float *__restrict__ partial, float *__restrict__ gradWeight, float *__restrict__ gradBias,
+                 const float *__restrict__ weight, const float *__restrict__ meanSrc,
+                 const float *__restrict__ stdSrc, BnGeom g, float scale, float eps) {
+  __shared__ float bc[2];
+  const int ch = blockIdx.x / g.chunks, chunk = blockIdx.x - ch * g.chunks;
+  const float mean = meanSrc[ch];
+  const float stdVal = TRAIN ? stdSrc[ch] : 1.f / sqrtf(stdSrc[ch] + eps);
+  const float weightVal = weight ? weight[ch] : 1.f;
+  float gradOutputSum = 0.f, dotP = 0.f;
+  if (partial) {
+    if (threadIdx.x < dev::kWave) {
+      double s0, s1;
+      mergeSums(partial + (long)ch * g.chunks * 2, g.chunks, s0, s1);
+      if (threadIdx.x == 0) {
+        bc[0] = (float)s0;
+        bc[1] = (float)s1;
+      }
+    }
+    __syncthreads();
+    gradOutputSum = bc[0];
+    dotP = bc[1];
+  }
+  const float norm = 1.f / ((float)g.N * (float)g.L);
+  const float gradMean = gradOutputSum * norm;
+  const float projScale = dotP * norm * stdVal * stdVal;
+  const float gradScale = stdVal * weightVal;
+  if (gx) {
+    const Chunk c = chunkOf(g, chunk);
+    forChunk<VEC>(g, ch, c, [&](long off) {
+      if (VEC) {
+        float4 d = *reinterpret_cast<const float4 *>(gy + off), r;
+        if (TRAIN) {
+          float4 q = *reinterpret_cast<const float4 *>(x + off);
+          r.x = (d.x - (q.x - mean) * projScale - gradMean) * gradScale;
+          r.y = (d.y - (q.y - mean) * projScale - gradMean) * gradScale;
+          r.z = (d.z - (q.z - mean) * projScale - gradMean) * gradScale;
+          r.w = (d.w - (q.w - mean) * projScale - gradMean) * gradScale;
+        } else {
+          r.x = d.x * gradScale, r.y = d.y * gradScale, r.z = d.z * gradScale, r.w = d.w * gradScale;
+        }
+        *reinterpret_cast<float4 *>(gx + off) = r;
+      } else {
+        if (TRAIN)
+          gx[off] = (gy[off] - (x[off] - mean) * projScale - gradMean) * gradScale;
+        else
+          gx[off] = gy[off] * gradScale;
+      }
+    });
+  }
+  if (chunk == 0 && threadIdx.x == 0) {
+    if (gradWeight) gradWeight[ch] += scale * dotP * stdVal;
+    if (gradBias) gradBias[ch] += scale * gradOutputSum;
+  }
+}
+
+// -------------------------------------------------------------- host side ----
+struct BnView {
+  BnGeom g;
+  bool vec;
+};
+
+// N x C x L view of the input (lib/THCUNN/generic/BatchNormalization.cu:8-32)
+// and the chunking policy.
+BnView bnView(const THCudaTensor *t, std::initializer_list<const void *> ptrs) {
+  const Tensor *e = erase(t);
+  THC_ARG_CHECK(e->nDimension >= 2, 2, "input of at least 2 dimensions (batch x features) expected, got: %s",
+                sizeDesc(e).c_str());
+  BnView v;
+  BnGeom &g = v.g;
+  long L = 1;
+  for (int i = 2; i < e->nDimension; ++i) L *= e->size[i];
+  if (e->size[0] >= 0x7fffffffL || e->size[1] >= 0x7fffffffL || L >= 0x7fffffffL)
+    error("BatchNormalization: dimensions of 2^31 or more elements are not supported");
+  g.N = (int)e->size[0], g.C = (int)e->size[1], g.L = (int)L;
+  v.vec = g.L % 4 == 0;
+  for (const void *p : ptrs) v.vec = v.vec && (p == nullptr || launch::aligned16(p));
+  // ~8K elements (32 KB) per workgroup: 8 x 16-byte loads per lane
+  const int target = 8192;
+  if (g.L >= target) {
+    g.planesPerChunk = 1;
+    g.segsPerPlane = launch::ceilDiv(g.L, target);
+    g.segLen = launch::roundUp(launch::ceilDiv(g.L, g.segsPerPlane), 4);
+    g.segsPerPlane = launch::ceilDiv(g.L, g.segLen);
+  } else {
+    g.segsPerPlane = 1;
+    g.segLen = g.L;
+    g.planesPerChunk = std::max(1, std::min(g.N, target / std::max(g.L, 1)));
+    // keep at least ~2048 workgroups in flight when the batch allows it
+    while (g.planesPerChunk > 1 && (long)g.C * launch::ceilDiv(g.N, g.planesPerChunk) < launch::kMinBlocks)
+      g.planesPerChunk = (g.planesPerChunk + 1) / 2;
+  }
+  g.chunks = launch::ceilDiv(g.N, g.planesPerChunk) * g.segsPerPlane;
+  return v;
+}
+
+void checkVector(const THCudaTensor *t, const char *name, int C, bool required) {
+  if (!t) {
+    if (required) error("%s tensor expected", name);
+    return;
+  }
+  const Tensor *e = erase(t);
+  if (numel(e) != C || !isContiguous(e))
+    error("%s must be a contiguous vector of %d elements, got: %s", name, C, sizeDesc(e).c_str());
+}
+
+inline float *dataOrNull(const THCudaTensor *t) { return t ? data(t) : nullptr; }
+
+}  // namespace
+
+extern "C" {
+
+void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *input_, THCudaTensor *output_,
+                                              THCudaTensor *weight_, THCudaTensor *bias_,
+                                              THCudaTensor *runningMean_, THCudaTensor *runningVar_,
+                                              THCudaTensor *saveMean_, THCudaTensor *saveStd_, bool train,
+                                              double momentum, double eps) {
+  THNN_ENTER
+  THC_ARG_CHECK(input_ != nullptr, 2, "input tensor expected");
+  THC_ARG_CHECK(output_ != nullptr, 3, "output tensor expected");
+  tensorResize(state, erase(output_), input_->nDimension, input_->size, sizeof(float));  // resizeAs (:40)
+  if (!isContiguous(erase(output_))) error("output tensor has to be contiguous");
+  Contiguous in(state, input_);
+  BnView v = bnView(input_, {in.ptr(), data(output_)});
+  const BnGeom &g = v.g;
+  checkVector(weight_, "weight", g.C, false);
+  checkVector(bias_, "bias", g.C, false);
+  checkVector(runningMean_, "runningMean", g.C, true);
+  checkVector(runningVar_, "runningVar", g.C, true);
+  if (train) {
+    checkVector(saveMean_, "saveMean", g.C, true);
+    checkVector(saveStd_, "saveStd", g.C, true);
+  }
+  if ((long)g.N * g.C * g.L == 0) return;
+  if ((long)g.C * g.chunks >= 0x7fffffffL) error("BatchNormalization: grid too large");
+  hipStream_t s = state->stream;
+  dim3 grid((unsigned)(g.C * g.chunks)), block(dev::kBlock);
+  if (train) {
+    Temp partial(s, (size_t)g.C * g.chunks * 3 * sizeof(float));
+    float *p = (float *)partial.get();
+    if (v.vec) {
+      bnStatsKernel<true><<<grid, block, 0, s>>>(in.ptr(), p, g);
+      bnApplyKernel<true, true><<<grid, block, 0, s>>>(in.ptr(), data(output_), p, dataOrNull(weight_),
+                                                       dataOrNull(bias_), data(runningMean_), data(runningVar_),
+                                                       data(saveMean_), data(saveStd_), g, (float)momentum,
+                                                       (float)eps);
+    } else {
+      bnStatsKernel<false><<<grid, block, 0, s>>>(in.ptr(), p, g);
+      bnApplyKernel<true, false><<<grid, block, 0, s>>>(in.ptr(), data(output_), p, dataOrNull(weight_),
+                                                        dataOrNull(bias_), data(runningMean_), data(runningVar_),
+                                                        data(saveMean_), data(saveStd_), g, (float)momentum,
+                                                        (float)eps);
+    }
+  } else {
+    if (v.vec)
+      bnApplyKernel<false, true><<<grid, block, 0, s>>>(in.ptr(), data(output_), nullptr, dataOrNull(weight_),
+                                                        dataOrNull(bias_), data(runningMean_), data(runningVar_),
+                                                        nullptr, nullptr, g, (float)momentum, (float)eps);
+    else
+      bnApplyKernel<false, false><<<grid, block, 0, s>>>(in.ptr(), data(output_), nullptr, dataOrNull(weight_),
+                                                         dataOrNull(bias_), data(runningMean_), data(runningVar_),
+                                                         nullptr, nullptr, g, (float)momentum, (float)eps);
+  }
+  THC_HIP_CHECK(hipGetLastError());
+  THNN_LEAVE
+}
+
+void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_, THCudaTensor *gradOutput_,
+                                          THCudaTensor *gradInput_, THCudaTensor *gradWeight_,
+                                          THCudaTensor *gradBias_, THCudaTensor *weight_,
+                                          THCudaTensor *runningMean_, THCudaTensor *runningVar_,
+                                          THCudaTensor *saveMean_, THCudaTensor *saveStd_, bool train, double scale,
+                                          double eps) {
+  THNN_ENTER
+  THC_ARG_CHECK(input_ != nullptr, 2, "input tensor expected");
+  THC_ARG_CHECK(gradOutput_ != nullptr, 3, "gradOutput tensor expected");
+  if (!sameSize(erase(input_), erase(gradOutput_)))  // THCUNN_check_shape (:74)
+    error("input_ and gradOutput_ shapes do not match: input_ %s, gradOutput_ %s", sizeDesc(erase(input_)).c_str(),
+          sizeDesc(erase(gradOutput_)).c_str());
+  if (gradInput_) {
+    // the reference writes through gradInput as it finds it; a tensor of another
+    // shape would be written out of bounds there, here it is an error
+    if (!sameSize(erase(input_), erase(gradInput_)))
+      error("input_ and gradInput_ shapes do not match: input_ %s, gradInput_ %s", sizeDesc(erase(input_)).c_str(),
+            sizeDesc(erase(gradInput_)).c_str());
+    if (!isContiguous(erase(gradInput_))) error("gradInput tensor has to be contiguous");
+  }
+  Contiguous in(state, input_);
+  Contiguous go(state, gradOutput_);
+  BnView v = bnView(input_, {in.ptr(), go.ptr(), gradInput_ ? data(gradInput_) : nullptr});
+  const BnGeom &g = v.g;
+  checkVector(gradWeight_, "gradWeight", g.C, false);
+  checkVector(gradBias_, "gradBias", g.C, false);
+  checkVector(weight_, "weight", g.C, false);
+  if (train) {
+    checkVector(saveMean_, "saveMean", g.C, true);
+    checkVector(saveStd_, "saveStd", g.C, true);
+  } else {
+    checkVector(runningMean_, "runningMean", g.C, true);
+    checkVector(runningVar_, "runningVar", g.C, true);
+  }
+  if ((long)g.N * g.C * g.L == 0) return;
+  if (!gradInput_ && !gradWeight_ && !gradBias_) return;
+  if ((long)g.C * g.chunks >= 0x7fffffffL) error("BatchNormalization: grid too large");
+  hipStream_t s = state->stream;
+  dim3 grid((unsigned)(g.C * g.chunks)), block(dev::kBlock);
+  const float *meanSrc = train ? data(saveMean_) : data(runningMean_);
+  const float *stdSrc = train ? data(saveStd_) : data(runningVar_);
+  const bool needSums = (train && gradInput_) || gradWeight_ || gradBias_;
+  Temp partial;
+  float *p = nullptr;
+  if (needSums) {
+    partial = Temp(s, (size_t)g.C * g.chunks * 2 * sizeof(float));
+    p = (float *)partial.get();
+    if (v.vec)
+      bnGradSumsKernel<true><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g);
+    else
+      bnGradSumsKernel<false><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g);
+    THC_HIP_CHECK(hipGetLastError());
+  }
+  BnGeom ga = g;
+  dim3 gridApply = grid;
+  float *gx = gradInput_ ? data(gradInput_) : nullptr;
+  float *gw = dataOrNull(gradWeight_), *gb = dataOrNull(gradBias_);
+  const float *w = dataOrNull(weight_);
+#define BN_BWD(TRAIN, VEC)                                                                                   \
+  bnBackwardKernel<TRAIN, VEC><<<gridApply, block, 0, s>>>(in.ptr(), go.ptr(), gx, p, gw, gb, w, meanSrc, stdSrc, ga, \
+                                                           (float)scale, (float)eps)
+  if (train) {
+    if (v.vec)
+      BN_BWD(true, true);
+    else
+      BN_BWD(true, false);
+  } else {
+    if (v.vec)
+      BN_BWD(false, true);
+    else
+      BN_BWD(false, false);
+  }
+#undef BN_BWD
+  THC_HIP_CHECK(hipGetLastError());
+  THNN_LEAVE
+}
+
+}  // extern "C"

@@ -1,0 +1,651 @@
+// SpatialConvolutionMM for gfx950: im2col/col2im + fp32 MFMA GEMM.
+//
+// The reference loops over the batch and per image launches im2col, an SGEMM
+// and (for the bias) a k=1 SGEMM, writing a (Cin*kH*kW) x (oH*oW) column
+// buffer to memory and reading it back
+// (lib/THCUNN/generic/SpatialConvolutionMM.cu:129-194, 272-308, 396-470).
+// Here each entry point is one batched GEMM over the whole mini-batch built on
+// v_mfma_f32_32x32x2_f32 with LDS-staged 128x128x16 tiles:
+//   updateOutput       C[o][n,l]  = bias[o] + sum_k W[o][k] * col[k][n,l]
+//                      col is never stored: the B-tile loader gathers it from
+//                      the NCHW input on the fly (implicit im2col, zero padded)
+//   accGradParameters  gW[o][k]  += scale * sum_{n,l} gy[n][o][l] * col[k][n,l]
+//                      split over groups of images; partial products go to the
+//                      caller's `columns` scratch and are folded in a fixed
+//                      order (deterministic, no atomics); gradBias is a
+//                      separate 64-lane shuffle reduction
+//   updateGradInput    gradCol[k][n,l] = sum_o W[o][k] * gy[n][o][l] for a group
+//                      of images into `gradColumns`, then the col2im gather of
+//                      lib/THCUNN/im2col.h:63-102 over the group.
+#include "device_utils.h"
+#include "launch_utils.h"
+#include "thc_internal.h"
+
+using namespace thc;
+
+namespace {
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BK = 16;
+constexpr int PITCH = 132;  // 8 * PITCH % 64 == 32: the two k-halves of a transposing store hit disjoint banks
+
+struct ConvGeom {
+  int N, Cin, Cout, H, W, oH, oW;
+  int kH, kW, dH, dW, padH, padW;
+  int K;  // Cin * kH * kW
+  int L;  // oH * oW
+};
+
+enum GemmMode { kForward = 0, kGradCol = 1, kGradWeight = 2 };
+
+struct GemmArgs {
+  const float *a;   // forward: W (Cout x K); gradCol: W; gradWeight: gy
+  const float *b;   // forward: x; gradCol: gy; gradWeight: x
+  float *c;         // forward: out; gradCol: gradCol of the group; gradWeight: partials
+  const float *bias;
+  int M, Ncols, R;  // GEMM extents: C is M x Ncols, reduction length R (per split)
+  int n0;           // first image of the group (gradCol) / images per split (gradWeight)
+  int nImages;      // images covered by this launch
+  int mTiles;
+  bool vecA;        // A rows may be fetched with 16-byte loads (extent % 4 == 0, aligned base)
+};
+
+// Decomposition of a flat output position lg = n*L + oh*oW + ow.
+struct Pos {
+  int n, oh, ow;
+};
+
+// ---- the MFMA core: one 128x128 tile, 4 waves of 64x64 -----------------------
+__device__ __forceinline__ void mfmaTile(const float (*As)[PITCH], const float (*Bs)[PITCH], float16v (&acc)[2][2],
+                                         int wm, int wn, int lane) {
+  const int kk = lane >> 5, idx = lane & 31;
+#pragma unroll
+  for (int k = 0; k < BK; k += 2) {
+    float a0 = As[k + kk][wm * 64 + idx], a1 = As[k + kk][wm * 64 + 32 + idx];
+    float b0 = Bs[k + kk][wn * 64 + idx], b1 = Bs[k + kk][wn * 64 + 32 + idx];
+    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+    acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+    acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+  }
+}
+
+// Element (r, col) of the implicit im2col matrix for image base xb:
+// x[c][oh*dH - padH + kh][ow*dW - padW + kw] or 0 (lib/THCUNN/im2col.h:24-36).
+__device__ __forceinline__ float gatherCol(const float *__restrict__ xb, const ConvGeom &g, int c, int kh, int kw,
+                                           int ih0, int iw0) {
+  int ih = ih0 + kh, iw = iw0 + kw;
+  return (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W) ? xb[((long)c * g.H + ih) * g.W + iw] : 0.f;
+}
+
+template <int MODE>
+__global__ void __launch_bounds__(dev::kBlock)
+convGemmKernel(GemmArgs p, ConvGeom g) {
+  __shared__ float As[2][BK][PITCH];
+  __shared__ float Bs[2][BK][PITCH];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int mTile = blockIdx.x % p.mTiles, nTile = blockIdx.x / p.mTiles;
+  const int m0 = mTile * BM, j0 = nTile * BN;
+  const int split = blockIdx.y;
+  const int KK = g.kH * g.kW;
+
+  float16v acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  float ra[8], rb[8];
+
+  // ---- per-thread loader state ------------------------------------------------
+  // "col-major" mapping: one tile column, 8 consecutive reduction rows
+  const int colA = t & 127, rowA8 = (t >> 7) * 8;
+  // "row-major" mapping: one tile row/column pair (t >> 1), 8 consecutive reduction elements
+  const int rowT = t >> 1, redT8 = (t & 1) * 8;
+
+  // forward / gradCol: B column = output position lg (fixed per thread)
+  Pos bp = {0, 0, 0};
+  bool bValid = false;
+  const float *bBase = nullptr;
+  int ih0 = 0, iw0 = 0;
+  if (MODE == kForward || MODE == kGradCol) {
+    long lg = (long)j0 + colA;
+    bValid = lg < (long)p.Ncols;
+    if (bValid) {
+      bp.n = (int)(lg / g.L);
+      int l = (int)(lg - (long)bp.n * g.L);
+      bp.oh = l / g.oW;
+      bp.ow = l - bp.oh * g.oW;
+      if (MODE == kForward) {
+        bBase = p.b + (long)(p.n0 + bp.n) * g.Cin * g.H * g.W;
+        ih0 = bp.oh * g.dH - g.padH;
+        iw0 = bp.ow * g.dW - g.padW;
+      } else {
+        bBase = p.b + (long)(p.n0 + bp.n) * g.Cout * g.L + l;  // + o * L
+      }
+    }
+  }
+  // gradWeight: B column = k index (c, kh, kw), 16-lane groups walk consecutive positions
+  const int gwR = t & 15, gwJ = t >> 4;  // reduction row within the tile, first of 8 columns (stride 16)
+  const int imgFirst = (MODE == kGradWeight) ? split * p.n0 : 0;
+  const int imgCount = (MODE == kGradWeight) ? min(p.n0, p.nImages - imgFirst) : 0;
+  const long Rlen = (MODE == kGradWeight) ? (long)imgCount * g.L : (long)p.R;
+  const int nkt = (int)((Rlen + BK - 1) / BK);
+
+  auto loadTiles = [&](int kt) {
+    const int r0 = kt * BK;
+    if (MODE == kForward) {
+      // A: W[o][k], k contiguous
+      {
+        int o = m0 + rowT, k = r0 + redT8;
+        const float *src = p.a + (long)o * g.K + k;
+        bool rowOk = o < p.M;
+        if (p.vecA && rowOk && k + 8 <= g.K) {
+          float4 v0 = reinterpret_cast<const float4 *>(src)[0], v1 = reinterpret_cast<const float4 *>(src)[1];
+          ra[0] = v0.x, ra[1] = v0.y, ra[2] = v0.z, ra[3] = v0.w;
+          ra[4] = v1.x, ra[5] = v1.y, ra[6] = v1.z, ra[7] = v1.w;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) ra[i] = (rowOk && k + i < g.K) ? src[i] : 0.f;
+        }
+      }
+      // B: implicit im2col, rows k = r0 + rowA8 + i
+      {
+        int k = r0 + rowA8;
+        int c = k / KK, rem = k - c * KK;
+        int kh = rem / g.kW, kw = rem - kh * g.kW;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          rb[i] = (bValid && k + i < g.K) ? gatherCol(bBase, g, c, kh, kw, ih0, iw0) : 0.f;
+          if (++kw == g.kW) {
+            kw = 0;
+            if (++kh == g.kH) {
+              kh = 0;
+              ++c;
+            }
+          }
+        }
+      }
+    } else if (MODE == kGradCol) {
+      // A[m = k][r = o] = W[o][k]: contiguous along m
+      {
+        int k = m0 + colA;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          int o = r0 + rowA8 + i;
+          ra[i] = (k < p.M && o < p.R) ? p.a[(long)o * g.K + k] : 0.f;
+        }
+      }
+      // B[r = o][lg] = gy[n][o][l]
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        int o = r0 + rowA8 + i;
+        rb[i] = (bValid && o < p.R) ? bBase[(long)o * g.L] : 0.f;
+      }
+    } else {
+      // gradWeight. A[m = o][r = (n,l)] = gy[n][o][l]: contiguous along r inside an image
+      {
+        int o = m0 + rowT;
+        long r = (long)r0 + redT8;
+        bool rowOk = o < p.M;
+        int n = (int)(r / g.L);
+        int l = (int)(r - (long)n * g.L);
+        if (p.vecA && rowOk && r + 8 <= Rlen) {
+          // with L % 4 == 0 a group of 4 never straddles an image
+          const float *s0 = p.a + ((long)(imgFirst + n) * g.Cout + o) * g.L + l;
+          float4 v0 = *reinterpret_cast<const float4 *>(s0);
+          int l2 = l + 4, n2 = n;
+          if (l2 >= g.L) {
+            l2 -= g.L;
+            ++n2;
+          }
+          const float *s1 = p.a + ((long)(imgFirst + n2) * g.Cout + o) * g.L + l2;
+          float4 v1 = *reinterpret_cast<const float4 *>(s1);
+          ra[0] = v0.x, ra[1] = v0.y, ra[2] = v0.z, ra[3] = v0.w;
+          ra[4] = v1.x, ra[5] = v1.y, ra[6] = v1.z, ra[7] = v1.w;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            ra[i] = (rowOk && r + i < Rlen) ? p.a[((long)(imgFirst + n) * g.Cout + o) * g.L + l] : 0.f;
+            if (++l == g.L) {
+              l = 0;
+              ++n;
+            }
+          }
+        }
+      }
+      // B[r = (n,l)][j = k] = col[k][n,l]; lanes 0..15 of a group walk consecutive l
+      {
+        long r = (long)r0 + gwR;
+        bool rOk = r < Rlen;
+        int n = rOk ? (int)(r / g.L) : 0;
+        int l = rOk ? (int)(r - (long)n * g.L) : 0;
+        int oh = l / g.oW, ow = l - oh * g.oW;
+        const float *xb = p.b + (long)(imgFirst + n) * g.Cin * g.H * g.W;
+        int ih0g = oh * g.dH - g.padH, iw0g = ow * g.dW - g.padW;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          int k = j0 + gwJ + 16 * i;
+          float v = 0.f;
+          if (rOk && k < p.Ncols) {
+            int c = k / KK, rem = k - c * KK;
+            int kh = rem / g.kW, kw = rem - kh * g.kW;
+            v = gatherCol(xb, g, c, kh, kw, ih0g, iw0g);
+          }
+          rb[i] = v;
+        }
+      }
+    }
+  };
+
+  auto storeTiles = [&](int buf) {
+    if (MODE == kForward) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) As[buf][redT8 + i][rowT] = ra[i];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) Bs[buf][rowA8 + i][colA] = rb[i];
+    } else if (MODE == kGradCol) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) As[buf][rowA8 + i][colA] = ra[i];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) Bs[buf][rowA8 + i][colA] = rb[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) As[buf][redT8 + i][rowT] = ra[i];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) Bs[buf][gwR][gwJ + 16 * i] = rb[i];
+    }
+  };
+
+  if (nkt > 0) {
+    loadTiles(0);
+    storeTiles(0);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nkt) loadTiles(kt + 1);
+    mfmaTile(As[buf], Bs[buf], acc, wm, wn, lane);
+    if (kt + 1 < nkt) storeTiles(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue ----------------------------------------------------------------
+  // 32x32 accumulator layout: lane holds column (lane & 31) and rows
+  // 8*(v/4) + 4*(lane/32) + v%4, v = 0..15.
+  const int colInTile = lane & 31, rowHalf = (lane >> 5) * 4;
+#pragma unroll
+  for (int tj = 0; tj < 2; ++tj) {
+    const long col = (long)j0 + wn * 64 + tj * 32 + colInTile;
+    if (col >= p.Ncols) continue;
+    long cOff;  // offset of (row 0, col) and row stride
+    long rowStride;
+    if (MODE == kForward) {
+      int n = (int)(col / g.L);
+      int l = (int)(col - (long)n * g.L);
+      cOff = (long)(p.n0 + n) * g.Cout * g.L + l;
+      rowStride = g.L;
+    } else if (MODE == kGradCol) {
+      int n = (int)(col / g.L);
+      int l = (int)(col - (long)n * g.L);
+      cOff = (long)n * g.K * g.L + l;
+      rowStride = g.L;
+    } else {
+      cOff = (long)split * p.M * p.Ncols + col;
+      rowStride = p.Ncols;
+    }
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
+        if (row < p.M) {
+          float val = acc[ti][tj][v];
+          if (MODE == kForward && p.bias) val += p.bias[row];
+          p.c[cOff + (long)row * rowStride] = val;
+        }
+      }
+    }
+  }
+}
+
+// gW[i] += scale * sum_s partial[s][i], s ascending
+__global__ void __launch_bounds__(dev::kBlock)
+foldPartialsKernel(const float *__restrict__ partial, float *__restrict__ dst, long count, int splits, float scale) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (long)gridDim.x * blockDim.x) {
+    float s = 0.f;
+    for (int k = 0; k < splits; ++k) s += partial[(long)k * count + i];
+    dst[i] += scale * s;
+  }
+}
+
+// gradBias[o] += scale * sum_{n,l} gy[n][o][l]   (lib/THCUNN/generic/SpatialConvolutionMM.cu:440-455)
+__global__ void __launch_bounds__(dev::kBlock)
+gradBiasKernel(const float *__restrict__ gy, float *__restrict__ gradBias, int N, int Cout, int L, float scale) {
+  __shared__ float red[dev::kBlock / dev::kWave];
+  const int o = blockIdx.x;
+  float acc = 0.f;
+  const long total = (long)N * L;
+  for (long i = threadIdx.x; i < total; i += blockDim.x) {
+    int n = (int)(i / L);
+    int l = (int)(i - (long)n * L);
+    acc += gy[((long)n * Cout + o) * L + l];
+  }
+  acc = dev::waveSum(acc);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.f;
+    for (int w = 0; w < dev::kBlock / dev::kWave; ++w) s += red[w];
+    gradBias[o] += scale * s;
+  }
+}
+
+// ---- im2col / col2im (lib/THCUNN/im2col.h) -----------------------------------
+// One lane per column entry; consecutive lanes write consecutive addresses.
+__global__ void __launch_bounds__(dev::kBlock)
+im2colKernel(const float *__restrict__ im, float *__restrict__ col, int nImg, int C, int H, int W, int kH, int kW,
+             int padH, int padW, int dH, int dW, int dilH, int dilW, int oH, int oW) {
+  const long L = (long)oH * oW;
+  const long perImg = (long)C * kH * kW * L;
+  const long total = perImg * nImg;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    long n = i / perImg;
+    long r = i - n * perImg;
+    int ow = (int)(r % oW);
+    r /= oW;
+    int oh = (int)(r % oH);
+    r /= oH;
+    int kw = (int)(r % kW);
+    r /= kW;
+    int kh = (int)(r % kH);
+    int c = (int)(r / kH);
+    int h = oh * dH - padH + kh * dilH, w = ow * dW - padW + kw * dilW;
+    col[i] = (h >= 0 && w >= 0 && h < H && w < W) ? im[((n * C + c) * H + h) * W + w] : 0.f;
+  }
+}
+
+// One lane per image pixel gathers every column entry that maps onto it
+// (lib/THCUNN/im2col.h:63-102); float accumulation in the reference's order.
+__global__ void __launch_bounds__(dev::kBlock)
+col2imKernel(const float *__restrict__ col, float *__restrict__ im, int nImg, int C, int H, int W, int kH, int kW,
+             int padH, int padW, int dH, int dW, int dilH, int dilW, int oH, int oW) {
+  const long total = (long)nImg * C * H * W;
+  const int extW = (kW - 1) * dilW + 1, extH = (kH - 1) * dilH + 1;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    int w_im = (int)(i % W) + padW;
+    int h_im = (int)((i / W) % H) + padH;
+    long nc = i / ((long)W * H);  // n * C + c
+    int ws = (w_im < extW) ? 0 : (w_im - extW) / dW + 1;
+    int we = min(w_im / dW + 1, oW);
+    int hs = (h_im < extH) ? 0 : (h_im - extH) / dH + 1;
+    int he = min(h_im / dH + 1, oH);
+    float val = 0.f;
+    for (int hc = hs; hc < he; ++hc)
+      for (int wc = ws; wc < we; ++wc) {
+        int hk = h_im - hc * dH, wk = w_im - wc * dW;
+        if (hk % dilH == 0 && wk % dilW == 0) {
+          hk /= dilH;
+          wk /= dilW;
+          val += col[(((nc * kH + hk) * kW + wk) * oH + hc) * oW + wc];
+        }
+      }
+    im[i] = val;
+  }
+}
+
+// ---- host side -----------------------------------------------------------------
+struct ConvCall {
+  ConvGeom g;
+  bool batch;
+};
+
+// lib/THCUNN/generic/SpatialConvolutionMM.cu:5-56. `weight` may be 2-D (Cout, Cin*kH*kW)
+// or 4-D contiguous; only its extents are read here.
+ConvCall convSetup(THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *weight, THCudaTensor *bias,
+                   const char *weightName, int kH, int kW, int dH, int dW, int padH, int padW) {
+  THC_ARG_CHECK(input && weight, 2, "input and weight tensors expected");
+  THC_ARG_CHECK(isContiguous(erase(weight)), 4, "%s tensor has to be contiguous", weightName);
+  THC_ARG_CHECK(kW > 0 && kH > 0, 9, "kernel size should be greater than zero, but got kH: %d kW: %d", kH, kW);
+  THC_ARG_CHECK(dW > 0 && dH > 0, 11, "stride should be greater than zero, but got dH: %d dW: %d", dH, dW);
+  THC_ARG_CHECK(!bias || isContiguous(erase(bias)), 5, "bias tensor has to be contiguous");
+  THC_ARG_CHECK(weight->nDimension == 2 || weight->nDimension == 4, 5,
+                "2D or 4D weight tensor expected, but got: %s", sizeDesc(erase(weight)).c_str());
+  long nOutputPlane = weight->size[0];
+  long wcols = weight->nDimension == 2 ? weight->size[1] : weight->size[1] * weight->size[2] * weight->size[3];
+  if (bias) checkDimSize(erase(bias), "bias", 1, 0, nOutputPlane);
+  int ndim = input->nDimension;
+  int dimf = 0, dimh = 1, dimw = 2;
+  if (ndim == 4) {
+    dimf++;
+    dimh++;
+    dimw++;
+  }
+  THC_ARG_CHECK(ndim == 3 || ndim == 4, 2, "3D or 4D input tensor expected but got: %s",
+                sizeDesc(erase(input)).c_str());
+  long nInputPlane = wcols / (kH * kW);
+  long inputHeight = input->size[dimh], inputWidth = input->size[dimw];
+  long outputHeight = (inputHeight + 2 * padH - kH) / dH + 1;
+  long outputWidth = (inputWidth + 2 * padW - kW) / dW + 1;
+  if (outputWidth < 1 || outputHeight < 1)
+    error("Given input size: (%ld x %ld x %ld). Calculated output size: (%ld x %ld x %ld). Output size is too small",
+          nInputPlane, inputHeight, inputWidth, nOutputPlane, outputHeight, outputWidth);
+  checkDimSize(erase(input), "input", ndim, dimf, nInputPlane);
+  if (gradOutput) {
+    checkDimSize(erase(gradOutput), "gradOutput", ndim, dimf, nOutputPlane);
+    checkDimSize(erase(gradOutput), "gradOutput", ndim, dimh, outputHeight);
+    checkDimSize(erase(gradOutput), "gradOutput", ndim, dimw, outputWidth);
+    if (ndim == 4 && gradOutput->size[0] != input->size[0])
+      error("input and gradOutput batch sizes do not match: input %s, gradOutput %s", sizeDesc(erase(input)).c_str(),
+            sizeDesc(erase(gradOutput)).c_str());
+  }
+  if (wcols != nInputPlane * kH * kW)
+    error("%s of shape %s does not match a %d x %d kernel", weightName, sizeDesc(erase(weight)).c_str(), kH, kW);
+  ConvCall call;
+  call.batch = ndim == 4;
+  ConvGeom &g = call.g;
+  g.N = call.batch ? (int)input->size[0] : 1;
+  g.Cin = (int)nInputPlane, g.Cout = (int)nOutputPlane;
+  g.H = (int)inputHeight, g.W = (int)inputWidth, g.oH = (int)outputHeight, g.oW = (int)outputWidth;
+  g.kH = kH, g.kW = kW, g.dH = dH, g.dW = dW, g.padH = padH, g.padW = padW;
+  g.K = g.Cin * kH * kW;
+  g.L = g.oH * g.oW;
+  if ((long)g.Cin * g.H * g.W >= 0x7fffffffL || (long)g.K * g.L >= 0x7fffffffL * 8L)
+    error("SpatialConvolutionMM: image too large");
+  return call;
+}
+
+inline unsigned tiles(long n, int b) { return (unsigned)((n + b - 1) / b); }
+
+}  // namespace
+
+extern "C" {
+
+void THNN_CudaSpatialConvolutionMM_updateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output,
+                                                THCudaTensor *weight, THCudaTensor *bias, THCudaTensor *columns,
+                                                THCudaTensor *ones, int kW, int kH, int dW, int dH, int padW,
+                                                int padH) {
+  THNN_ENTER
+  (void)columns;  // the implicit-im2col GEMM needs neither buffer; both are left untouched
+  (void)ones;
+  THC_ARG_CHECK(output != nullptr, 3, "output tensor expected");
+  ConvCall call = convSetup(input, nullptr, weight, bias, "weight", kH, kW, dH, dW, padH, padW);
+  ConvGeom &g = call.g;
+  Contiguous in(state, input);
+  if (call.batch)
+    resize(state, output, {g.N, g.Cout, g.oH, g.oW});
+  else
+    resize(state, output, {g.Cout, g.oH, g.oW});
+  if (!isContiguous(erase(output))) error("output tensor has to be contiguous");
+  if ((long)g.N * g.Cout == 0) return;
+  hipStream_t s = state->stream;
+  // images per launch so that the flat column index n*L + l fits an int
+  int group = (int)std::min<long>(g.N, std::max<long>(1, 0x7fffffffL / 2 / g.L));
+  for (int n0 = 0; n0 < g.N; n0 += group) {
+    int cnt = std::min(group, g.N - n0);
+    GemmArgs p{};
+    p.a = data(weight);
+    p.b = in.ptr();
+    p.c = data(output);
+    p.bias = bias ? data(bias) : nullptr;
+    p.M = g.Cout;
+    p.Ncols = cnt * g.L;
+    p.R = g.K;
+    p.n0 = n0;
+    p.nImages = cnt;
+    p.mTiles = (int)tiles(p.M, BM);
+    p.vecA = (g.K % 4 == 0) && launch::aligned16(p.a);
+    dim3 grid(p.mTiles * tiles(p.Ncols, BN), 1);
+    convGemmKernel<kForward><<<grid, dev::kBlock, 0, s>>>(p, g);
+    THC_HIP_CHECK(hipGetLastError());
+  }
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialConvolutionMM_updateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput,
+                                                   THCudaTensor *gradInput, THCudaTensor *weight,
+                                                   THCudaTensor *gradColumns, THCudaTensor *ones, int kW, int kH,
+                                                   int dW, int dH, int padW, int padH) {
+  THNN_ENTER
+  (void)ones;
+  THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
+  THC_ARG_CHECK(gradInput != nullptr, 4, "gradInput tensor expected");
+  ConvCall call = convSetup(input, gradOutput, weight, nullptr, "weight", kH, kW, dH, dW, padH, padW);
+  ConvGeom &g = call.g;
+  Contiguous go(state, gradOutput);
+  if (call.batch)
+    resize(state, gradInput, {g.N, g.Cin, g.H, g.W});
+  else
+    resize(state, gradInput, {g.Cin, g.H, g.W});
+  if (!isContiguous(erase(gradInput))) error("gradInput tensor has to be contiguous");
+  if ((long)g.N * g.Cin == 0) return;
+  hipStream_t s = state->stream;
+  // gradient columns of a group of images at a time (<= 64 MB so the buffer stays cache resident)
+  const long perImg = (long)g.K * g.L;
+  int group = (int)std::max<long>(1, std::min<long>(g.N, (64L << 20) / 4 / perImg));
+  group = (int)std::min<long>(group, std::max<long>(1, 0x7fffffffL / 2 / g.L));
+  Temp tmp;
+  float *gcol;
+  if (gradColumns) {
+    resize(state, gradColumns, {(long)group * g.K, g.L});
+    if (!isContiguous(erase(gradColumns))) error("gradColumns tensor has to be contiguous");
+    gcol = data(gradColumns);
+  } else {
+    tmp = Temp(s, (size_t)group * perImg * sizeof(float));
+    gcol = (float *)tmp.get();
+  }
+  for (int n0 = 0; n0 < g.N; n0 += group) {
+    int cnt = std::min(group, g.N - n0);
+    GemmArgs p{};
+    p.a = data(weight);
+    p.b = go.ptr();
+    p.c = gcol;
+    p.M = g.K;
+    p.Ncols = cnt * g.L;
+    p.R = g.Cout;
+    p.n0 = n0;
+    p.nImages = cnt;
+    p.mTiles = (int)tiles(p.M, BM);
+    dim3 grid(p.mTiles * tiles(p.Ncols, BN), 1);
+    convGemmKernel<kGradCol><<<grid, dev::kBlock, 0, s>>>(p, g);
+    THC_HIP_CHECK(hipGetLastError());
+    long total = (long)cnt * g.Cin * g.H * g.W;
+    col2imKernel<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(
+        gcol, data(gradInput) + (long)n0 * g.Cin * g.H * g.W, cnt, g.Cin, g.H, g.W, g.kH, g.kW, g.padH, g.padW, g.dH,
+        g.dW, 1, 1, g.oH, g.oW);
+    THC_HIP_CHECK(hipGetLastError());
+  }
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput,
+                                                     THCudaTensor *gradWeight, THCudaTensor *gradBias,
+                                                     THCudaTensor *columns, THCudaTensor *ones, int kW, int kH,
+                                                     int dW, int dH, int padW, int padH, float scale) {
+  THNN_ENTER
+  (void)ones;
+  THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
+  THC_ARG_CHECK(gradWeight != nullptr, 4, "gradWeight tensor expected");
+  ConvCall call = convSetup(input, gradOutput, gradWeight, gradBias, "weight", kH, kW, dH, dW, padH, padW);
+  ConvGeom &g = call.g;
+  Contiguous in(state, input);
+  Contiguous go(state, gradOutput);
+  if ((long)g.N * g.Cout * g.K == 0) return;
+  hipStream_t s = state->stream;
+
+  // split the reduction over groups of images until the grid fills the chip
+  const int mT = (int)tiles(g.Cout, BM), nT = (int)tiles(g.K, BN);
+  int splits = (int)std::min<long>(g.N, std::max<long>(1, (2 * 256 + mT * nT - 1) / (mT * nT)));
+  int perSplit = launch::ceilDiv(g.N, splits);
+  perSplit = (int)std::min<long>(perSplit, std::max<long>(1, 0x7fffffffL / 2 / g.L));
+  splits = launch::ceilDiv(g.N, perSplit);
+  const long count = (long)g.Cout * g.K;
+  Temp tmp;
+  float *partial;
+  if (columns) {
+    resize(state, columns, {(long)splits * g.Cout, g.K});
+    if (!isContiguous(erase(columns))) error("columns tensor has to be contiguous");
+    partial = data(columns);
+  } else {
+    tmp = Temp(s, (size_t)splits * count * sizeof(float));
+    partial = (float *)tmp.get();
+  }
+  GemmArgs p{};
+  p.a = go.ptr();
+  p.b = in.ptr();
+  p.c = partial;
+  p.M = g.Cout;
+  p.Ncols = g.K;
+  p.R = 0;
+  p.n0 = perSplit;
+  p.nImages = g.N;
+  p.mTiles = mT;
+  p.vecA = (g.L % 4 == 0) && launch::aligned16(p.a);
+  dim3 grid(mT * nT, splits);
+  convGemmKernel<kGradWeight><<<grid, dev::kBlock, 0, s>>>(p, g);
+  THC_HIP_CHECK(hipGetLastError());
+  foldPartialsKernel<<<launch::directGrid(count, dev::kBlock), dev::kBlock, 0, s>>>(partial, data(gradWeight), count,
+                                                                                   splits, scale);
+  THC_HIP_CHECK(hipGetLastError());
+  if (gradBias) {
+    gradBiasKernel<<<g.Cout, dev::kBlock, 0, s>>>(go.ptr(), data(gradBias), g.N, g.Cout, g.L, scale);
+    THC_HIP_CHECK(hipGetLastError());
+  }
+  THNN_LEAVE
+}
+
+// Stand-alone im2col / col2im over a batch of images with the semantics of
+// lib/THCUNN/im2col.h:40-61 and :104-121 (the reference keeps them as C++
+// templates inside the library; they are exported here so that their parity
+// can be checked on their own).
+void THNN_Cuda_im2col(THCState *state, const float *im, int nImages, int channels, int height, int width, int kH,
+                      int kW, int padH, int padW, int dH, int dW, int dilH, int dilW, float *col) {
+  THNN_ENTER
+  int oH = (height + 2 * padH - (dilH * (kH - 1) + 1)) / dH + 1;
+  int oW = (width + 2 * padW - (dilW * (kW - 1) + 1)) / dW + 1;
+  long total = (long)nImages * channels * kH * kW * oH * oW;
+  if (total <= 0) return;
+  im2colKernel<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, state->stream>>>(
+      im, col, nImages, channels, height, width, kH, kW, padH, padW, dH, dW, dilH, dilW, oH, oW);
+  THC_HIP_CHECK(hipGetLastError());
+  THNN_LEAVE
+}
+
+void THNN_Cuda_col2im(THCState *state, const float *col, int nImages, int channels, int height, int width, int kH,
+                      int kW, int padH, int padW, int dH, int dW, int dilH, int dilW, float *im) {
+  THNN_ENTER
+  int oH = (height + 2 * padH - (dilH * (kH - 1) + 1)) / dH + 1;
+  int oW = (width + 2 * padW - (dilW * (kW - 1) + 1)) / dW + 1;
+  long total = (long)nImages * channels * height * width;
+  if (total <= 0) return;
+  col2imKernel<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, state->stream>>>(
+      col, im, nImages, channels, height, width, kH, kW, padH, padW, dH, dW, dilH, dilW, oH, oW);
+  THC_HIP_CHECK(hipGetLastError());
+  THNN_LEAVE
+}
+
+}  // extern "C"

@@ -1,0 +1,594 @@
+// SpatialMaxPooling / SpatialDilatedMaxPooling / SpatialAveragePooling for gfx950.
+//
+// All four kernels are pure streaming: a workgroup owns a band of rows of one
+// (n,c) plane, stages the rows of the other tensor that the band depends on in
+// LDS with one contiguous (16-byte where aligned) copy, and produces its band
+// with coalesced stores. Window scans keep the reference's order (rows outer,
+// columns inner, strict '>' for max) so ties resolve identically
+// (lib/THCUNN/SpatialDilatedMaxPooling.cu:7-42) and float sums associate
+// identically (lib/THCUNN/SpatialAveragePooling.cu:6-82). The backward passes are
+// gathers per input pixel, as in the reference, hence deterministic.
+#include <cfloat>
+#include <cmath>
+
+#include "device_utils.h"
+#include "launch_utils.h"
+#include "thc_internal.h"
+
+using namespace thc;
+
+namespace {
+
+struct PoolGeom {
+  int H, W, oH, oW;
+  int kH, kW, dH, dW, padH, padW, dilH, dilW;
+  int tileRows, tilesPerPlane, nblk;
+  int maxStageRows;  // rows of the staged tensor per band (upper bound)
+};
+
+// ----------------------------------------------------------- max: forward ----
+template <int KS, int ST, bool VEC>
+__global__ void __launch_bounds__(dev::kBlock)
+maxPoolFwdTiled(const float *__restrict__ in, float *__restrict__ out, long *__restrict__ indices, PoolGeom g) {
+  extern __shared__ float smem[];
+  const int kH = KS ? KS : g.kH, kW = KS ? KS : g.kW;
+  const int dH = ST ? ST : g.dH, dW = ST ? ST : g.dW;
+  const int dilH = KS ? 1 : g.dilH, dilW = KS ? 1 : g.dilW;
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  const int ph0 = tile * g.tileRows;
+  const int nOut = min(g.tileRows, g.oH - ph0);
+  const int hLo = max(0, ph0 * dH - g.padH);
+  const int hHi = min(g.H, (ph0 + nOut - 1) * dH - g.padH + (kH - 1) * dilH + 1);
+  dev::loadFlat<VEC>(smem, in + ((long)plane * g.H + hLo) * g.W, max(0, hHi - hLo) * g.W);
+  __syncthreads();
+
+  const long obase = ((long)plane * g.oH + ph0) * g.oW;
+  const int total = nOut * g.oW;
+  for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    int r = i / g.oW, pw = i - r * g.oW;
+    int hstart = (ph0 + r) * dH - g.padH;
+    int wstart = pw * dW - g.padW;
+    float maxval = -FLT_MAX;
+    int maxidx = -1;
+    if (KS) {
+#pragma unroll
+      for (int kh = 0; kh < KS; ++kh) {
+        int h = hstart + kh;
+        bool hv = h >= 0 && h < g.H;
+#pragma unroll
+        for (int kw = 0; kw < KS; ++kw) {
+          int w = wstart + kw;
+          if (hv && w >= 0 && w < g.W) {
+            float v = smem[(h - hLo) * g.W + w];
+            if (v > maxval) {
+              maxval = v;
+              maxidx = h * g.W + w;
+            }
+          }
+        }
+      }
+    } else {
+      int hend = min(hstart + (kH - 1) * dilH + 1, g.H);
+      int wend = min(wstart + (kW - 1) * dilW + 1, g.W);
+      while (hstart < 0) hstart += dilH;
+      while (wstart < 0) wstart += dilW;
+      for (int h = hstart; h < hend; h += dilH)
+        for (int w = wstart; w < wend; w += dilW) {
+          float v = smem[(h - hLo) * g.W + w];
+          if (v > maxval) {
+            maxval = v;
+            maxidx = h * g.W + w;
+          }
+        }
+    }
+    out[obase + i] = maxval;
+    indices[obase + i] = (long)maxidx + TH_INDEX_BASE;
+  }
+}
+
+__global__ void __launch_bounds__(dev::kBlock)
+maxPoolFwdDirect(const float *__restrict__ in, float *__restrict__ out, long *__restrict__ indices, PoolGeom g,
+                 long total) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    int pw = (int)(i % g.oW);
+    long t = i / g.oW;
+    int ph = (int)(t % g.oH);
+    long plane = t / g.oH;
+    const float *ip = in + plane * g.H * g.W;
+    int hstart = ph * g.dH - g.padH, wstart = pw * g.dW - g.padW;
+    int hend = min(hstart + (g.kH - 1) * g.dilH + 1, g.H);
+    int wend = min(wstart + (g.kW - 1) * g.dilW + 1, g.W);
+    while (hstart < 0) hstart += g.dilH;
+    while (wstart < 0) wstart += g.dilW;
+    float maxval = -FLT_MAX;
+    int maxidx = -1;
+    for (int h = hstart; h < hend; h += g.dilH)
+      for (int w = wstart; w < wend; w += g.dilW) {
+        float v = ip[(long)h * g.W + w];
+        if (v > maxval) {
+          maxval = v;
+          maxidx = h * g.W + w;
+        }
+      }
+    out[i] = maxval;
+    indices[i] = (long)maxidx + TH_INDEX_BASE;
+  }
+}
+
+// ---------------------------------------------------------- max: backward ----
+// Band of gradInput rows; the gradOutput rows and indices (narrowed to 32 bits,
+// base removed) of every window that can reach the band are staged in LDS.
+template <bool VEC>
+__global__ void __launch_bounds__(dev::kBlock)
+maxPoolBwdTiled(const float *__restrict__ gradOut, const long *__restrict__ indices, float *__restrict__ gradIn,
+                PoolGeom g) {
+  extern __shared__ float smem[];
+  const int extH = (g.kH - 1) * g.dilH + 1, extW = (g.kW - 1) * g.dilW + 1;
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  const int h0 = tile * g.tileRows;
+  const int nRows = min(g.tileRows, g.H - h0);
+  const int phLo = max(0, dev::ceilDivPos(h0 + g.padH - extH + 1, g.dH));
+  const int phHi = min(g.oH - 1, (h0 + nRows - 1 + g.padH) / g.dH);
+  const int nPh = max(0, phHi - phLo + 1);
+  float *gs = smem;
+  int *is = reinterpret_cast<int *>(smem + (size_t)g.maxStageRows * g.oW);
+  const long sbase = ((long)plane * g.oH + phLo) * g.oW;
+  const int cnt = nPh * g.oW;
+  dev::loadFlat<VEC>(gs, gradOut + sbase, cnt);
+  for (int i = threadIdx.x; i < cnt; i += blockDim.x) is[i] = (int)(indices[sbase + i] - TH_INDEX_BASE);
+  __syncthreads();
+
+  float *o = gradIn + ((long)plane * g.H + h0) * g.W;
+  const int total = nRows * g.W;
+  for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    int r = i / g.W, w = i - r * g.W;
+    int h = h0 + r;
+    int phstart = (h + g.padH < extH) ? 0 : (h + g.padH - extH) / g.dH + 1;
+    int phend = min((h + g.padH) / g.dH + 1, g.oH);
+    int pwstart = (w + g.padW < extW) ? 0 : (w + g.padW - extW) / g.dW + 1;
+    int pwend = min((w + g.padW) / g.dW + 1, g.oW);
+    const int me = h * g.W + w;
+    float grad = 0.f;
+    for (int ph = phstart; ph < phend; ++ph)
+      for (int pw = pwstart; pw < pwend; ++pw) {
+        int k = (ph - phLo) * g.oW + pw;
+        if (is[k] == me) grad += gs[k];
+      }
+    o[i] = grad;
+  }
+}
+
+__global__ void __launch_bounds__(dev::kBlock)
+maxPoolBwdDirect(const float *__restrict__ gradOut, const long *__restrict__ indices, float *__restrict__ gradIn,
+                 PoolGeom g, long total) {
+  const int extH = (g.kH - 1) * g.dilH + 1, extW = (g.kW - 1) * g.dilW + 1;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    int w = (int)(i % g.W);
+    long t = i / g.W;
+    int h = (int)(t % g.H);
+    long plane = t / g.H;
+    int phstart = (h + g.padH < extH) ? 0 : (h + g.padH - extH) / g.dH + 1;
+    int phend = min((h + g.padH) / g.dH + 1, g.oH);
+    int pwstart = (w + g.padW < extW) ? 0 : (w + g.padW - extW) / g.dW + 1;
+    int pwend = min((w + g.padW) / g.dW + 1, g.oW);
+    const float *gp = gradOut + plane * g.oH * g.oW;
+    const long *ix = indices + plane * g.oH * g.oW;
+    float grad = 0.f;
+    for (int ph = phstart; ph < phend; ++ph)
+      for (int pw = pwstart; pw < pwend; ++pw)
+        if (ix[ph * g.oW + pw] - TH_INDEX_BASE == (long)h * g.W + w) grad += gp[ph * g.oW + pw];
+    gradIn[i] = grad;
+  }
+}
+
+// ------------------------------------------------------- average: forward ----
+template <bool INCLUDE_PAD>
+__device__ __forceinline__ float avgDivisor(int ph, int pw, const PoolGeom &g, int &hs, int &he, int &ws, int &we) {
+  hs = ph * g.dH - g.padH;
+  ws = pw * g.dW - g.padW;
+  he = min(hs + g.kH, g.H + g.padH);
+  we = min(ws + g.kW, g.W + g.padW);
+  const int pool = (he - hs) * (we - ws);
+  hs = max(hs, 0);
+  ws = max(ws, 0);
+  he = min(he, g.H);
+  we = min(we, g.W);
+  return INCLUDE_PAD ? (float)pool : (float)((he - hs) * (we - ws));
+}
+
+template <bool INCLUDE_PAD, bool VEC>
+__global__ void __launch_bounds__(dev::kBlock)
+avgPoolFwdTiled(const float *__restrict__ in, float *__restrict__ out, PoolGeom g) {
+  extern __shared__ float smem[];
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  const int ph0 = tile * g.tileRows;
+  const int nOut = min(g.tileRows, g.oH - ph0);
+  const int hLo = max(0, ph0 * g.dH - g.padH);
+  const int hHi = min(g.H, (ph0 + nOut - 1) * g.dH - g.padH + g.kH);
+  dev::loadFlat<VEC>(smem, in + ((long)plane * g.H + hLo) * g.W, max(0, hHi - hLo) * g.W);
+  __syncthreads();
+  const long obase = ((long)plane * g.oH + ph0) * g.oW;
+  const int total = nOut * g.oW;
+  for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    int r = i / g.oW, pw = i - r * g.oW;
+    int hs, he, ws, we;
+    float div = avgDivisor<INCLUDE_PAD>(ph0 + r, pw, g, hs, he, ws, we);
+    float s = 0.f;
+    for (int h = hs; h < he; ++h)
+      for (int w = ws; w < we; ++w) s += smem[(h - hLo) * g.W + w];
+    out[obase + i] = s / div;
+  }
+}
+
+template <bool INCLUDE_PAD>
+__global__ void __launch_bounds__(dev::kBlock)
+avgPoolFwdDirect(const float *__restrict__ in, float *__restrict__ out, PoolGeom g, long total) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    int pw = (int)(i % g.oW);
+    long t = i / g.oW;
+    int ph = (int)(t % g.oH);
+    long plane = t / g.oH;
+    const float *ip = in + plane * g.H * g.W;
+    int hs, he, ws, we;
+    float div = avgDivisor<INCLUDE_PAD>(ph, pw, g, hs, he, ws, we);
+    float s = 0.f;
+    for (int h = hs; h < he; ++h)
+      for (int w = ws; w < we; ++w) s += ip[(long)h * g.W + w];
+    out[i] = s / div;
+  }
+}
+
+// ------------------------------------------------------ average: backward ----
+template <bool INCLUDE_PAD>
+__device__ __forceinline__ float avgGather(const float *__restrict__ gp, int rowOff, int h, int w, const PoolGeom &g) {
+  const int hp = h + g.padH, wp = w + g.padW;
+  const int phstart = (hp < g.kH) ? 0 : (hp - g.kH) / g.dH + 1;
+  const int phend = min(hp / g.dH + 1, g.oH);
+  const int pwstart = (wp < g.kW) ? 0 : (wp - g.kW) / g.dW + 1;
+  const int pwend = min(wp / g.dW + 1, g.oW);
+  float grad = 0.f;
+  for (int ph = phstart; ph < phend; ++ph)
+    for (int pw = pwstart; pw < pwend; ++pw) {
+      int hs, he, ws, we;
+      float div = avgDivisor<INCLUDE_PAD>(ph, pw, g, hs, he, ws, we);
+      grad += gp[(ph - rowOff) * g.oW + pw] / div;
+    }
+  return grad;
+}
+
+template <bool INCLUDE_PAD, bool VEC>
+__global__ void __launch_bounds__(dev::kBlock)
+avgPoolBwdTiled(const float *__restrict__ gradOut, float *__restrict__ gradIn, PoolGeom g) {
+  extern __shared__ float smem[];
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  const int h0 = tile * g.tileRows;
+  const int nRows = min(g.tileRows, g.H - h0);
+  const int phLo = max(0, dev::ceilDivPos(h0 + g.padH - g.kH + 1, g.dH));
+  const int phHi = min(g.oH - 1, (h0 + nRows - 1 + g.padH) / g.dH);
+  const int nPh = max(0, phHi - phLo + 1);
+  dev::loadFlat<VEC>(smem, gradOut + ((long)plane * g.oH + phLo) * g.oW, nPh * g.oW);
+  __syncthreads();
+  float *o = gradIn + ((long)plane * g.H + h0) * g.W;
+  const int total = nRows * g.W;
+  for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    int r = i / g.W, w = i - r * g.W;
+    o[i] = avgGather<INCLUDE_PAD>(smem, phLo, h0 + r, w, g);
+  }
+}
+
+template <bool INCLUDE_PAD>
+__global__ void __launch_bounds__(dev::kBlock)
+avgPoolBwdDirect(const float *__restrict__ gradOut, float *__restrict__ gradIn, PoolGeom g, long total) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    int w = (int)(i % g.W);
+    long t = i / g.W;
+    int h = (int)(t % g.H);
+    long plane = t / g.H;
+    gradIn[i] = avgGather<INCLUDE_PAD>(gradOut + plane * g.oH * g.oW, 0, h, w, g);
+  }
+}
+
+// -------------------------------------------------------------- host side ----
+using launch::aligned16;
+
+bool forceDirect() {
+  const char *e = getenv("THCUNN_POOL_FORCE_DIRECT");
+  return e && e[0] == '1';
+}
+
+// Output extent rule shared by max and average pooling
+// (lib/THCUNN/generic/SpatialDilatedMaxPooling.cu:47-64,
+//  lib/THCUNN/generic/SpatialAveragePooling.cu:41-58): float division,
+// floor/ceil, +1, then - only when padded - drop a last window that would start
+// beyond the input plus its leading pad.
+long poolExtent(long in, int k, int d, int pad, int dil, bool ceil_mode) {
+  float q = float(in - (dil * (k - 1) + 1) + 2 * pad) / float(d);
+  return (long)(ceil_mode ? ceilf(q) : floorf(q)) + 1;
+}
+
+struct PoolCall {
+  PoolGeom g;
+  long N, C;
+  bool batch;
+};
+
+// lib/THCUNN/generic/SpatialDilatedMaxPooling.cu:7-82 / generic/SpatialAveragePooling.cu:7-70
+PoolCall poolSetup(THCudaTensor *input, THCudaTensor *gradOutput, THCudaLongTensor *indices, int kH, int kW, int dH,
+                   int dW, int padH, int padW, int dilH, int dilW, bool ceil_mode, bool isMax) {
+  THC_ARG_CHECK(input != nullptr, 2, "input tensor expected");
+  THC_ARG_CHECK(kW > 0 && kH > 0, 5, "kernel size should be greater than zero, but got kH: %d kW: %d", kH, kW);
+  THC_ARG_CHECK(dW > 0 && dH > 0, 8, "stride should be greater than zero, but got dH: %d dW: %d", dH, dW);
+  if (isMax)
+    THC_ARG_CHECK(dilH > 0 && dilW > 0, 12,
+                  "dilation should be greater than zero, but got dilationH: %d dilationW: %d", dilH, dilW);
+  int ndim = input->nDimension;
+  int dimf = 0, dimh = 1, dimw = 2;
+  long batchSize = 1;
+  THC_ARG_CHECK(ndim == 3 || ndim == 4, 2, "3D or 4D input tensor expected but got: %s",
+                sizeDesc(erase(input)).c_str());
+  if (ndim == 4) {
+    batchSize = input->size[0];
+    dimf++;
+    dimh++;
+    dimw++;
+  }
+  THC_ARG_CHECK(kW / 2 >= padW && kH / 2 >= padH, 2,
+                "pad should be smaller than half of kernel size, but got padW = %d, padH = %d, kW = %d, kH = %d",
+                padW, padH, kW, kH);
+  long nInputPlane = input->size[dimh - 1];
+  long nInputRows = input->size[dimh], nInputCols = input->size[dimw];
+  long nOutputCols = poolExtent(nInputCols, kW, dW, padW, dilW, ceil_mode);
+  long nOutputRows = poolExtent(nInputRows, kH, dH, padH, dilH, ceil_mode);
+  if (padW || padH) {
+    if ((nOutputRows - 1) * dH >= nInputRows + padH) --nOutputRows;
+    if ((nOutputCols - 1) * dW >= nInputCols + padW) --nOutputCols;
+  }
+  if (nOutputCols < 1 || nOutputRows < 1)
+    error("Given input size: (%ldx%ldx%ld). Calculated output size: (%ldx%ldx%ld). Output size is too small",
+          nInputPlane, nInputRows, nInputCols, nInputPlane, nOutputRows, nOutputCols);
+  if (gradOutput) {
+    checkDimSize(erase(gradOutput), "gradOutput", ndim, dimf, nInputPlane);
+    checkDimSize(erase(gradOutput), "gradOutput", ndim, dimh, nOutputRows);
+    checkDimSize(erase(gradOutput), "gradOutput", ndim, dimw, nOutputCols);
+  }
+  if (indices) {
+    checkDimSize(erase(indices), "indices", 4, 0, batchSize);
+    checkDimSize(erase(indices), "indices", 4, 1, nInputPlane);
+    checkDimSize(erase(indices), "indices", 4, 2, nOutputRows);
+    checkDimSize(erase(indices), "indices", 4, 3, nOutputCols);
+  }
+  if (nInputRows * nInputCols >= 0x7fffffffL) error("input planes of 2^31 or more elements are not supported");
+  PoolCall c;
+  c.batch = ndim == 4;
+  c.N = batchSize;
+  c.C = nInputPlane;
+  PoolGeom &g = c.g;
+  g.H = (int)nInputRows, g.W = (int)nInputCols, g.oH = (int)nOutputRows, g.oW = (int)nOutputCols;
+  g.kH = kH, g.kW = kW, g.dH = dH, g.dW = dW, g.padH = padH, g.padW = padW, g.dilH = dilH, g.dilW = dilW;
+  g.tileRows = g.tilesPerPlane = g.nblk = g.maxStageRows = 0;
+  return c;
+}
+
+template <bool VEC>
+void launchMaxFwd(hipStream_t s, size_t lds, const float *in, float *out, long *idx, const PoolGeom &g) {
+  dim3 grid(g.nblk), block(dev::kBlock);
+  bool sq = g.kH == g.kW && g.dH == g.dW && g.dilH == 1 && g.dilW == 1;
+  if (sq && g.kH == 3 && g.dH == 2)
+    maxPoolFwdTiled<3, 2, VEC><<<grid, block, lds, s>>>(in, out, idx, g);
+  else if (sq && g.kH == 2 && g.dH == 2)
+    maxPoolFwdTiled<2, 2, VEC><<<grid, block, lds, s>>>(in, out, idx, g);
+  else if (sq && g.kH == 3 && g.dH == 1)
+    maxPoolFwdTiled<3, 1, VEC><<<grid, block, lds, s>>>(in, out, idx, g);
+  else
+    maxPoolFwdTiled<0, 0, VEC><<<grid, block, lds, s>>>(in, out, idx, g);
+}
+
+void maxPoolUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output, THCudaLongTensor *indices,
+                         int kW, int kH, int dW, int dH, int padW, int padH, int dilW, int dilH, bool ceil_mode) {
+  THC_ARG_CHECK(output != nullptr, 3, "output tensor expected");
+  THC_ARG_CHECK(indices != nullptr, 4, "indices tensor expected");
+  PoolCall call = poolSetup(input, nullptr, nullptr, kH, kW, dH, dW, padH, padW, dilH, dilW, ceil_mode, true);
+  PoolGeom &g = call.g;
+  Contiguous in(state, input);
+  resize(state, output, {call.N, call.C, g.oH, g.oW});
+  resize(state, indices, {call.N, call.C, g.oH, g.oW});  // always 4-D (:140-141)
+  if (!isContiguous(erase(output)) || !isContiguous(erase(indices)))
+    error("output and indices tensors have to be contiguous");
+  hipStream_t s = state->stream;
+  const long planes = call.N * call.C;
+  if (planes > 0) {
+    bool vec = g.W % 4 == 0 && aligned16(in.ptr());
+    auto stageRows = [&](int rows) { return std::min(g.H, (rows - 1) * g.dH + (g.kH - 1) * g.dilH + 1); };
+    auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.W * sizeof(float); };
+    if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
+      g.nblk = (int)(planes * g.tilesPerPlane);
+      if (vec)
+        launchMaxFwd<true>(s, bytes(g.tileRows), in.ptr(), data(output), data(indices), g);
+      else
+        launchMaxFwd<false>(s, bytes(g.tileRows), in.ptr(), data(output), data(indices), g);
+    } else {
+      long total = planes * g.oH * g.oW;
+      maxPoolFwdDirect<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(in.ptr(), data(output),
+                                                                                      data(indices), g, total);
+    }
+    THC_HIP_CHECK(hipGetLastError());
+  }
+  if (!call.batch) resize(state, output, {call.C, g.oH, g.oW});
+}
+
+void maxPoolUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradInput,
+                            THCudaLongTensor *indices, int kW, int kH, int dW, int dH, int padW, int padH, int dilW,
+                            int dilH, bool ceil_mode) {
+  THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
+  THC_ARG_CHECK(gradInput != nullptr, 4, "gradInput tensor expected");
+  THC_ARG_CHECK(indices != nullptr, 5, "indices tensor expected");
+  PoolCall call = poolSetup(input, gradOutput, indices, kH, kW, dH, dW, padH, padW, dilH, dilW, ceil_mode, true);
+  PoolGeom &g = call.g;
+  Contiguous go(state, gradOutput);
+  if (!isContiguous(erase(indices))) error("indices tensor has to be contiguous");
+  if (call.batch)
+    resize(state, gradInput, {call.N, call.C, g.H, g.W});
+  else
+    resize(state, gradInput, {call.C, g.H, g.W});
+  if (!isContiguous(erase(gradInput))) error("gradInput tensor has to be contiguous");
+  hipStream_t s = state->stream;
+  const long planes = call.N * call.C;
+  if (planes == 0) return;
+  const int extH = (g.kH - 1) * g.dilH + 1;
+  bool vec = g.oW % 4 == 0 && aligned16(go.ptr());
+  auto stageRows = [&](int rows) { return std::min(g.oH, (rows + extH - 2) / g.dH + 2); };
+  auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.oW * (sizeof(float) + sizeof(int)); };
+  if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
+    g.nblk = (int)(planes * g.tilesPerPlane);
+    g.maxStageRows = stageRows(g.tileRows);
+    dim3 grid(g.nblk), block(dev::kBlock);
+    if (vec)
+      maxPoolBwdTiled<true><<<grid, block, bytes(g.tileRows), s>>>(go.ptr(), data(indices), data(gradInput), g);
+    else
+      maxPoolBwdTiled<false><<<grid, block, bytes(g.tileRows), s>>>(go.ptr(), data(indices), data(gradInput), g);
+  } else {
+    long total = planes * g.H * g.W;
+    maxPoolBwdDirect<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(go.ptr(), data(indices),
+                                                                                    data(gradInput), g, total);
+  }
+  THC_HIP_CHECK(hipGetLastError());
+}
+
+}  // namespace
+
+extern "C" {
+
+void THNN_CudaSpatialDilatedMaxPooling_updateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output,
+                                                    THCudaLongTensor *indices, int kW, int kH, int dW, int dH,
+                                                    int padW, int padH, int dilationW, int dilationH,
+                                                    bool ceil_mode) {
+  THNN_ENTER
+  maxPoolUpdateOutput(state, input, output, indices, kW, kH, dW, dH, padW, padH, dilationW, dilationH, ceil_mode);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialDilatedMaxPooling_updateGradInput(THCState *state, THCudaTensor *input,
+                                                       THCudaTensor *gradOutput, THCudaTensor *gradInput,
+                                                       THCudaLongTensor *indices, int kW, int kH, int dW, int dH,
+                                                       int padW, int padH, int dilationW, int dilationH,
+                                                       bool ceil_mode) {
+  THNN_ENTER
+  maxPoolUpdateGradInput(state, input, gradOutput, gradInput, indices, kW, kH, dW, dH, padW, padH, dilationW,
+                         dilationH, ceil_mode);
+  THNN_LEAVE
+}
+
+// lib/THCUNN/generic/SpatialMaxPooling.cu:7-38: dilation 1
+void THNN_CudaSpatialMaxPooling_updateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output,
+                                             THCudaLongTensor *indices, int kW, int kH, int dW, int dH, int padW,
+                                             int padH, bool ceil_mode) {
+  THNN_ENTER
+  maxPoolUpdateOutput(state, input, output, indices, kW, kH, dW, dH, padW, padH, 1, 1, ceil_mode);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialMaxPooling_updateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput,
+                                                THCudaTensor *gradInput, THCudaLongTensor *indices, int kW, int kH,
+                                                int dW, int dH, int padW, int padH, bool ceil_mode) {
+  THNN_ENTER
+  maxPoolUpdateGradInput(state, input, gradOutput, gradInput, indices, kW, kH, dW, dH, padW, padH, 1, 1, ceil_mode);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output, int kW,
+                                                 int kH, int dW, int dH, int padW, int padH, bool ceil_mode,
+                                                 bool count_include_pad) {
+  THNN_ENTER
+  THC_ARG_CHECK(output != nullptr, 3, "output tensor expected");
+  PoolCall call = poolSetup(input, nullptr, nullptr, kH, kW, dH, dW, padH, padW, 1, 1, ceil_mode, false);
+  PoolGeom &g = call.g;
+  Contiguous in(state, input);
+  resize(state, output, {call.N, call.C, g.oH, g.oW});
+  if (!isContiguous(erase(output))) error("output tensor has to be contiguous");
+  hipStream_t s = state->stream;
+  const long planes = call.N * call.C;
+  if (planes > 0) {
+    bool vec = g.W % 4 == 0 && aligned16(in.ptr());
+    auto stageRows = [&](int rows) { return std::min(g.H, (rows - 1) * g.dH + g.kH); };
+    auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.W * sizeof(float); };
+    if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
+      g.nblk = (int)(planes * g.tilesPerPlane);
+      dim3 grid(g.nblk), block(dev::kBlock);
+      size_t lds = bytes(g.tileRows);
+      if (count_include_pad) {
+        if (vec)
+          avgPoolFwdTiled<true, true><<<grid, block, lds, s>>>(in.ptr(), data(output), g);
+        else
+          avgPoolFwdTiled<true, false><<<grid, block, lds, s>>>(in.ptr(), data(output), g);
+      } else {
+        if (vec)
+          avgPoolFwdTiled<false, true><<<grid, block, lds, s>>>(in.ptr(), data(output), g);
+        else
+          avgPoolFwdTiled<false, false><<<grid, block, lds, s>>>(in.ptr(), data(output), g);
+      }
+    } else {
+      long total = planes * g.oH * g.oW;
+      unsigned grid = launch::directGrid(total, dev::kBlock);
+      if (count_include_pad)
+        avgPoolFwdDirect<true><<<grid, dev::kBlock, 0, s>>>(in.ptr(), data(output), g, total);
+      else
+        avgPoolFwdDirect<false><<<grid, dev::kBlock, 0, s>>>(in.ptr(), data(output), g, total);
+    }
+    THC_HIP_CHECK(hipGetLastError());
+  }
+  if (!call.batch) resize(state, output, {call.C, g.oH, g.oW});
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput,
+                                                    THCudaTensor *gradInput, int kW, int kH, int dW, int dH,
+                                                    int padW, int padH, bool ceil_mode, bool count_include_pad) {
+  THNN_ENTER
+  THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
+  THC_ARG_CHECK(gradInput != nullptr, 4, "gradInput tensor expected");
+  PoolCall call = poolSetup(input, gradOutput, nullptr, kH, kW, dH, dW, padH, padW, 1, 1, ceil_mode, false);
+  PoolGeom &g = call.g;
+  Contiguous go(state, gradOutput);
+  if (call.batch)
+    resize(state, gradInput, {call.N, call.C, g.H, g.W});
+  else
+    resize(state, gradInput, {call.C, g.H, g.W});
+  if (!isContiguous(erase(gradInput))) error("gradInput tensor has to be contiguous");
+  hipStream_t s = state->stream;
+  const long planes = call.N * call.C;
+  if (planes == 0) return;
+  bool vec = g.oW % 4 == 0 && aligned16(go.ptr());
+  auto stageRows = [&](int rows) { return std::min(g.oH, (rows + g.kH - 2) / g.dH + 2); };
+  auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.oW * sizeof(float); };
+  if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
+    g.nblk = (int)(planes * g.tilesPerPlane);
+    dim3 grid(g.nblk), block(dev::kBlock);
+    size_t lds = bytes(g.tileRows);
+    if (count_include_pad) {
+      if (vec)
+        avgPoolBwdTiled<true, true><<<grid, block, lds, s>>>(go.ptr(), data(gradInput), g);
+      else
+        avgPoolBwdTiled<true, false><<<grid, block, lds, s>>>(go.ptr(), data(gradInput), g);
+    } else {
+      if (vec)
+        avgPoolBwdTiled<false, true><<<grid, block, lds, s>>>(go.ptr(), data(gradInput), g);
+      else
+        avgPoolBwdTiled<false, false><<<grid, block, lds, s>>>(go.ptr(), data(gradInput), g);
+    }
+  } else {
+    long total = planes * g.H * g.W;
+    unsigned grid = launch::directGrid(total, dev::kBlock);
+    if (count_include_pad)
+      avgPoolBwdDirect<true><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g, total);
+    else
+      avgPoolBwdDirect<false><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g, total);
+  }
+  THC_HIP_CHECK(hipGetLastError());
+  THNN_LEAVE
+}
+
+}  // extern "C"

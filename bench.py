@@ -1,0 +1,395 @@
+#!/usr/bin/env python3
+"""Benchmark of the THCUNN spatial-conv hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2] [--all]
+
+A step is one pass of the workload's entry points over one synthetic batch,
+called through the C ABI of libTHCUNN.so. The default workload is the one the
+headline metric is quoted on: SpatialDepthWiseConvolution forward +
+updateGradInput + accGradParameters, fp32, N=64 C=128 56x56 -> 28x28, 3x3
+stride 2 pad 1 (BASELINE.json configs[1]). Inputs live in HBM before the timed
+region; four buffer sets are rotated so that no step finds its inputs in the
+256 MB Infinity Cache from the step before.
+
+Prints ONE JSON line: images/s for the whole job, plus
+  roofline     - the dominant kernel's algorithmic bytes (or flops) per launch
+                 over its average duration measured with HIP events on the
+                 stream the kernels run on, against MI355X's published peak;
+  cpu_baseline - the CPU oracle (a port of the reference algorithm) timed on
+                 this host's cores on a bounded sample of the same workload;
+  workloads    - with --all, the same figures for the other four configurations.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+FP32_MFMA_PEAK_TFLOPS = 157.3
+METRIC = "DW-conv fwd+bwd images/s + achieved HBM GB/s (% of peak), 1 MI355X"
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/dwconv_cfg2_pmc.txt gives the runs and the copy-kernel scale factor);
+# None until a counter run exists for that kernel.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+class Hip:
+    def __init__(self):
+        self.lib = C.CDLL("libamdhip64.so")
+        self.lib.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.lib.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.lib.hipEventSynchronize.argtypes = [C.c_void_p]
+
+    def check(self, rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what} failed with hipError {rc}")
+
+    def event(self):
+        e = C.c_void_p()
+        self.check(self.lib.hipEventCreate(C.byref(e)), "hipEventCreate")
+        return e
+
+    def record(self, e, stream):
+        self.check(self.lib.hipEventRecord(e, stream), "hipEventRecord")
+
+    def elapsed_ms(self, a, b):
+        self.check(self.lib.hipEventSynchronize(b), "hipEventSynchronize")
+        ms = C.c_float()
+        self.check(self.lib.hipEventElapsedTime(C.byref(ms), a, b), "hipEventElapsedTime")
+        return float(ms.value)
+
+    def sync(self):
+        self.check(self.lib.hipDeviceSynchronize(), "hipDeviceSynchronize")
+
+
+# --------------------------------------------------------------- workloads ----
+# Each workload builds `nsets` independent buffer sets and returns
+#   calls(set_index) -> list of (kernel_name, fn)       the step, in order
+#   work              -> {kernel_name: (amount, "bytes"|"flops")} algorithmic work per launch
+#   images            -> batch size
+#   cpu(sample)       -> (seconds, images) of the oracle on a bounded sample
+
+def _kaiming_uniform(rng, shape, fan_in):
+    b = np.sqrt(6.0 / fan_in)
+    return rng.uniform(-b, b, shape).astype(np.float32)
+
+
+def wl_dw(cfg, nsets):
+    from cunn_amd import CudaTensor as CT, THNN
+    from oracle import oracle as O
+    if cfg == "cfg1":
+        N, Cc, H, k, s, p, seed, full = 32, 32, 112, 3, 1, 1, 0, False
+    else:
+        N, Cc, H, k, s, p, seed, full = 64, 128, 56, 3, 2, 1, 1, True
+    oH = (H + 2 * p - k) // s + 1
+    rng = np.random.default_rng(seed)
+    x = (rng.uniform(-1, 1, (N, Cc, H, H)) if cfg == "cfg1" else rng.standard_normal((N, Cc, H, H))).astype(np.float32)
+    w = _kaiming_uniform(rng, (1, Cc, k, k), k * k)
+    b = rng.uniform(-1 / 3, 1 / 3, (1, Cc)).astype(np.float32)
+    gy = rng.standard_normal((N, Cc, oH, oH)).astype(np.float32)
+    sets = []
+    for _ in range(nsets):
+        sets.append(dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), gx=CT(), w=CT.from_numpy(w),
+                         b=CT.from_numpy(b), gw=CT.from_numpy(np.zeros_like(w)), gb=CT.from_numpy(np.zeros_like(b)),
+                         cols=CT(), ones=CT()))
+    xb, yb = x.nbytes, gy.nbytes
+
+    def calls(i):
+        t = sets[i]
+        g = (k, k, s, s, p, p)
+        fwd = ("dw_updateOutput", lambda: THNN.SpatialDepthWiseConvolution_updateOutput(
+            t["x"], t["y"], t["w"], t["b"], t["cols"], t["ones"], *g))
+        if not full:
+            return [fwd]
+        return [fwd,
+                ("dw_updateGradInput", lambda: THNN.SpatialDepthWiseConvolution_updateGradInput(
+                    t["x"], t["gy"], t["gx"], t["w"], t["cols"], t["ones"], *g)),
+                ("dw_accGradParameters", lambda: THNN.SpatialDepthWiseConvolution_accGradParameters(
+                    t["x"], t["gy"], t["gw"], t["gb"], t["cols"], t["ones"], *g, 1.0))]
+
+    work = {"dw_updateOutput": (xb + yb, "bytes"), "dw_updateGradInput": (xb + yb, "bytes"),
+            "dw_accGradParameters": (xb + yb, "bytes")}
+
+    def cpu(reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            O.dwconv_updateOutput(x, w, b, k, k, s, s, p, p)
+            if full:
+                O.dwconv_updateGradInput(x.shape, gy, w, k, k, s, s, p, p)
+                O.dwconv_accGradParameters(x, gy, np.zeros_like(w), np.zeros_like(b), k, k, s, s, p, p, 1.0)
+        return time.perf_counter() - t0, reps * N, f"{reps} full passes of {cfg} ({N} images each)"
+
+    def verify():
+        t = sets[0]
+        for _, fn in calls(0):
+            fn()
+        np.testing.assert_allclose(t["y"].numpy(), O.dwconv_updateOutput(x, w, b, k, k, s, s, p, p), rtol=1e-5, atol=1e-4)
+        if full:
+            np.testing.assert_allclose(t["gx"].numpy(), O.dwconv_updateGradInput(x.shape, gy, w, k, k, s, s, p, p),
+                                       rtol=1e-5, atol=1e-4)
+            rgw, rgb = O.dwconv_accGradParameters(x, gy, np.zeros_like(w), np.zeros_like(b), k, k, s, s, p, p, 1.0)
+            np.testing.assert_allclose(t["gw"].numpy(), rgw, rtol=1e-3, atol=1e-3)
+            np.testing.assert_allclose(t["gb"].numpy(), rgb, rtol=1e-3, atol=1e-3)
+            t["gw"].fill(0.0), t["gb"].fill(0.0)
+
+    desc = (f"SpatialDepthWiseConvolution {'fwd+gradInput+accGradParameters' if full else 'fwd'} fp32 "
+            f"N={N} C={Cc} {H}x{H}->{oH}x{oH} k{k} s{s} p{p} M=1")
+    return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, desc=desc, bound="hbm")
+
+
+def wl_bn(nsets):
+    from cunn_amd import CudaTensor as CT, THNN
+    from oracle import oracle as O
+    N, Cc, H = 64, 256, 28
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal((N, Cc, H, H)) * 2 + 0.5).astype(np.float32)
+    gy = rng.standard_normal((N, Cc, H, H)).astype(np.float32)
+    g = rng.random(Cc).astype(np.float32)
+    b = np.zeros(Cc, np.float32)
+    sets = []
+    for _ in range(nsets):
+        sets.append(dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), gx=CT.with_size(N, Cc, H, H), g=CT.from_numpy(g),
+                         b=CT.from_numpy(b), rm=CT.from_numpy(np.zeros(Cc, np.float32)),
+                         rv=CT.from_numpy(np.ones(Cc, np.float32)), sm=CT.with_size(Cc), ss=CT.with_size(Cc),
+                         gw=CT.from_numpy(np.zeros(Cc, np.float32)), gb=CT.from_numpy(np.zeros(Cc, np.float32))))
+
+    def calls(i):
+        t = sets[i]
+        return [("bn_updateOutput", lambda: THNN.BatchNormalization_updateOutput(
+                    t["x"], t["y"], t["g"], t["b"], t["rm"], t["rv"], t["sm"], t["ss"], True, 0.1, 1e-5)),
+                ("bn_backward", lambda: THNN.BatchNormalization_backward(
+                    t["x"], t["gy"], t["gx"], t["gw"], t["gb"], t["g"], t["rm"], t["rv"], t["sm"], t["ss"], True, 1.0, 1e-5))]
+
+    work = {"bn_updateOutput": (2 * x.nbytes, "bytes"), "bn_backward": (3 * x.nbytes, "bytes")}
+
+    def cpu(reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            rm, rv = np.zeros(Cc, np.float32), np.ones(Cc, np.float32)
+            _, sm, ss = O.bn_updateOutput(x, g, b, rm, rv, True, 0.1, 1e-5)
+            O.bn_backward(x, gy, g, rm, rv, sm, ss, True, 1.0, 1e-5, np.zeros(Cc, np.float32), np.zeros(Cc, np.float32))
+        return time.perf_counter() - t0, reps * N, f"{reps} full passes of cfg3 ({N} images each)"
+
+    def verify():
+        t = sets[0]
+        for _, fn in calls(0):
+            fn()
+        rm, rv = np.zeros(Cc, np.float32), np.ones(Cc, np.float32)
+        ry, sm, ss = O.bn_updateOutput(x, g, b, rm, rv, True, 0.1, 1e-5)
+        np.testing.assert_allclose(t["y"].numpy(), ry, rtol=1e-5, atol=2e-4)
+        np.testing.assert_allclose(t["ss"].numpy(), ss, rtol=1e-3)
+        rgi, rgw, _ = O.bn_backward(x, gy, g, rm, rv, sm, ss, True, 1.0, 1e-5, np.zeros(Cc, np.float32), np.zeros(Cc, np.float32))
+        np.testing.assert_allclose(t["gx"].numpy(), rgi, rtol=1e-4, atol=2e-4)
+        np.testing.assert_allclose(t["gw"].numpy(), rgw, rtol=1e-3, atol=1e-2)
+
+    return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="hbm",
+                desc=f"SpatialBatchNormalization train fwd+bwd fp32 N={N} C={Cc} {H}x{H} affine eps=1e-5 momentum=0.1")
+
+
+def wl_pool(nsets):
+    from cunn_amd import CudaLongTensor as LT, CudaTensor as CT, THNN
+    from oracle import oracle as O
+    N, Cc, H = 64, 64, 112
+    rng = np.random.default_rng(3)
+    x = (np.round(rng.uniform(-1, 1, (N, Cc, H, H)) * 64) / 64).astype(np.float32)
+    gy = rng.standard_normal((N, Cc, 56, 56)).astype(np.float32)
+    sets = []
+    for _ in range(nsets):
+        sets.append(dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), idx=LT(), gx=CT(), ya=CT(), gxa=CT()))
+
+    def calls(i):
+        t = sets[i]
+        return [("maxpool_updateOutput", lambda: THNN.SpatialMaxPooling_updateOutput(t["x"], t["y"], t["idx"], 3, 3, 2, 2, 1, 1, False)),
+                ("maxpool_updateGradInput", lambda: THNN.SpatialMaxPooling_updateGradInput(t["x"], t["gy"], t["gx"], t["idx"], 3, 3, 2, 2, 1, 1, False)),
+                ("avgpool_updateOutput", lambda: THNN.SpatialAveragePooling_updateOutput(t["x"], t["ya"], 2, 2, 2, 2, 0, 0, False, True)),
+                ("avgpool_updateGradInput", lambda: THNN.SpatialAveragePooling_updateGradInput(t["x"], t["gy"], t["gxa"], 2, 2, 2, 2, 0, 0, False, True))]
+
+    xb, yb = x.nbytes, gy.nbytes
+    work = {"maxpool_updateOutput": (xb + yb + 2 * yb, "bytes"), "maxpool_updateGradInput": (yb + 2 * yb + xb, "bytes"),
+            "avgpool_updateOutput": (xb + yb, "bytes"), "avgpool_updateGradInput": (yb + xb, "bytes")}
+
+    def cpu(reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            _, idx = O.maxpool_updateOutput(x, 3, 3, 2, 2, 1, 1, False)
+            O.maxpool_updateGradInput(x.shape, gy, idx, 3, 3, 2, 2, 1, 1, False)
+            O.avgpool_updateOutput(x, 2, 2, 2, 2, 0, 0, False, True)
+            O.avgpool_updateGradInput(x.shape, gy, 2, 2, 2, 2, 0, 0, False, True)
+        return time.perf_counter() - t0, reps * N, f"{reps} full passes of cfg4 ({N} images each)"
+
+    def verify():
+        t = sets[0]
+        for _, fn in calls(0):
+            fn()
+        ry, ridx = O.maxpool_updateOutput(x, 3, 3, 2, 2, 1, 1, False)
+        assert np.array_equal(t["y"].numpy(), ry) and np.array_equal(t["idx"].numpy(), ridx)
+        np.testing.assert_allclose(t["gx"].numpy(), O.maxpool_updateGradInput(x.shape, gy, ridx, 3, 3, 2, 2, 1, 1, False), rtol=1e-5, atol=1e-4)
+        np.testing.assert_allclose(t["ya"].numpy(), O.avgpool_updateOutput(x, 2, 2, 2, 2, 0, 0, False, True), rtol=1e-5, atol=1e-4)
+        np.testing.assert_allclose(t["gxa"].numpy(), O.avgpool_updateGradInput(x.shape, gy, 2, 2, 2, 2, 0, 0, False, True), rtol=1e-5, atol=1e-4)
+
+    return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="hbm",
+                desc=f"SpatialMaxPooling 3x3 s2 p1 (+indices) and SpatialAveragePooling 2x2 s2, fwd+bwd fp32 N={N} C={Cc} 112x112->56x56")
+
+
+def wl_conv(nsets):
+    from cunn_amd import CudaTensor as CT, THNN
+    from oracle import oracle as O
+    N, Ci, Co, H, k = 64, 256, 256, 28, 3
+    K = Ci * k * k
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((N, Ci, H, H)).astype(np.float32)
+    gy = rng.standard_normal((N, Co, H, H)).astype(np.float32)
+    w = (rng.standard_normal((Co, K)) * np.sqrt(2.0 / K)).astype(np.float32)
+    b = rng.uniform(-0.02, 0.02, Co).astype(np.float32)
+    sets = []
+    for _ in range(nsets):
+        sets.append(dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), gx=CT(), w=CT.from_numpy(w), b=CT.from_numpy(b),
+                         gw=CT.from_numpy(np.zeros_like(w)), gb=CT.from_numpy(np.zeros_like(b)), cols=CT(), gcols=CT(), ones=CT()))
+    g = (k, k, 1, 1, 1, 1)
+
+    def calls(i):
+        t = sets[i]
+        return [("convmm_updateOutput", lambda: THNN.SpatialConvolutionMM_updateOutput(t["x"], t["y"], t["w"], t["b"], t["cols"], t["ones"], *g)),
+                ("convmm_updateGradInput", lambda: THNN.SpatialConvolutionMM_updateGradInput(t["x"], t["gy"], t["gx"], t["w"], t["gcols"], t["ones"], *g)),
+                ("convmm_accGradParameters", lambda: THNN.SpatialConvolutionMM_accGradParameters(t["x"], t["gy"], t["gw"], t["gb"], t["cols"], t["ones"], *g, 1.0))]
+
+    fl = 2.0 * Co * K * H * H * N
+    work = {"convmm_updateOutput": (fl, "flops"), "convmm_updateGradInput": (fl, "flops"), "convmm_accGradParameters": (fl, "flops")}
+    ns = 4  # images of the CPU sample
+
+    def cpu(reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            O.convmm_updateOutput(x[:ns], w, b, *g)
+            O.convmm_updateGradInput((ns,) + x.shape[1:], gy[:ns], w, *g)
+            O.convmm_accGradParameters(x[:ns], gy[:ns], np.zeros_like(w), np.zeros_like(b), *g, 1.0)
+        return time.perf_counter() - t0, reps * ns, f"{reps} passes over the first {ns} of {N} images of cfg5"
+
+    def verify():
+        t = sets[0]
+        for _, fn in calls(0):
+            fn()
+        m = 2  # images checked against the oracle
+        np.testing.assert_allclose(t["y"].numpy()[:m], O.convmm_updateOutput(x[:m], w, b, *g), rtol=1e-5, atol=1e-4)
+        np.testing.assert_allclose(t["gx"].numpy()[:m], O.convmm_updateGradInput((m,) + x.shape[1:], gy[:m], w, *g), rtol=1e-5, atol=1e-4)
+        t["gw"].fill(0.0), t["gb"].fill(0.0)
+
+    return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="mfma",
+                desc=f"SpatialConvolutionMM fwd+gradInput+accGradParameters fp32 N={N} Cin={Ci} Cout={Co} {H}x{H} k3 s1 p1 bias")
+
+
+WORKLOADS = {"cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda n: wl_dw("cfg2", n), "cfg3": wl_bn, "cfg4": wl_pool,
+             "cfg5": wl_conv}
+
+
+def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds):
+    wl = WORKLOADS[name](nsets)
+    wl["verify"]()                       # parity against the oracle in this very run
+    names = [n for n, _ in wl["calls"](0)]
+    for i in range(warmup):
+        for _, fn in wl["calls"](i % nsets):
+            fn()
+    hip.sync()
+    ev = [[hip.event() for _ in range(len(names) + 1)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        calls = wl["calls"](i % nsets)
+        hip.record(ev[i][0], stream)
+        for j, (_, fn) in enumerate(calls):
+            fn()
+            hip.record(ev[i][j + 1], stream)
+    hip.sync()
+    wall = time.perf_counter() - t0
+    per_kernel = {n: [] for n in names}
+    for i in range(steps):
+        for j, n in enumerate(names):
+            per_kernel[n].append(hip.elapsed_ms(ev[i][j], ev[i][j + 1]))
+    kern = {}
+    for n in names:
+        avg = float(np.mean(per_kernel[n]))
+        amount, kind = wl["work"][n]
+        if kind == "bytes":
+            ach, peak, unit = amount / (avg * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
+        else:
+            ach, peak, unit = amount / (avg * 1e-3) / 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
+        kern[n] = dict(avg_ms=avg, min_ms=float(np.min(per_kernel[n])), achieved=ach, peak=peak, unit=unit,
+                       frac=ach / peak, algorithmic=amount, kind=kind)
+    ms_per_step = wall * 1e3 / steps
+    dominant = max(names, key=lambda n: kern[n]["avg_ms"])
+    d = kern[dominant]
+    roofline = dict(bound=wl["bound"], kernel=dominant, achieved=round(d["achieved"], 3), peak=d["peak"], unit=d["unit"],
+                    frac=round(d["frac"], 4), traffic=MEASURED_TRAFFIC_BYTES.get((name, dominant)),
+                    algorithmic_per_launch=d["algorithmic"], avg_launch_ms=round(d["avg_ms"], 5))
+    res = dict(workload=wl["desc"], images_per_s=wl["images"] / (ms_per_step * 1e-3), ms_per_step=ms_per_step,
+               device_ms_per_step=float(sum(kern[n]["avg_ms"] for n in names)), roofline=roofline,
+               kernels={n: {k: (round(v, 5) if isinstance(v, float) else v) for k, v in kern[n].items()} for n in names})
+    if cpu_seconds > 0:
+        from oracle import oracle as O
+        sec, imgs, sample = wl["cpu"](1)          # calibrate
+        reps = max(1, min(50, int(cpu_seconds / max(sec, 1e-3))))
+        sec, imgs, sample = wl["cpu"](reps)
+        res["cpu_baseline"] = dict(value=round(imgs / sec, 2), unit="images/s", cores=O.num_threads(), kind="port",
+                                   sample=sample + f", {sec:.1f} s of CPU time; oracle/thnn_oracle.c with OpenMP")
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--all", action="store_true", help="also time the other four configurations")
+    ap.add_argument("--sets", type=int, default=4, help="buffer sets rotated between steps (1 = cache-warm variant)")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU time budget of the oracle baseline (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
+              "(the path shards by batch, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import cunn_amd
+    from cunn_amd.tensor import state
+    lib = cunn_amd._lib.load()   # raises if libTHCUNN.so is missing: there is no fallback path
+    st = state()
+    stream = lib.THCState_getCurrentStream(st)
+    hip = Hip()
+
+    main_res = run_workload(args.workload, args.steps, args.warmup, hip, stream, args.sets, args.cpu_seconds)
+    out = {
+        "metric": METRIC, "value": round(main_res["images_per_s"], 1), "unit": "images/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(main_res["ms_per_step"], 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {main_res['workload']}", "buffer_sets": args.sets,
+                   "entry": "C ABI libTHCUNN.so (THNN_Cuda*) via ctypes"},
+        "device_ms_per_step": round(main_res["device_ms_per_step"], 5),
+        "roofline": main_res["roofline"],
+        "cpu_baseline": main_res.get("cpu_baseline"),
+        "kernels": main_res["kernels"],
+    }
+    if args.all:
+        others = {}
+        for name in sorted(WORKLOADS):
+            if name == args.workload:
+                continue
+            r = run_workload(name, max(20, args.steps // 4), max(5, args.warmup // 2), hip, stream,
+                             args.sets, min(args.cpu_seconds, 8.0))
+            others[name] = dict(workload=r["workload"], images_per_s=round(r["images_per_s"], 1),
+                                ms_per_step=round(r["ms_per_step"], 5), roofline=r["roofline"],
+                                cpu_baseline=r.get("cpu_baseline"), kernels=r["kernels"])
+        out["workloads"] = others
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

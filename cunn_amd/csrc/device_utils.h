@@ -11,10 +11,27 @@ constexpr int kWave = 64;     // CDNA wavefront width
 constexpr int kXcds = 8;      // MI355X: 8 XCDs, each with its own L2
 constexpr int kBlock = 256;   // 4 wavefronts per workgroup
 
+// v + (v of the lane selected by the DPP control), computed on the VALU: no LDS
+// crossbar traffic, unlike ds_bpermute-based shuffles.
+template <int CTRL>
+__device__ __forceinline__ float dppAdd(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over the 64 lanes of a wavefront, returned in every lane (wave-uniform).
+// Four DPP steps fold each row of 16 lanes (quad xor 1, quad xor 2, half-row
+// mirror, row mirror), then the four row sums are read as scalars and added.
 __device__ __forceinline__ float waveSum(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-  return v;
+  v = dppAdd<0xB1>(v);   // quad_perm [1,0,3,2]
+  v = dppAdd<0x4E>(v);   // quad_perm [2,3,0,1]
+  v = dppAdd<0x141>(v);  // row_half_mirror
+  v = dppAdd<0x140>(v);  // row_mirror
+  const int b = __builtin_bit_cast(int, v);
+  float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+  float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+  float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return (r0 + r1) + (r2 + r3);
 }
 
 // Workgroups are handed to the XCDs round-robin (block b runs on XCD b % 8).
@@ -31,6 +48,12 @@ __device__ __forceinline__ int ceilDivPos(int a, int b) {  // ceil(a / b) for b 
   return (a >= 0) ? (a + b - 1) / b : -((-a) / b);
 }
 
+// Number of independent 16-byte (or 4-byte) global loads a lane keeps in flight
+// before it starts storing to LDS: the loads of one batch are issued back to
+// back, so a band costs ceil(per-lane loads / kLoadBatch) memory round trips
+// instead of one round trip per load.
+constexpr int kLoadBatch = 4;
+
 // Copies rows [r0, r0 + nRows) of a (H x W) plane into LDS at
 //   dst[r * pitch + padL + col],  r = 0 .. nRows-1, col = 0 .. W-1
 // Rows outside the plane are zero-filled and so are the padL cells in front of
@@ -46,19 +69,38 @@ __device__ __forceinline__ void loadRowsPadded(float *__restrict__ dst, const fl
   if (VEC) {
     const int W4 = W >> 2;
     const int total = nRows * W4;
-    for (int i = tid; i < total; i += nt) {
-      int r = i / W4, c4 = i - r * W4;
-      int gr = r0 + r;
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (gr >= 0 && gr < H) v = reinterpret_cast<const float4 *>(plane + (long)gr * W)[c4];
-      *reinterpret_cast<float4 *>(dst + r * pitch + padL + (c4 << 2)) = v;
+    for (int base = 0; base < total; base += kLoadBatch * nt) {
+      float4 v[kLoadBatch];
+      int off[kLoadBatch];
+#pragma unroll
+      for (int u = 0; u < kLoadBatch; ++u) {
+        int i = base + u * nt + tid;
+        int r = i / W4, c4 = i - r * W4;
+        int gr = r0 + r;
+        off[u] = (i < total) ? r * pitch + padL + (c4 << 2) : -1;
+        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < total && gr >= 0 && gr < H) v[u] = reinterpret_cast<const float4 *>(plane + (long)gr * W)[c4];
+      }
+#pragma unroll
+      for (int u = 0; u < kLoadBatch; ++u)
+        if (off[u] >= 0) *reinterpret_cast<float4 *>(dst + off[u]) = v[u];
     }
   } else {
     const int total = nRows * W;
-    for (int i = tid; i < total; i += nt) {
-      int r = i / W, c = i - r * W;
-      int gr = r0 + r;
-      dst[r * pitch + padL + c] = (gr >= 0 && gr < H) ? plane[(long)gr * W + c] : 0.f;
+    for (int base = 0; base < total; base += kLoadBatch * nt) {
+      float v[kLoadBatch];
+      int off[kLoadBatch];
+#pragma unroll
+      for (int u = 0; u < kLoadBatch; ++u) {
+        int i = base + u * nt + tid;
+        int r = i / W, c = i - r * W;
+        int gr = r0 + r;
+        off[u] = (i < total) ? r * pitch + padL + c : -1;
+        v[u] = (i < total && gr >= 0 && gr < H) ? plane[(long)gr * W + c] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < kLoadBatch; ++u)
+        if (off[u] >= 0) dst[off[u]] = v[u];
     }
   }
   if (padL > 0) {
@@ -77,10 +119,96 @@ __device__ __forceinline__ void loadFlat(T *__restrict__ dst, const T *__restric
   const int tid = threadIdx.x, nt = blockDim.x;
   if (VEC && sizeof(T) == 4) {
     const int n4 = count >> 2;
-    for (int i = tid; i < n4; i += nt)
-      reinterpret_cast<float4 *>(dst)[i] = reinterpret_cast<const float4 *>(src)[i];
+    for (int base = 0; base < n4; base += kLoadBatch * nt) {
+      float4 v[kLoadBatch];
+#pragma unroll
+      for (int u = 0; u < kLoadBatch; ++u) {
+        int i = base + u * nt + tid;
+        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < n4) v[u] = reinterpret_cast<const float4 *>(src)[i];
+      }
+#pragma unroll
+      for (int u = 0; u < kLoadBatch; ++u) {
+        int i = base + u * nt + tid;
+        if (i < n4) reinterpret_cast<float4 *>(dst)[i] = v[u];
+      }
+    }
   } else {
-    for (int i = tid; i < count; i += nt) dst[i] = src[i];
+    for (int base = 0; base < count; base += kLoadBatch * nt) {
+      T v[kLoadBatch];
+#pragma unroll
+      for (int u = 0; u < kLoadBatch; ++u) {
+        int i = base + u * nt + tid;
+        v[u] = T(0);
+        if (i < count) v[u] = src[i];
+      }
+#pragma unroll
+      for (int u = 0; u < kLoadBatch; ++u) {
+        int i = base + u * nt + tid;
+        if (i < count) dst[i] = v[u];
+      }
+    }
+  }
+}
+
+// De-interleaving variant for stride-2 consumers: row r of the band is stored as
+//   dst[r * pitch + 4 + m]           = x[r][2m]      (even columns)
+//   dst[r * pitch + oddOff + m]      = x[r][2m + 1]  (odd columns), oddOff = W/2 + 8
+// with 4 zero cells in front of each half and 4 after the last row, so that a
+// lane reading 4 consecutive even (or odd) columns issues one 16-byte LDS read at
+// unit stride across lanes instead of a 32-byte-strided one (which maps 64 lanes
+// onto 8 banks). Requires W % 8 == 0, pitch % 4 == 0, 16-byte aligned plane.
+__device__ __forceinline__ void loadRowsSplit(float *__restrict__ dst, const float *__restrict__ plane, int H, int W,
+                                              int r0, int nRows, int pitch) {
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int W4 = W >> 2;
+  const int oddOff = (W >> 1) + 8;
+  const int total = nRows * W4;
+  for (int base = 0; base < total; base += kLoadBatch * nt) {
+    float4 v[kLoadBatch];
+    int off[kLoadBatch];
+#pragma unroll
+    for (int u = 0; u < kLoadBatch; ++u) {
+      int i = base + u * nt + tid;
+      int r = i / W4, c4 = i - r * W4;
+      int gr = r0 + r;
+      off[u] = (i < total) ? r * pitch + 4 + (c4 << 1) : -1;
+      v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (i < total && gr >= 0 && gr < H) v[u] = reinterpret_cast<const float4 *>(plane + (long)gr * W)[c4];
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadBatch; ++u)
+      if (off[u] >= 0) {
+        *reinterpret_cast<float2 *>(dst + off[u]) = make_float2(v[u].x, v[u].z);
+        *reinterpret_cast<float2 *>(dst + off[u] + oddOff - 4) = make_float2(v[u].y, v[u].w);
+      }
+  }
+  // zero cells: [0,4) and [4 + W/2, 8 + W/2) of every row, [0,4) after the last row
+  const int totalPad = nRows * 8 + 4;
+  for (int i = tid; i < totalPad; i += nt) {
+    int r = i >> 3, k = i & 7;
+    dst[r * pitch + (k < 4 ? k : (W >> 1) + k)] = 0.f;
+  }
+}
+
+// Reads N consecutive floats starting at p into w[], using the widest LDS reads
+// the known alignment allows. OFF = element offset of p from an ALIGN-element
+// aligned address (ALIGN is 4, 2 or 1), both compile-time.
+template <int J, int N, int OFF, int ALIGN>
+__device__ __forceinline__ void readWindow(const float *__restrict__ p, float (&w)[N]) {
+  if constexpr (J < N) {
+    if constexpr (ALIGN >= 4 && ((OFF + J) % 4 == 0) && (J + 4 <= N)) {
+      float4 v = *reinterpret_cast<const float4 *>(p + J);
+      w[J] = v.x, w[J + 1] = v.y, w[J + 2] = v.z, w[J + 3] = v.w;
+      readWindow<J + 4, N, OFF, ALIGN>(p, w);
+    } else if constexpr (ALIGN >= 2 && ((OFF + J) % 2 == 0) && (J + 2 <= N)) {
+      float2 v = *reinterpret_cast<const float2 *>(p + J);
+      w[J] = v.x, w[J + 1] = v.y;
+      readWindow<J + 2, N, OFF, ALIGN>(p, w);
+    } else {
+      w[J] = p[J];
+      readWindow<J + 1, N, OFF, ALIGN>(p, w);
+    }
   }
 }
 

@@ -274,7 +274,7 @@ dwAccGradStage1(const float *__restrict__ in, const float *__restrict__ gradOut,
 // slots in a fixed order and accumulates scale * sum into the caller's tensors.
 __global__ void __launch_bounds__(dev::kBlock)
 dwAccGradStage2(const float *__restrict__ partial, float *__restrict__ gradWeight, Strides4 gs,
-                float *__restrict__ gradBias, Strides2 bs, int C, int M, int kW, int T, int nslots, float scale) {
+                float *__restrict__ gradBias, Strides2 bs, int M, int kW, int T, int nslots, float scale) {
   const int cj = blockIdx.x;
   const int c = cj / M, j = cj - c * M;
   const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
@@ -333,6 +333,271 @@ dwAccGradDirect(const float *__restrict__ in, const float *__restrict__ gradOut,
       gradWeight[j * gs.s0 + c * gs.s1 + kh * gs.s2 + kw * gs.s3] += scale * v;
     else
       gradBias[j * bs.s0 + c * bs.s1] += scale * v;
+  }
+}
+
+// ============================================================ strip kernels ==
+// Fast paths for the geometries depthwise layers actually use: square odd
+// kernel KS with "same" padding KS/2, stride ST in {1,2}, row lengths that are
+// multiples of 4. A lane produces 4 consecutive outputs (one 16-byte store);
+// the taps it needs form a (3*ST+KS)-wide window per input row which is read
+// from LDS with 16/8-byte loads at compile-time-known alignment, and every
+// index inside the window is a compile-time constant, so the inner loops are
+// straight-line FMAs on registers.
+
+// Offsets q = (d + PAD - k) / ST, over d in [0, ND) and taps k in [0, KS) with
+// (d + PAD - k) divisible by ST: the gradOutput rows/columns (relative to
+// h/ST resp. w/ST) that reach gradInput positions d.
+template <int KS, int ST, int ND>
+struct TapSpan {
+  static constexpr int lo() {
+    int m = 1 << 20;
+    for (int d = 0; d < ND; ++d)
+      for (int k = 0; k < KS; ++k) {
+        int t = d + KS / 2 - k;
+        if (t % ST == 0 && t / ST < m) m = t / ST;
+      }
+    return m;
+  }
+  static constexpr int hi() {
+    int m = -(1 << 20);
+    for (int d = 0; d < ND; ++d)
+      for (int k = 0; k < KS; ++k) {
+        int t = d + KS / 2 - k;
+        if (t % ST == 0 && t / ST > m) m = t / ST;
+      }
+    return m;
+  }
+};
+
+constexpr int kStripPadL = 4;  // left zero pad of staged rows (>= KS/2 for KS <= 9, keeps rows 16-byte aligned)
+
+// How the input band of a strip kernel is laid out in LDS and how a lane reads
+// the NW = 3*ST + KS consecutive input columns its 4 outputs need.
+//   ST == 1: plain rows, pitch W + 4, element (r, col) at r*pitch + 4 + col.
+//   ST == 2: rows split into even and odd columns (dev::loadRowsSplit), so the
+//            window becomes two unit-stride runs; the pitch is skewed to
+//            16 (mod 32) floats so that consecutive output rows (2 input rows
+//            apart) start 32 banks apart.
+template <int KS, int ST>
+struct Strip {
+  static constexpr int PAD = KS / 2, NW = 3 * ST + KS;
+  __host__ __device__ static int pitch(int W) {
+    return ST == 1 ? W + kStripPadL : (W + 8 - 16 + 31) / 32 * 32 + 16;
+  }
+  __host__ __device__ static size_t floats(int rows, int W) { return (size_t)rows * pitch(W) + kStripPadL; }
+  __device__ static void stage(float *dst, const float *plane, int H, int W, int r0, int nRows) {
+    if (ST == 1)
+      dev::loadRowsPadded<true>(dst, plane, H, W, r0, nRows, pitch(W), kStripPadL);
+    else
+      dev::loadRowsSplit(dst, plane, H, W, r0, nRows, pitch(W));
+  }
+  // window element j is input column 4*ST*b4 - PAD + j
+  static constexpr int half(int j) { return (j - PAD) % 2 == 0 ? (j - PAD) / 2 : (j - PAD - 1) / 2; }
+  static constexpr bool even(int j) { return (j - PAD) % 2 == 0; }
+  static constexpr int lo(bool e) {
+    int m = 1 << 20;
+    for (int j = 0; j < NW; ++j)
+      if (even(j) == e && half(j) < m) m = half(j);
+    return m;
+  }
+  static constexpr int hi(bool e) {
+    int m = -(1 << 20);
+    for (int j = 0; j < NW; ++j)
+      if (even(j) == e && half(j) > m) m = half(j);
+    return m;
+  }
+  __device__ static void loadWin(const float *__restrict__ row, int b4, int W, float (&win)[NW]) {
+    if constexpr (ST == 1) {
+      dev::readWindow<0, NW, (kStripPadL - PAD) & 3, 4>(row + (kStripPadL - PAD) + b4 * 4, win);
+    } else {
+      constexpr int ELO = lo(true), EHI = hi(true), OLO = lo(false), OHI = hi(false);
+      constexpr int NE = EHI - ELO + 1, NO = OHI - OLO + 1;
+      float ew[NE], ow[NO];
+      dev::readWindow<0, NE, ((ELO % 4) + 4) % 4, 4>(row + 4 + b4 * 4 + ELO, ew);
+      dev::readWindow<0, NO, ((OLO % 4) + 4) % 4, 4>(row + (W >> 1) + 8 + b4 * 4 + OLO, ow);
+#pragma unroll
+      for (int j = 0; j < NW; ++j) win[j] = even(j) ? ew[half(j) - ELO] : ow[half(j) - OLO];
+    }
+  }
+};
+
+template <int KS, int ST>
+__global__ void __launch_bounds__(dev::kBlock)
+dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strides4 ws,
+           const float *__restrict__ bias, Strides2 bs, float *__restrict__ out, DwGeom g) {
+  using S = Strip<KS, ST>;
+  constexpr int PAD = KS / 2, NW = S::NW;
+  extern __shared__ float smem[];
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  const int c = plane % g.C;
+  const int oh0 = tile * g.tileRows;
+  const int nOut = min(g.tileRows, g.oH - oh0);
+  const int nIn = (nOut - 1) * ST + KS;
+  const int pitch = S::pitch(g.W);
+  S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
+  __syncthreads();
+  const int oW4 = g.oW >> 2;
+  const int total = nOut * oW4;
+  for (int j = 0; j < g.M; ++j) {
+    float w[KS * KS];
+#pragma unroll
+    for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+      for (int kw = 0; kw < KS; ++kw) w[kh * KS + kw] = weight[j * ws.s0 + c * ws.s1 + kh * ws.s2 + kw * ws.s3];
+    const float b = bias ? bias[j * bs.s0 + c * bs.s1] : 0.f;
+    float *o = out + (((long)plane * g.M + j) * g.oH + oh0) * g.oW;
+    for (int i = threadIdx.x; i < total; i += blockDim.x) {
+      const int r = i / oW4, b4 = i - r * oW4;
+      const float *p = smem + r * ST * pitch;
+      float acc[4] = {b, b, b, b};
+#pragma unroll
+      for (int kh = 0; kh < KS; ++kh) {
+        float win[NW];
+        S::loadWin(p + kh * pitch, b4, g.W, win);
+#pragma unroll
+        for (int kw = 0; kw < KS; ++kw)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) acc[q] = fmaf(win[q * ST + kw], w[kh * KS + kw], acc[q]);
+      }
+      *reinterpret_cast<float4 *>(o + (long)r * g.oW + b4 * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    }
+  }
+}
+
+// gradInput: a lane produces an ST x 4 patch (rows ST*a .. ST*a+ST-1, columns
+// 4b .. 4b+3). The gradOutput rows are staged zero-padded, so no tap needs a
+// bounds test, and which (kh, kw) reaches which patch element is resolved at
+// compile time: only the K*K/(ST*ST) taps that really contribute are executed.
+template <int KS, int ST>
+__global__ void __launch_bounds__(dev::kBlock)
+dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ weight, Strides4 ws,
+                 float *__restrict__ gradIn, DwGeom g, int stageRows) {
+  constexpr int PAD = KS / 2;
+  constexpr int QH0 = TapSpan<KS, ST, ST>::lo(), QH1 = TapSpan<KS, ST, ST>::hi();
+  constexpr int QW0 = TapSpan<KS, ST, 4>::lo(), QW1 = TapSpan<KS, ST, 4>::hi();
+  constexpr int NW = QW1 - QW0 + 1;
+  constexpr int CPB = 4 / ST;  // gradOutput columns a patch advances per b
+  constexpr int OFF = ((kStripPadL + QW0) % 4 + 4) % 4;
+  constexpr int ALIGN = (CPB % 4 == 0) ? 4 : 2;
+  extern __shared__ float smem[];
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  const int c = plane % g.C;
+  const int h0 = tile * g.tileRows;  // multiple of ST
+  const int nRows = min(g.tileRows, g.H - h0);
+  const int pitch = g.oW + kStripPadL;
+  const long L = (long)g.oH * g.oW;
+  for (int j = 0; j < g.M; ++j)
+    dev::loadRowsPadded<true>(smem + (size_t)j * (stageRows * pitch + kStripPadL),
+                              gradOut + ((long)plane * g.M + j) * L, g.oH, g.oW, h0 / ST + QH0, stageRows, pitch,
+                              kStripPadL);
+  __syncthreads();
+  const int W4 = g.W >> 2;
+  const int nA = (nRows + ST - 1) / ST;
+  const int total = nA * W4;
+  float *o = gradIn + ((long)plane * g.H + h0) * g.W;
+  for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    const int a = i / W4, b = i - a * W4;
+    float acc[ST][4];
+#pragma unroll
+    for (int dy = 0; dy < ST; ++dy)
+#pragma unroll
+      for (int dx = 0; dx < 4; ++dx) acc[dy][dx] = 0.f;
+    for (int j = 0; j < g.M; ++j) {
+      float w[KS * KS];
+#pragma unroll
+      for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+        for (int kw = 0; kw < KS; ++kw) w[kh * KS + kw] = weight[j * ws.s0 + c * ws.s1 + kh * ws.s2 + kw * ws.s3];
+      const float *gj = smem + (size_t)j * (stageRows * pitch + kStripPadL) + kStripPadL + QW0 + b * CPB;
+#pragma unroll
+      for (int qh = QH0; qh <= QH1; ++qh) {
+        float win[NW];
+        dev::readWindow<0, NW, OFF, ALIGN>(gj + (a + qh - QH0) * pitch, win);
+#pragma unroll
+        for (int dy = 0; dy < ST; ++dy) {
+          const int kh = dy + PAD - qh * ST;
+          if (kh < 0 || kh >= KS) continue;
+#pragma unroll
+          for (int dx = 0; dx < 4; ++dx)
+#pragma unroll
+            for (int kw = 0; kw < KS; ++kw) {
+              const int t = dx + PAD - kw;
+              if (t % ST != 0) continue;
+              acc[dy][dx] = fmaf(win[t / ST - QW0], w[kh * KS + kw], acc[dy][dx]);
+            }
+        }
+      }
+    }
+#pragma unroll
+    for (int dy = 0; dy < ST; ++dy)
+      if (a * ST + dy < nRows)
+        *reinterpret_cast<float4 *>(o + (long)(a * ST + dy) * g.W + b * 4) =
+            make_float4(acc[dy][0], acc[dy][1], acc[dy][2], acc[dy][3]);
+  }
+}
+
+// accGradParameters stage 1 with the same 4-wide windows as the forward pass.
+template <int KS, int ST>
+__global__ void __launch_bounds__(dev::kBlock)
+dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, float *__restrict__ partial,
+               DwGeom g) {
+  using S = Strip<KS, ST>;
+  constexpr int PAD = KS / 2, NW = S::NW;
+  constexpr int T = KS * KS + 1;
+  constexpr int nWaves = dev::kBlock / dev::kWave;
+  extern __shared__ float smem[];
+  __shared__ float red[nWaves][T];
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  const int n = plane / g.C, c = plane - n * g.C;
+  const int oh0 = tile * g.tileRows;
+  const int nOut = min(g.tileRows, g.oH - oh0);
+  const int nIn = (nOut - 1) * ST + KS;
+  const int pitch = S::pitch(g.W);
+  float *gs = smem + S::floats((g.tileRows - 1) * ST + KS, g.W);  // multiple of 4 floats
+  S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
+  const int oW4 = g.oW >> 2;
+  const int total = nOut * oW4;
+  const int slot = n * g.tilesPerPlane + tile;
+  const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
+  for (int j = 0; j < g.M; ++j) {
+    if (j > 0) __syncthreads();
+    dev::loadFlat<true>(gs, gradOut + (((long)plane * g.M + j) * g.oH + oh0) * g.oW, nOut * g.oW);
+    __syncthreads();
+    float acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[t] = 0.f;
+    for (int i = threadIdx.x; i < total; i += blockDim.x) {
+      const int r = i / oW4, b4 = i - r * oW4;
+      const float *p = smem + r * ST * pitch;
+      const float4 gy4 = *reinterpret_cast<const float4 *>(gs + r * g.oW + b4 * 4);
+      const float gy[4] = {gy4.x, gy4.y, gy4.z, gy4.w};
+#pragma unroll
+      for (int kh = 0; kh < KS; ++kh) {
+        float win[NW];
+        S::loadWin(p + kh * pitch, b4, g.W, win);
+#pragma unroll
+        for (int kw = 0; kw < KS; ++kw)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) acc[kh * KS + kw] = fmaf(gy[q], win[q * ST + kw], acc[kh * KS + kw]);
+      }
+      acc[T - 1] += (gy[0] + gy[1]) + (gy[2] + gy[3]);
+    }
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      float v = dev::waveSum(acc[t]);
+      if (lane == 0) red[wave][t] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < T) {
+      float v = 0.f;
+#pragma unroll
+      for (int w = 0; w < nWaves; ++w) v += red[w][threadIdx.x];
+      partial[(((long)c * g.M + j) * T + threadIdx.x) * g.nslots + slot] = v;
+    }
   }
 }
 
@@ -470,9 +735,40 @@ void launchAcc1(hipStream_t s, size_t lds, bool vec, bool vecg, const float *in,
 
 // Environment switch used by the tests to exercise the shape-agnostic kernels on
 // shapes the tiled ones would otherwise take.
-bool forceDirect() {
+// 1: shape-agnostic direct kernels, 2: generic LDS-tiled kernels (no strip fast path).
+int forcedPath() {
   const char *e = getenv("THCUNN_DW_FORCE_DIRECT");
-  return e && e[0] == '1';
+  return e ? atoi(e) : 0;
+}
+bool forceDirect() { return forcedPath() == 1; }
+
+// Geometry the strip kernels are compiled for.
+bool stripGeometry(const DwGeom &g) {
+  bool sq = g.kH == g.kW && g.dH == g.dW && g.padH == g.padW;
+  return forcedPath() == 0 && sq && (g.kH == 3 || g.kH == 5) && (g.dH == 1 || g.dH == 2) && g.padH == g.kH / 2 &&
+         g.W % 4 == 0 && g.oW % 4 == 0;
+}
+
+#define DW_STRIP_DISPATCH(KERNEL, ...)                                           \
+  do {                                                                           \
+    if (g.kH == 3 && g.dH == 1) KERNEL<3, 1><<<grid, block, lds, s>>>(__VA_ARGS__); \
+    if (g.kH == 3 && g.dH == 2) KERNEL<3, 2><<<grid, block, lds, s>>>(__VA_ARGS__); \
+    if (g.kH == 5 && g.dH == 1) KERNEL<5, 1><<<grid, block, lds, s>>>(__VA_ARGS__); \
+    if (g.kH == 5 && g.dH == 2) KERNEL<5, 2><<<grid, block, lds, s>>>(__VA_ARGS__); \
+  } while (0)
+
+// LDS floats of a staged input band of `rows` rows in the strip layout
+size_t stripFloats(const DwGeom &g, int rows) {
+  if (g.dH == 1) return g.kH == 3 ? Strip<3, 1>::floats(rows, g.W) : Strip<5, 1>::floats(rows, g.W);
+  return g.kH == 3 ? Strip<3, 2>::floats(rows, g.W) : Strip<5, 2>::floats(rows, g.W);
+}
+
+// rows of gradOutput staged beyond the h/ST rows of a gradInput band
+int gradInputExtraRows(int ks, int st) {
+  if (ks == 3 && st == 1) return TapSpan<3, 1, 1>::hi() - TapSpan<3, 1, 1>::lo();
+  if (ks == 3 && st == 2) return TapSpan<3, 2, 2>::hi() - TapSpan<3, 2, 2>::lo();
+  if (ks == 5 && st == 1) return TapSpan<5, 1, 1>::hi() - TapSpan<5, 1, 1>::lo();
+  return TapSpan<5, 2, 2>::hi() - TapSpan<5, 2, 2>::lo();
 }
 
 }  // namespace
@@ -506,6 +802,17 @@ void THNN_CudaSpatialDepthWiseConvolution_updateOutput(THCState *state, THCudaTe
   auto bytes = [&](int rows) {
     return ((size_t)((rows - 1) * g.dH + g.kH) * g.pitch + g.padL + (size_t)g.M * g.kH * g.kW) * sizeof(float);
   };
+  if (stripGeometry(g) && vec && aligned16(data(output))) {
+    auto sbytes = [&](int rows) { return stripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
+    if (launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane)) {
+      g.nblk = (int)(planes * g.tilesPerPlane);
+      size_t lds = sbytes(g.tileRows);
+      dim3 grid(g.nblk), block(dev::kBlock);
+      DW_STRIP_DISPATCH(dwFwdStrip, in.ptr(), data(weight), strides4(weight), bptr, strides2(bias), data(output), g);
+      THC_HIP_CHECK(hipGetLastError());
+      return;
+    }
+  }
   if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
     size_t lds = bytes(g.tileRows);
@@ -550,6 +857,21 @@ void THNN_CudaSpatialDepthWiseConvolution_updateGradInput(THCState *state, THCud
   auto bytes = [&](int rows) {
     return ((size_t)g.M * ohRows(rows) * g.oW + (size_t)g.M * g.kH * g.kW) * sizeof(float);
   };
+  if (stripGeometry(g) && vec && aligned16(data(gradInput))) {
+    const int extra = gradInputExtraRows(g.kH, g.dH);
+    const int pitch = g.oW + kStripPadL;
+    auto sbytes = [&](int units) { return (size_t)g.M * ((size_t)(units + extra) * pitch + kStripPadL) * sizeof(float); };
+    int units = 0;
+    if (launch::pickBand(ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
+      g.tileRows = units * g.dH;
+      g.nblk = (int)(planes * g.tilesPerPlane);
+      size_t lds = sbytes(units);
+      dim3 grid(g.nblk), block(dev::kBlock);
+      DW_STRIP_DISPATCH(dwGradInputStrip, go.ptr(), data(weight), strides4(weight), data(gradInput), g, units + extra);
+      THC_HIP_CHECK(hipGetLastError());
+      return;
+    }
+  }
   if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
     int maxOh = ohRows(g.tileRows);
@@ -589,11 +911,14 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
   int ks = sq ? g.kH : 0, st = sq ? g.dH : 0;
   bool haveKernel = (ks == 3 || ks == 5) && (st == 1 || st == 2);
   bool vec = (g.W % 4 == 0) && aligned16(in.ptr());
+  const bool useStrip = stripGeometry(g) && vec && aligned16(go.ptr());
   g.padL = vec ? roundUp(g.padW, 4) : g.padW;
   g.pitch = g.W + g.padL;
   // staged input band (rounded up so the gradOutput band behind it stays 16-byte aligned) + gradOutput band
   auto bytes = [&](int rows) {
-    return ((size_t)roundUp(((rows - 1) * g.dH + g.kH) * g.pitch + g.padL, 4) + (size_t)rows * g.oW) * sizeof(float);
+    size_t band = useStrip ? stripFloats(g, (rows - 1) * g.dH + g.kH)
+                           : (size_t)roundUp(((rows - 1) * g.dH + g.kH) * g.pitch + g.padL, 4);
+    return (band + (size_t)rows * g.oW) * sizeof(float);
   };
   if (haveKernel && !forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
@@ -616,13 +941,18 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
     }
     // a band of gradOutput rows starts at ((plane*M+j)*oH + oh0) * oW
     bool vecg = aligned16(go.ptr()) && (g.oW % 4 == 0 || (g.tilesPerPlane == 1 && ((long)g.oH * g.oW) % 4 == 0));
-    if (ks == 3 && st == 1) launchAcc1<3, 1>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
-    if (ks == 3 && st == 2) launchAcc1<3, 2>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
-    if (ks == 5 && st == 1) launchAcc1<5, 1>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
-    if (ks == 5 && st == 2) launchAcc1<5, 2>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
+    if (useStrip) {
+      dim3 grid(g.nblk), block(dev::kBlock);
+      DW_STRIP_DISPATCH(dwAccGradStrip, in.ptr(), go.ptr(), partial, g);
+    } else {
+      if (ks == 3 && st == 1) launchAcc1<3, 1>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
+      if (ks == 3 && st == 2) launchAcc1<3, 2>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
+      if (ks == 5 && st == 1) launchAcc1<5, 1>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
+      if (ks == 5 && st == 2) launchAcc1<5, 2>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
+    }
     THC_HIP_CHECK(hipGetLastError());
     dwAccGradStage2<<<g.C * g.M, dev::kBlock, 0, s>>>(partial, data(gradWeight), strides4(gradWeight), gbPtr,
-                                                      strides2(gradBias), g.C, g.M, g.kW, T, g.nslots, scale);
+                                                      strides2(gradBias), g.M, g.kW, T, g.nslots, scale);
   } else {
     int T = g.kH * g.kW + 1;
     dwAccGradDirect<<<g.C * g.M * T, dev::kBlock, 0, s>>>(in.ptr(), go.ptr(), data(gradWeight),

@@ -32,13 +32,14 @@ def close(a, b, rtol=OUT_RTOL, atol=OUT_ATOL):
 
 
 class force_direct:
-    """Routes a call to the shape-agnostic kernels instead of the LDS-tiled ones."""
+    """Routes a call to the shape-agnostic kernels ("1") or, for the depthwise
+    convolution, to the generic LDS-tiled kernels ("2") instead of the fastest path."""
 
-    def __init__(self, var):
-        self.var = var
+    def __init__(self, var, mode="1"):
+        self.var, self.mode = var, mode
 
     def __enter__(self):
-        os.environ[self.var] = "1"
+        os.environ[self.var] = self.mode
 
     def __exit__(self, *a):
         os.environ.pop(self.var, None)
@@ -57,6 +58,10 @@ DW_CASES = [
     (1, 6, 1, 7, 7, 3, 3, 1, 1, 1, 1),       # tiny planes
     (2, 2, 1, 150, 260, 3, 3, 1, 1, 1, 1),   # several row bands per plane
     (1, 2, 1, 12, 12, 7, 7, 2, 2, 3, 3),
+    (2, 3, 2, 24, 32, 5, 5, 1, 1, 2, 2),     # 5x5 strip kernels
+    (2, 3, 1, 40, 48, 5, 5, 2, 2, 2, 2),
+    (2, 3, 2, 57, 56, 3, 3, 2, 2, 1, 1),     # odd height under stride 2
+    (1, 2, 1, 8, 8, 3, 3, 2, 2, 1, 1),
 ]
 
 
@@ -105,10 +110,11 @@ def test_dwconv_tiled(T, case):
     _dw_run(T, case, x, w, b)
 
 
-@pytest.mark.parametrize("case", DW_CASES[:7])
-def test_dwconv_direct_kernels(T, case):
+@pytest.mark.parametrize("case", DW_CASES[:7] + DW_CASES[10:12])
+@pytest.mark.parametrize("mode", ["1", "2"])
+def test_dwconv_fallback_kernels(T, case, mode):
     _, x, w, b = _dw_inputs(case, 2)
-    with force_direct("THCUNN_DW_FORCE_DIRECT"):
+    with force_direct("THCUNN_DW_FORCE_DIRECT", mode):
         _dw_run(T, case, x, w, b)
 
 

@@ -309,6 +309,267 @@ bnBackwardKernel(const float *__restrict__ x, const float *__restrict__ gy, floa
   }
 }
 
+// ============================================================ resident path ==
+// When a channel's N*L elements fit the register file of one CU, a single
+// 1024-lane workgroup per channel loads them once (R 16-byte loads in flight
+// per lane), derives the statistics from registers with the reference's exact
+// two-pass formulas (mean first, then sum (x - mean)^2,
+// lib/THCUNN/BatchNormalization.cu:181-191) and writes the result: every byte
+// crosses HBM exactly once. Needs C of the order of the CU count to fill the chip.
+constexpr int kResBlock = 1024;
+constexpr int kResWaves = kResBlock / dev::kWave;
+
+// Buffer-addressed 16-byte accesses: the channel base lives in a scalar
+// resource descriptor and each access carries only a 32-bit byte offset, so
+// the unrolled R-deep load/store sequences do not tie up a 64-bit address
+// register pair per access.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t makeRsrc(const float *base, long bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ float4 bufLoad4(__amdgpu_buffer_rsrc_t r, int byteOff) {
+  u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byteOff, 0, 0);
+  return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+}
+__device__ __forceinline__ void bufStore4(__amdgpu_buffer_rsrc_t r, int byteOff, float4 f) {
+  u32x4 v = {__float_as_uint(f.x), __float_as_uint(f.y), __float_as_uint(f.z), __float_as_uint(f.w)};
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, byteOff, 0, 0);
+}
+
+__device__ __forceinline__ float blockSum1024(float v, float *red) {
+  const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
+  v = dev::waveSum(v);
+  __syncthreads();  // red may still be read from a previous reduction
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float s = 0.f;
+#pragma unroll
+  for (int w = 0; w < kResWaves; ++w) s += red[w];
+  return s;
+}
+
+// Walks the float4s tid, tid + 1024, tid + 2048, ... of channel ch (numbered
+// n-major over the channel's N planes of L/4 float4s) without a division per
+// step. Offsets are 32-bit byte offsets from the channel's first plane (the
+// host checks that the tensor is smaller than 2 GiB).
+struct ResWalker {
+  int off, l4, stepOff, stepL, L4, wrapOff;
+  __device__ ResWalker(int L, int C) : L4(L >> 2) {
+    const int n = threadIdx.x / L4;
+    l4 = threadIdx.x - n * L4;
+    const int stepN = kResBlock / L4;
+    stepL = kResBlock - stepN * L4;
+    off = (n * C * L + (l4 << 2)) * 4;
+    stepOff = (stepN * C * L + (stepL << 2)) * 4;
+    wrapOff = (C * L - L) * 4;
+  }
+  __device__ int offset() const { return off; }
+  __device__ void next() {
+    off += stepOff;
+    l4 += stepL;
+    if (l4 >= L4) {
+      l4 -= L4;
+      off += wrapOff;
+    }
+  }
+};
+
+template <int R>
+__global__ void __launch_bounds__(kResBlock)
+bnFwdResident(const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ weight,
+              const float *__restrict__ bias, float *__restrict__ runningMean, float *__restrict__ runningVar,
+              float *__restrict__ saveMean, float *__restrict__ saveStd, int N, int C, int L, float momentum,
+              float eps) {
+  __shared__ float red[kResWaves];
+  const int ch = blockIdx.x;
+  const int total4 = N * (L >> 2);
+  const long span = ((long)(N - 1) * C * L + L) * 4;  // bytes from the channel's first to past its last element
+  const __amdgpu_buffer_rsrc_t xr = makeRsrc(x + (long)ch * L, span), yr = makeRsrc(y + (long)ch * L, span);
+  float4 v[R];
+  {
+    ResWalker wk(L, C);
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (u * kResBlock + (int)threadIdx.x < total4) v[u] = bufLoad4(xr, wk.offset());
+      wk.next();
+    }
+  }
+  const float cnt = (float)N * (float)L, norm = 1.f / cnt;
+  float s = 0.f;
+#pragma unroll
+  for (int u = 0; u < R; ++u) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+  const float mean = blockSum1024(s, red) * norm;
+  float q = 0.f;
+#pragma unroll
+  for (int u = 0; u < R; ++u)
+    if (u * kResBlock + (int)threadIdx.x < total4) {
+      float a = v[u].x - mean, b = v[u].y - mean, c = v[u].z - mean, d = v[u].w - mean;
+      q += (a * a + b * b) + (c * c + d * d);
+    }
+  const float varN = blockSum1024(q, red);
+  float invStd = 0.f;
+  if (varN != 0.f || eps != 0.f) invStd = 1.f / sqrtf(varN * norm + eps);
+  if (threadIdx.x == 0) {
+    float unbiased = varN / (cnt - 1.f);
+    saveMean[ch] = mean;
+    saveStd[ch] = invStd;
+    runningMean[ch] = (1.f - momentum) * runningMean[ch] + momentum * mean;
+    runningVar[ch] = (1.f - momentum) * runningVar[ch] + momentum * unbiased;
+  }
+  const float gamma = weight ? weight[ch] : 1.f, beta = bias ? bias[ch] : 0.f;
+  ResWalker wk(L, C);
+#pragma unroll
+  for (int u = 0; u < R; ++u) {
+    if (u * kResBlock + (int)threadIdx.x < total4) {
+      float4 r;
+      r.x = gamma * (v[u].x - mean) * invStd + beta;
+      r.y = gamma * (v[u].y - mean) * invStd + beta;
+      r.z = gamma * (v[u].z - mean) * invStd + beta;
+      r.w = gamma * (v[u].w - mean) * invStd + beta;
+      bufStore4(yr, wk.offset(), r);
+    }
+    wk.next();
+  }
+}
+
+// Backward with gradOutput resident in registers. KEEPX: (x - mean) stays in
+// registers as well (2R float4 per lane); otherwise x is read a second time in
+// the apply phase - it was streamed by this CU a moment ago, so the re-read is
+// served by the L2 / Infinity Cache rather than HBM.
+template <int R, bool TRAIN, bool KEEPX>
+__global__ void __launch_bounds__(kResBlock)
+bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
+              float *__restrict__ gradWeight, float *__restrict__ gradBias, const float *__restrict__ weight,
+              const float *__restrict__ meanSrc, const float *__restrict__ stdSrc, int N, int C, int L, float scale,
+              float eps) {
+  __shared__ float red[kResWaves];
+  const int ch = blockIdx.x;
+  const int total4 = N * (L >> 2);
+  const float mean = meanSrc[ch];
+  const float stdVal = TRAIN ? stdSrc[ch] : 1.f / sqrtf(stdSrc[ch] + eps);
+  const float weightVal = weight ? weight[ch] : 1.f;
+  const long span = ((long)(N - 1) * C * L + L) * 4;
+  const __amdgpu_buffer_rsrc_t xr = makeRsrc(x + (long)ch * L, span), gr = makeRsrc(gy + (long)ch * L, span);
+  const __amdgpu_buffer_rsrc_t or_ = makeRsrc(gx ? gx + (long)ch * L : x, gx ? span : 0);
+  float4 d[R], xc[KEEPX ? R : 1];
+  float s0 = 0.f, s1 = 0.f;
+  {
+    ResWalker wk(L, C);
+    if (KEEPX) {
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        d[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        xc[KEEPX ? u : 0] = make_float4(mean, mean, mean, mean);
+        if (u * kResBlock + (int)threadIdx.x < total4) {
+          const int off = wk.offset();
+          d[u] = bufLoad4(gr, off);
+          xc[KEEPX ? u : 0] = bufLoad4(xr, off);
+        }
+        wk.next();
+      }
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        float4 &q = xc[KEEPX ? u : 0];
+        q.x -= mean, q.y -= mean, q.z -= mean, q.w -= mean;
+        s0 += (d[u].x + d[u].y) + (d[u].z + d[u].w);
+        s1 += (d[u].x * q.x + d[u].y * q.y) + (d[u].z * q.z + d[u].w * q.w);
+      }
+    } else {
+      // gy for the whole channel first (kept), x in batches of 4 (consumed)
+      ResWalker wx = wk;
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        d[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (u * kResBlock + (int)threadIdx.x < total4) d[u] = bufLoad4(gr, wk.offset());
+        wk.next();
+      }
+#pragma unroll
+      for (int u0 = 0; u0 < R; u0 += 4) {
+        float4 q[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          q[k] = make_float4(mean, mean, mean, mean);
+          if (u0 + k < R) {
+            if ((u0 + k) * kResBlock + (int)threadIdx.x < total4) q[k] = bufLoad4(xr, wx.offset());
+            wx.next();
+          }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (u0 + k < R) {
+            const float4 &g4 = d[u0 + k];
+            s0 += (g4.x + g4.y) + (g4.z + g4.w);
+            s1 += (g4.x * (q[k].x - mean) + g4.y * (q[k].y - mean)) + (g4.z * (q[k].z - mean) + g4.w * (q[k].w - mean));
+          }
+        __asm__ volatile("" ::: "memory");  // keep the batches apart: 4 loads in flight, not R
+      }
+    }
+  }
+  const float gradOutputSum = blockSum1024(s0, red);
+  const float dotP = blockSum1024(s1, red);
+  const float norm = 1.f / ((float)N * (float)L);
+  const float gradMean = gradOutputSum * norm;
+  const float projScale = dotP * norm * stdVal * stdVal;
+  const float gradScale = stdVal * weightVal;
+  if (gx) {
+    ResWalker wk(L, C);
+    if (KEEPX || !TRAIN) {
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        if (u * kResBlock + (int)threadIdx.x < total4) {
+          float4 r;
+          const float4 q = xc[KEEPX ? u : 0];
+          if (TRAIN) {
+            r.x = (d[u].x - q.x * projScale - gradMean) * gradScale;
+            r.y = (d[u].y - q.y * projScale - gradMean) * gradScale;
+            r.z = (d[u].z - q.z * projScale - gradMean) * gradScale;
+            r.w = (d[u].w - q.w * projScale - gradMean) * gradScale;
+          } else {
+            r.x = d[u].x * gradScale, r.y = d[u].y * gradScale, r.z = d[u].z * gradScale, r.w = d[u].w * gradScale;
+          }
+          bufStore4(or_, wk.offset(), r);
+        }
+        wk.next();
+      }
+    } else {
+#pragma unroll
+      for (int u0 = 0; u0 < R; u0 += 4) {
+        float4 q[4];
+        int off[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          off[k] = -1;
+          q[k] = make_float4(mean, mean, mean, mean);
+          if (u0 + k < R) {
+            if ((u0 + k) * kResBlock + (int)threadIdx.x < total4) {
+              off[k] = wk.offset();
+              q[k] = bufLoad4(xr, off[k]);
+            }
+            wk.next();
+          }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (u0 + k < R && off[k] >= 0) {
+            const float4 &g4 = d[u0 + k];
+            float4 r;
+            r.x = (g4.x - (q[k].x - mean) * projScale - gradMean) * gradScale;
+            r.y = (g4.y - (q[k].y - mean) * projScale - gradMean) * gradScale;
+            r.z = (g4.z - (q[k].z - mean) * projScale - gradMean) * gradScale;
+            r.w = (g4.w - (q[k].w - mean) * projScale - gradMean) * gradScale;
+            bufStore4(or_, off[k], r);
+          }
+        __asm__ volatile("" ::: "memory");
+      }
+    }
+  }
+  if (threadIdx.x == 0) {
+    if (gradWeight) gradWeight[ch] += scale * dotP * stdVal;
+    if (gradBias) gradBias[ch] += scale * gradOutputSum;
+  }
+}
+
 // -------------------------------------------------------------- host side ----
 struct BnView {
   BnGeom g;
@@ -361,6 +622,21 @@ void checkVector(const THCudaTensor *t, const char *name, int C, bool required) 
 
 inline float *dataOrNull(const THCudaTensor *t) { return t ? data(t) : nullptr; }
 
+// The resident kernels hold a channel in the registers of one 1024-lane
+// workgroup: at most maxR float4 per lane, and enough channels to occupy the chip.
+int residentR(const BnView &v, int maxR) {
+  const char *e = getenv("THCUNN_BN_FORCE_CHUNKED");
+  if (e && e[0] == '1') return 0;
+  const BnGeom &g = v.g;
+  if (!v.vec || g.C < 96 || g.L / 4 > kResBlock || (long)g.N * g.C * g.L * 4 >= 0x7fffffffL) return 0;
+  long total4 = (long)g.N * (g.L / 4);
+  int need = (int)((total4 + kResBlock - 1) / kResBlock);
+  const int sizes[] = {2, 4, 8, 12, 13, 14};
+  for (int r : sizes)
+    if (need <= r && r <= maxR) return r;
+  return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -390,6 +666,17 @@ void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *inp
   if ((long)g.C * g.chunks >= 0x7fffffffL) error("BatchNormalization: grid too large");
   hipStream_t s = state->stream;
   dim3 grid((unsigned)(g.C * g.chunks)), block(dev::kBlock);
+  if (int R = train ? residentR(v, 14) : 0) {
+#define BN_FWD_RES(RR)                                                                                              \
+  if (R == RR)                                                                                                      \
+    bnFwdResident<RR><<<g.C, kResBlock, 0, s>>>(in.ptr(), data(output_), dataOrNull(weight_), dataOrNull(bias_),    \
+                                                data(runningMean_), data(runningVar_), data(saveMean_),             \
+                                                data(saveStd_), g.N, g.C, g.L, (float)momentum, (float)eps);
+    BN_FWD_RES(2) BN_FWD_RES(4) BN_FWD_RES(8) BN_FWD_RES(12) BN_FWD_RES(13) BN_FWD_RES(14)
+#undef BN_FWD_RES
+    THC_HIP_CHECK(hipGetLastError());
+    return;
+  }
   if (train) {
     Temp partial(s, (size_t)g.C * g.chunks * 3 * sizeof(float));
     float *p = (float *)partial.get();
@@ -462,6 +749,24 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
   const float *meanSrc = train ? data(saveMean_) : data(runningMean_);
   const float *stdSrc = train ? data(saveStd_) : data(runningVar_);
   const bool needSums = (train && gradInput_) || gradWeight_ || gradBias_;
+  if (int R = needSums ? residentR(v, 13) : 0) {
+    float *gxp = gradInput_ ? data(gradInput_) : nullptr;
+#define BN_BWD_RES(RR)                                                                                             \
+  if (R == RR) {                                                                                                   \
+    if (train)                                                                                                     \
+      bnBwdResident<RR, true, (RR <= 8)><<<g.C, kResBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),          \
+                                                        dataOrNull(gradBias_), dataOrNull(weight_), meanSrc,       \
+                                                        stdSrc, g.N, g.C, g.L, (float)scale, (float)eps);          \
+    else                                                                                                           \
+      bnBwdResident<RR, false, (RR <= 8)><<<g.C, kResBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),         \
+                                                         dataOrNull(gradBias_), dataOrNull(weight_), meanSrc,      \
+                                                         stdSrc, g.N, g.C, g.L, (float)scale, (float)eps);         \
+  }
+    BN_BWD_RES(2) BN_BWD_RES(4) BN_BWD_RES(8) BN_BWD_RES(12) BN_BWD_RES(13)
+#undef BN_BWD_RES
+    THC_HIP_CHECK(hipGetLastError());
+    return;
+  }
   Temp partial;
   float *p = nullptr;
   if (needSums) {

@@ -56,15 +56,17 @@ constexpr int kLoadBatch = 4;
 
 // Copies rows [r0, r0 + nRows) of a (H x W) plane into LDS at
 //   dst[r * pitch + padL + col],  r = 0 .. nRows-1, col = 0 .. W-1
-// Rows outside the plane are zero-filled and so are the padL cells in front of
-// every row plus padL cells after the last one, so that a reader may run up to
-// padL columns off either side of a row and see zeros (the right overhang of
-// row r is the left pad of row r+1). VEC: W % 4 == 0, pitch % 4 == 0,
+// Rows outside the plane are filled with `fill` (0 for sums, -FLT_MAX for max
+// scans) and so are the padL cells in front of every row plus padL cells after
+// the last one, so that a reader may run up to padL columns off either side of
+// a row and see the fill value (the right overhang of row r is the left pad of
+// row r+1). VEC: W % 4 == 0, pitch % 4 == 0,
 // padL % 4 == 0 and a 16-byte aligned plane, which makes every transfer a
 // 16-byte global load and a 16-byte LDS store.
 template <bool VEC>
 __device__ __forceinline__ void loadRowsPadded(float *__restrict__ dst, const float *__restrict__ plane,
-                                               int H, int W, int r0, int nRows, int pitch, int padL) {
+                                               int H, int W, int r0, int nRows, int pitch, int padL,
+                                               float fill = 0.f) {
   const int tid = threadIdx.x, nt = blockDim.x;
   if (VEC) {
     const int W4 = W >> 2;
@@ -78,7 +80,7 @@ __device__ __forceinline__ void loadRowsPadded(float *__restrict__ dst, const fl
         int r = i / W4, c4 = i - r * W4;
         int gr = r0 + r;
         off[u] = (i < total) ? r * pitch + padL + (c4 << 2) : -1;
-        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        v[u] = make_float4(fill, fill, fill, fill);
         if (i < total && gr >= 0 && gr < H) v[u] = reinterpret_cast<const float4 *>(plane + (long)gr * W)[c4];
       }
 #pragma unroll
@@ -96,7 +98,7 @@ __device__ __forceinline__ void loadRowsPadded(float *__restrict__ dst, const fl
         int r = i / W, c = i - r * W;
         int gr = r0 + r;
         off[u] = (i < total) ? r * pitch + padL + c : -1;
-        v[u] = (i < total && gr >= 0 && gr < H) ? plane[(long)gr * W + c] : 0.f;
+        v[u] = (i < total && gr >= 0 && gr < H) ? plane[(long)gr * W + c] : fill;
       }
 #pragma unroll
       for (int u = 0; u < kLoadBatch; ++u)
@@ -107,7 +109,7 @@ __device__ __forceinline__ void loadRowsPadded(float *__restrict__ dst, const fl
     const int totalPad = (nRows + 1) * padL;
     for (int i = tid; i < totalPad; i += nt) {
       int r = i / padL, k = i - r * padL;
-      dst[r * pitch + k] = 0.f;
+      dst[r * pitch + k] = fill;
     }
   }
 }
@@ -154,12 +156,12 @@ __device__ __forceinline__ void loadFlat(T *__restrict__ dst, const T *__restric
 // De-interleaving variant for stride-2 consumers: row r of the band is stored as
 //   dst[r * pitch + 4 + m]           = x[r][2m]      (even columns)
 //   dst[r * pitch + oddOff + m]      = x[r][2m + 1]  (odd columns), oddOff = W/2 + 8
-// with 4 zero cells in front of each half and 4 after the last row, so that a
+// with 4 fill cells in front of each half and 4 after the last row, so that a
 // lane reading 4 consecutive even (or odd) columns issues one 16-byte LDS read at
 // unit stride across lanes instead of a 32-byte-strided one (which maps 64 lanes
 // onto 8 banks). Requires W % 8 == 0, pitch % 4 == 0, 16-byte aligned plane.
 __device__ __forceinline__ void loadRowsSplit(float *__restrict__ dst, const float *__restrict__ plane, int H, int W,
-                                              int r0, int nRows, int pitch) {
+                                              int r0, int nRows, int pitch, float fill = 0.f) {
   const int tid = threadIdx.x, nt = blockDim.x;
   const int W4 = W >> 2;
   const int oddOff = (W >> 1) + 8;
@@ -173,7 +175,7 @@ __device__ __forceinline__ void loadRowsSplit(float *__restrict__ dst, const flo
       int r = i / W4, c4 = i - r * W4;
       int gr = r0 + r;
       off[u] = (i < total) ? r * pitch + 4 + (c4 << 1) : -1;
-      v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      v[u] = make_float4(fill, fill, fill, fill);
       if (i < total && gr >= 0 && gr < H) v[u] = reinterpret_cast<const float4 *>(plane + (long)gr * W)[c4];
     }
 #pragma unroll
@@ -187,7 +189,7 @@ __device__ __forceinline__ void loadRowsSplit(float *__restrict__ dst, const flo
   const int totalPad = nRows * 8 + 4;
   for (int i = tid; i < totalPad; i += nt) {
     int r = i >> 3, k = i & 7;
-    dst[r * pitch + (k < 4 ? k : (W >> 1) + k)] = 0.f;
+    dst[r * pitch + (k < 4 ? k : (W >> 1) + k)] = fill;
   }
 }
 

@@ -13,6 +13,7 @@
 // fixed order (deterministic) and accumulates into gradWeight/gradBias.
 #include "device_utils.h"
 #include "launch_utils.h"
+#include "strip.h"
 #include "thc_internal.h"
 
 using namespace thc;
@@ -345,88 +346,11 @@ dwAccGradDirect(const float *__restrict__ in, const float *__restrict__ gradOut,
 // index inside the window is a compile-time constant, so the inner loops are
 // straight-line FMAs on registers.
 
-// Offsets q = (d + PAD - k) / ST, over d in [0, ND) and taps k in [0, KS) with
-// (d + PAD - k) divisible by ST: the gradOutput rows/columns (relative to
-// h/ST resp. w/ST) that reach gradInput positions d.
-template <int KS, int ST, int ND>
-struct TapSpan {
-  static constexpr int lo() {
-    int m = 1 << 20;
-    for (int d = 0; d < ND; ++d)
-      for (int k = 0; k < KS; ++k) {
-        int t = d + KS / 2 - k;
-        if (t % ST == 0 && t / ST < m) m = t / ST;
-      }
-    return m;
-  }
-  static constexpr int hi() {
-    int m = -(1 << 20);
-    for (int d = 0; d < ND; ++d)
-      for (int k = 0; k < KS; ++k) {
-        int t = d + KS / 2 - k;
-        if (t % ST == 0 && t / ST > m) m = t / ST;
-      }
-    return m;
-  }
-};
-
-constexpr int kStripPadL = 4;  // left zero pad of staged rows (>= KS/2 for KS <= 9, keeps rows 16-byte aligned)
-
-// How the input band of a strip kernel is laid out in LDS and how a lane reads
-// the NW = 3*ST + KS consecutive input columns its 4 outputs need.
-//   ST == 1: plain rows, pitch W + 4, element (r, col) at r*pitch + 4 + col.
-//   ST == 2: rows split into even and odd columns (dev::loadRowsSplit), so the
-//            window becomes two unit-stride runs; the pitch is skewed to
-//            16 (mod 32) floats so that consecutive output rows (2 input rows
-//            apart) start 32 banks apart.
-template <int KS, int ST>
-struct Strip {
-  static constexpr int PAD = KS / 2, NW = 3 * ST + KS;
-  __host__ __device__ static int pitch(int W) {
-    return ST == 1 ? W + kStripPadL : (W + 8 - 16 + 31) / 32 * 32 + 16;
-  }
-  __host__ __device__ static size_t floats(int rows, int W) { return (size_t)rows * pitch(W) + kStripPadL; }
-  __device__ static void stage(float *dst, const float *plane, int H, int W, int r0, int nRows) {
-    if (ST == 1)
-      dev::loadRowsPadded<true>(dst, plane, H, W, r0, nRows, pitch(W), kStripPadL);
-    else
-      dev::loadRowsSplit(dst, plane, H, W, r0, nRows, pitch(W));
-  }
-  // window element j is input column 4*ST*b4 - PAD + j
-  static constexpr int half(int j) { return (j - PAD) % 2 == 0 ? (j - PAD) / 2 : (j - PAD - 1) / 2; }
-  static constexpr bool even(int j) { return (j - PAD) % 2 == 0; }
-  static constexpr int lo(bool e) {
-    int m = 1 << 20;
-    for (int j = 0; j < NW; ++j)
-      if (even(j) == e && half(j) < m) m = half(j);
-    return m;
-  }
-  static constexpr int hi(bool e) {
-    int m = -(1 << 20);
-    for (int j = 0; j < NW; ++j)
-      if (even(j) == e && half(j) > m) m = half(j);
-    return m;
-  }
-  __device__ static void loadWin(const float *__restrict__ row, int b4, int W, float (&win)[NW]) {
-    if constexpr (ST == 1) {
-      dev::readWindow<0, NW, (kStripPadL - PAD) & 3, 4>(row + (kStripPadL - PAD) + b4 * 4, win);
-    } else {
-      constexpr int ELO = lo(true), EHI = hi(true), OLO = lo(false), OHI = hi(false);
-      constexpr int NE = EHI - ELO + 1, NO = OHI - OLO + 1;
-      float ew[NE], ow[NO];
-      dev::readWindow<0, NE, ((ELO % 4) + 4) % 4, 4>(row + 4 + b4 * 4 + ELO, ew);
-      dev::readWindow<0, NO, ((OLO % 4) + 4) % 4, 4>(row + (W >> 1) + 8 + b4 * 4 + OLO, ow);
-#pragma unroll
-      for (int j = 0; j < NW; ++j) win[j] = even(j) ? ew[half(j) - ELO] : ow[half(j) - OLO];
-    }
-  }
-};
-
 template <int KS, int ST>
 __global__ void __launch_bounds__(dev::kBlock)
 dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strides4 ws,
            const float *__restrict__ bias, Strides2 bs, float *__restrict__ out, DwGeom g) {
-  using S = Strip<KS, ST>;
+  using S = dev::Strip<KS, ST, KS / 2>;
   constexpr int PAD = KS / 2, NW = S::NW;
   extern __shared__ float smem[];
   const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
@@ -475,11 +399,11 @@ __global__ void __launch_bounds__(dev::kBlock)
 dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ weight, Strides4 ws,
                  float *__restrict__ gradIn, DwGeom g, int stageRows) {
   constexpr int PAD = KS / 2;
-  constexpr int QH0 = TapSpan<KS, ST, ST>::lo(), QH1 = TapSpan<KS, ST, ST>::hi();
-  constexpr int QW0 = TapSpan<KS, ST, 4>::lo(), QW1 = TapSpan<KS, ST, 4>::hi();
+  constexpr int QH0 = dev::TapSpan<KS, ST, ST, KS / 2>::lo(), QH1 = dev::TapSpan<KS, ST, ST, KS / 2>::hi();
+  constexpr int QW0 = dev::TapSpan<KS, ST, 4, KS / 2>::lo(), QW1 = dev::TapSpan<KS, ST, 4, KS / 2>::hi();
   constexpr int NW = QW1 - QW0 + 1;
   constexpr int CPB = 4 / ST;  // gradOutput columns a patch advances per b
-  constexpr int OFF = ((kStripPadL + QW0) % 4 + 4) % 4;
+  constexpr int OFF = ((dev::kStripPadL + QW0) % 4 + 4) % 4;
   constexpr int ALIGN = (CPB % 4 == 0) ? 4 : 2;
   extern __shared__ float smem[];
   const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
@@ -487,12 +411,12 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
   const int c = plane % g.C;
   const int h0 = tile * g.tileRows;  // multiple of ST
   const int nRows = min(g.tileRows, g.H - h0);
-  const int pitch = g.oW + kStripPadL;
+  const int pitch = g.oW + dev::kStripPadL;
   const long L = (long)g.oH * g.oW;
   for (int j = 0; j < g.M; ++j)
-    dev::loadRowsPadded<true>(smem + (size_t)j * (stageRows * pitch + kStripPadL),
+    dev::loadRowsPadded<true>(smem + (size_t)j * (stageRows * pitch + dev::kStripPadL),
                               gradOut + ((long)plane * g.M + j) * L, g.oH, g.oW, h0 / ST + QH0, stageRows, pitch,
-                              kStripPadL);
+                              dev::kStripPadL);
   __syncthreads();
   const int W4 = g.W >> 2;
   const int nA = (nRows + ST - 1) / ST;
@@ -511,7 +435,7 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
       for (int kh = 0; kh < KS; ++kh)
 #pragma unroll
         for (int kw = 0; kw < KS; ++kw) w[kh * KS + kw] = weight[j * ws.s0 + c * ws.s1 + kh * ws.s2 + kw * ws.s3];
-      const float *gj = smem + (size_t)j * (stageRows * pitch + kStripPadL) + kStripPadL + QW0 + b * CPB;
+      const float *gj = smem + (size_t)j * (stageRows * pitch + dev::kStripPadL) + dev::kStripPadL + QW0 + b * CPB;
 #pragma unroll
       for (int qh = QH0; qh <= QH1; ++qh) {
         float win[NW];
@@ -544,7 +468,7 @@ template <int KS, int ST>
 __global__ void __launch_bounds__(dev::kBlock)
 dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, float *__restrict__ partial,
                DwGeom g) {
-  using S = Strip<KS, ST>;
+  using S = dev::Strip<KS, ST, KS / 2>;
   constexpr int PAD = KS / 2, NW = S::NW;
   constexpr int T = KS * KS + 1;
   constexpr int nWaves = dev::kBlock / dev::kWave;
@@ -759,16 +683,16 @@ bool stripGeometry(const DwGeom &g) {
 
 // LDS floats of a staged input band of `rows` rows in the strip layout
 size_t stripFloats(const DwGeom &g, int rows) {
-  if (g.dH == 1) return g.kH == 3 ? Strip<3, 1>::floats(rows, g.W) : Strip<5, 1>::floats(rows, g.W);
-  return g.kH == 3 ? Strip<3, 2>::floats(rows, g.W) : Strip<5, 2>::floats(rows, g.W);
+  if (g.dH == 1) return g.kH == 3 ? dev::Strip<3, 1, 1>::floats(rows, g.W) : dev::Strip<5, 1, 2>::floats(rows, g.W);
+  return g.kH == 3 ? dev::Strip<3, 2, 1>::floats(rows, g.W) : dev::Strip<5, 2, 2>::floats(rows, g.W);
 }
 
 // rows of gradOutput staged beyond the h/ST rows of a gradInput band
 int gradInputExtraRows(int ks, int st) {
-  if (ks == 3 && st == 1) return TapSpan<3, 1, 1>::hi() - TapSpan<3, 1, 1>::lo();
-  if (ks == 3 && st == 2) return TapSpan<3, 2, 2>::hi() - TapSpan<3, 2, 2>::lo();
-  if (ks == 5 && st == 1) return TapSpan<5, 1, 1>::hi() - TapSpan<5, 1, 1>::lo();
-  return TapSpan<5, 2, 2>::hi() - TapSpan<5, 2, 2>::lo();
+  if (ks == 3 && st == 1) return dev::TapSpan<3, 1, 1, 1>::hi() - dev::TapSpan<3, 1, 1, 1>::lo();
+  if (ks == 3 && st == 2) return dev::TapSpan<3, 2, 2, 1>::hi() - dev::TapSpan<3, 2, 2, 1>::lo();
+  if (ks == 5 && st == 1) return dev::TapSpan<5, 1, 1, 2>::hi() - dev::TapSpan<5, 1, 1, 2>::lo();
+  return dev::TapSpan<5, 2, 2, 2>::hi() - dev::TapSpan<5, 2, 2, 2>::lo();
 }
 
 }  // namespace
@@ -859,8 +783,8 @@ void THNN_CudaSpatialDepthWiseConvolution_updateGradInput(THCState *state, THCud
   };
   if (stripGeometry(g) && vec && aligned16(data(gradInput))) {
     const int extra = gradInputExtraRows(g.kH, g.dH);
-    const int pitch = g.oW + kStripPadL;
-    auto sbytes = [&](int units) { return (size_t)g.M * ((size_t)(units + extra) * pitch + kStripPadL) * sizeof(float); };
+    const int pitch = g.oW + dev::kStripPadL;
+    auto sbytes = [&](int units) { return (size_t)g.M * ((size_t)(units + extra) * pitch + dev::kStripPadL) * sizeof(float); };
     int units = 0;
     if (launch::pickBand(ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
       g.tileRows = units * g.dH;

@@ -13,6 +13,7 @@
 
 #include "device_utils.h"
 #include "launch_utils.h"
+#include "strip.h"
 #include "thc_internal.h"
 
 using namespace thc;
@@ -292,12 +293,242 @@ avgPoolBwdDirect(const float *__restrict__ gradOut, float *__restrict__ gradIn, 
   }
 }
 
+// ============================================================ strip kernels ==
+// Fast paths for square windows without dilation whose geometry (KS, ST, PAD) is
+// known at compile time and whose rows are multiples of 4 (see strip.h). A lane
+// produces 4 consecutive outputs (forward) or an ST x 4 patch (backward); cells
+// outside the image hold a neutral fill (-FLT_MAX for max, 0 for sums), so the
+// scans run without bounds tests while visiting elements in the reference's
+// order (rows outer, columns inner).
+
+template <int KS, int ST, int PAD>
+__global__ void __launch_bounds__(dev::kBlock)
+maxPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, long *__restrict__ indices, PoolGeom g) {
+  using S = dev::Strip<KS, ST, PAD>;
+  constexpr int NW = S::NW;
+  extern __shared__ float smem[];
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  const int ph0 = tile * g.tileRows;
+  const int nOut = min(g.tileRows, g.oH - ph0);
+  const int nIn = (nOut - 1) * ST + KS;
+  const int pitch = S::pitch(g.W);
+  S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, ph0 * ST - PAD, nIn, -FLT_MAX);
+  __syncthreads();
+  const int oW4 = g.oW >> 2;
+  const int total = nOut * oW4;
+  const long obase = ((long)plane * g.oH + ph0) * g.oW;
+  for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    const int r = i / oW4, b4 = i - r * oW4;
+    const float *p = smem + r * ST * pitch;
+    float mv[4] = {-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+    int mi[4] = {-1, -1, -1, -1};
+    const int idx0 = ((ph0 + r) * ST - PAD) * g.W + b4 * 4 * ST - PAD;  // flat index of window element (kh=0, j=0)
+#pragma unroll
+    for (int kh = 0; kh < KS; ++kh) {
+      float win[NW];
+      S::loadWin(p + kh * pitch, b4, g.W, win);
+#pragma unroll
+      for (int kw = 0; kw < KS; ++kw)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (win[q * ST + kw] > mv[q]) {
+            mv[q] = win[q * ST + kw];
+            mi[q] = idx0 + kh * g.W + q * ST + kw;
+          }
+    }
+    const long o = obase + (long)r * g.oW + b4 * 4;
+    *reinterpret_cast<float4 *>(out + o) = make_float4(mv[0], mv[1], mv[2], mv[3]);
+    long2 i01, i23;
+    i01.x = (long)mi[0] + TH_INDEX_BASE, i01.y = (long)mi[1] + TH_INDEX_BASE;
+    i23.x = (long)mi[2] + TH_INDEX_BASE, i23.y = (long)mi[3] + TH_INDEX_BASE;
+    *reinterpret_cast<long2 *>(indices + o) = i01;
+    *reinterpret_cast<long2 *>(indices + o + 2) = i23;
+  }
+}
+
+template <int KS, int ST, int PAD, bool INCLUDE_PAD>
+__global__ void __launch_bounds__(dev::kBlock)
+avgPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, PoolGeom g) {
+  using S = dev::Strip<KS, ST, PAD>;
+  constexpr int NW = S::NW;
+  extern __shared__ float smem[];
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  const int ph0 = tile * g.tileRows;
+  const int nOut = min(g.tileRows, g.oH - ph0);
+  const int nIn = (nOut - 1) * ST + KS;
+  const int pitch = S::pitch(g.W);
+  S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, ph0 * ST - PAD, nIn, 0.f);
+  __syncthreads();
+  const int oW4 = g.oW >> 2;
+  const int total = nOut * oW4;
+  const long obase = ((long)plane * g.oH + ph0) * g.oW;
+  for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    const int r = i / oW4, b4 = i - r * oW4;
+    const float *p = smem + r * ST * pitch;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kh = 0; kh < KS; ++kh) {
+      float win[NW];
+      S::loadWin(p + kh * pitch, b4, g.W, win);
+#pragma unroll
+      for (int kw = 0; kw < KS; ++kw)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[q] += win[q * ST + kw];
+    }
+    float res[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      int hs, he, ws, we;
+      res[q] = acc[q] / avgDivisor<INCLUDE_PAD>(ph0 + r, b4 * 4 + q, g, hs, he, ws, we);
+    }
+    *reinterpret_cast<float4 *>(out + obase + (long)r * g.oW + b4 * 4) = make_float4(res[0], res[1], res[2], res[3]);
+  }
+}
+
+// Backward gathers. MAX: gradOutput and the argmax (narrowed to int32, base
+// removed, -2 outside) are staged with a 4-cell fill in front of every row; a
+// patch element adds the gradOutput of each covering window whose argmax is that
+// element. Otherwise (average): gradOutput / divisor(window) is staged and the
+// covering windows are summed.
+template <int KS, int ST, int PAD, bool MAX, bool INCLUDE_PAD>
+__global__ void __launch_bounds__(dev::kBlock)
+poolBwdStrip(const float *__restrict__ gradOut, const long *__restrict__ indices, float *__restrict__ gradIn,
+             PoolGeom g, int stageRows) {
+  constexpr int QH0 = dev::TapSpan<KS, ST, ST, PAD>::lo(), QH1 = dev::TapSpan<KS, ST, ST, PAD>::hi();
+  constexpr int QW0 = dev::TapSpan<KS, ST, 4, PAD>::lo(), QW1 = dev::TapSpan<KS, ST, 4, PAD>::hi();
+  constexpr int NW = QW1 - QW0 + 1;
+  constexpr int CPB = 4 / ST;
+  constexpr int OFF = ((dev::kStripPadL + QW0) % 4 + 4) % 4;
+  constexpr int ALIGN = (CPB % 4 == 0) ? 4 : 2;
+  extern __shared__ float smem[];
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  const int h0 = tile * g.tileRows;  // multiple of ST
+  const int nRows = min(g.tileRows, g.H - h0);
+  const int pitch = g.oW + dev::kStripPadL;
+  const int region = stageRows * pitch + dev::kStripPadL;
+  float *gs = smem;
+  float *is = smem + region;  // int32 bit patterns (MAX only)
+  const int ph0 = h0 / ST + QH0;
+  const float *gp = gradOut + (long)plane * g.oH * g.oW;
+  if (MAX) {
+    dev::loadRowsPadded<true>(gs, gp, g.oH, g.oW, ph0, stageRows, pitch, dev::kStripPadL, 0.f);
+    const long *ip = indices + (long)plane * g.oH * g.oW;
+    const int cnt = stageRows * pitch + dev::kStripPadL;
+    for (int i = threadIdx.x; i < cnt; i += blockDim.x) {
+      int r = i / pitch, cc = i - r * pitch - dev::kStripPadL;
+      int ph = ph0 + r;
+      int v = -2;
+      if (cc >= 0 && r < stageRows && ph >= 0 && ph < g.oH) v = (int)(ip[(long)ph * g.oW + cc] - TH_INDEX_BASE);
+      is[i] = __int_as_float(v);
+    }
+  } else {
+    const int cnt = stageRows * pitch + dev::kStripPadL;
+    for (int i = threadIdx.x; i < cnt; i += blockDim.x) {
+      int r = i / pitch, cc = i - r * pitch - dev::kStripPadL;
+      int ph = ph0 + r;
+      float v = 0.f;
+      if (cc >= 0 && r < stageRows && ph >= 0 && ph < g.oH) {
+        int hs, he, ws, we;
+        v = gp[(long)ph * g.oW + cc] / avgDivisor<INCLUDE_PAD>(ph, cc, g, hs, he, ws, we);
+      }
+      gs[i] = v;
+    }
+  }
+  __syncthreads();
+  const int W4 = g.W >> 2;
+  const int nA = (nRows + ST - 1) / ST;
+  const int total = nA * W4;
+  float *o = gradIn + ((long)plane * g.H + h0) * g.W;
+  for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    const int a = i / W4, b = i - a * W4;
+    float acc[ST][4];
+#pragma unroll
+    for (int dy = 0; dy < ST; ++dy)
+#pragma unroll
+      for (int dx = 0; dx < 4; ++dx) acc[dy][dx] = 0.f;
+    const int me0 = (h0 + a * ST) * g.W + b * 4;  // flat index of patch element (0, 0)
+    const int woff = dev::kStripPadL + QW0 + b * CPB;
+#pragma unroll
+    for (int qh = QH0; qh <= QH1; ++qh) {
+      float gw[NW], iw[NW];
+      dev::readWindow<0, NW, OFF, ALIGN>(gs + (a + qh - QH0) * pitch + woff, gw);
+      if (MAX) dev::readWindow<0, NW, OFF, ALIGN>(is + (a + qh - QH0) * pitch + woff, iw);
+#pragma unroll
+      for (int dy = 0; dy < ST; ++dy) {
+        const int kh = dy + PAD - qh * ST;
+        if (kh < 0 || kh >= KS) continue;
+#pragma unroll
+        for (int dx = 0; dx < 4; ++dx)
+#pragma unroll
+          for (int kw = KS - 1; kw >= 0; --kw) {  // descending kw = ascending window column
+            const int t = dx + PAD - kw;
+            if (t % ST != 0) continue;
+            if (MAX) {
+              if (__float_as_int(iw[t / ST - QW0]) == me0 + dy * g.W + dx) acc[dy][dx] += gw[t / ST - QW0];
+            } else {
+              acc[dy][dx] += gw[t / ST - QW0];
+            }
+          }
+      }
+    }
+#pragma unroll
+    for (int dy = 0; dy < ST; ++dy)
+      if (a * ST + dy < nRows)
+        *reinterpret_cast<float4 *>(o + (long)(a * ST + dy) * g.W + b * 4) =
+            make_float4(acc[dy][0], acc[dy][1], acc[dy][2], acc[dy][3]);
+  }
+}
+
 // -------------------------------------------------------------- host side ----
 using launch::aligned16;
 
-bool forceDirect() {
+// 1: shape-agnostic direct kernels, 2: generic LDS-tiled kernels (no strip fast path).
+int forcedPath() {
   const char *e = getenv("THCUNN_POOL_FORCE_DIRECT");
-  return e && e[0] == '1';
+  return e ? atoi(e) : 0;
+}
+bool forceDirect() { return forcedPath() == 1; }
+
+// (KS, ST, PAD) combinations the strip kernels are instantiated for
+#define POOL_STRIP_COMBOS(X) X(3, 2, 1) X(2, 2, 0) X(3, 2, 0) X(3, 1, 1)
+
+bool stripCombo(const PoolGeom &g) {
+  if (g.kH != g.kW || g.dH != g.dW || g.padH != g.padW || g.dilH != 1 || g.dilW != 1) return false;
+#define X(K, S, P) \
+  if (g.kH == K && g.dH == S && g.padH == P) return true;
+  POOL_STRIP_COMBOS(X)
+#undef X
+  return false;
+}
+
+// Forward strips read 4 fill cells beyond a row at most (and, in the split
+// stride-2 layout, only even columns may overhang).
+bool stripFwdOk(const PoolGeom &g) {
+  if (forcedPath() != 0 || !stripCombo(g) || g.oW % 4 != 0) return false;
+  if (g.W % (4 * g.dW) != 0) return false;
+  int cmax = (g.oW - 1) * g.dW - g.padW + g.kW - 1;  // last column any window touches
+  if (g.dW == 1) return cmax <= g.W + 3;
+  int emax = cmax % 2 == 0 ? cmax : cmax - 1, omax = cmax % 2 == 1 ? cmax : cmax - 1;
+  return emax <= g.W + 6 && omax <= g.W - 1;
+}
+bool stripBwdOk(const PoolGeom &g) { return forcedPath() == 0 && stripCombo(g) && g.oW % 4 == 0 && g.W % 4 == 0; }
+
+int bwdExtraRows(const PoolGeom &g) {
+#define X(K, S, P) \
+  if (g.kH == K && g.dH == S && g.padH == P) return dev::TapSpan<K, S, S, P>::hi() - dev::TapSpan<K, S, S, P>::lo();
+  POOL_STRIP_COMBOS(X)
+#undef X
+  return 0;
+}
+size_t fwdStripFloats(const PoolGeom &g, int rows) {
+#define X(K, S, P) \
+  if (g.kH == K && g.dH == S && g.padH == P) return dev::Strip<K, S, P>::floats(rows, g.W);
+  POOL_STRIP_COMBOS(X)
+#undef X
+  return 0;
 }
 
 // Output extent rule shared by max and average pooling
@@ -404,7 +635,18 @@ void maxPoolUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *out
     bool vec = g.W % 4 == 0 && aligned16(in.ptr());
     auto stageRows = [&](int rows) { return std::min(g.H, (rows - 1) * g.dH + (g.kH - 1) * g.dilH + 1); };
     auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.W * sizeof(float); };
-    if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
+    auto sbytes = [&](int rows) { return fwdStripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
+    if (stripFwdOk(g) && vec && aligned16(data(output)) && aligned16(data(indices)) &&
+        launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane)) {
+      g.nblk = (int)(planes * g.tilesPerPlane);
+      dim3 grid(g.nblk), block(dev::kBlock);
+      size_t lds = sbytes(g.tileRows);
+#define X(K, S, P)                                  \
+  if (g.kH == K && g.dH == S && g.padH == P)       \
+    maxPoolFwdStrip<K, S, P><<<grid, block, lds, s>>>(in.ptr(), data(output), data(indices), g);
+      POOL_STRIP_COMBOS(X)
+#undef X
+    } else if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
       if (vec)
         launchMaxFwd<true>(s, bytes(g.tileRows), in.ptr(), data(output), data(indices), g);
@@ -442,7 +684,22 @@ void maxPoolUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *
   bool vec = g.oW % 4 == 0 && aligned16(go.ptr());
   auto stageRows = [&](int rows) { return std::min(g.oH, (rows + extH - 2) / g.dH + 2); };
   auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.oW * (sizeof(float) + sizeof(int)); };
-  if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
+  const int extra = bwdExtraRows(g);
+  const int spitch = g.oW + dev::kStripPadL;
+  auto sbytes = [&](int units) { return 2 * ((size_t)(units + extra) * spitch + dev::kStripPadL) * sizeof(float); };
+  int units = 0;
+  if (stripBwdOk(g) && vec && aligned16(data(gradInput)) &&
+      launch::pickBand(launch::ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
+    g.tileRows = units * g.dH;
+    g.nblk = (int)(planes * g.tilesPerPlane);
+    dim3 grid(g.nblk), block(dev::kBlock);
+    size_t lds = sbytes(units);
+#define X(K, S, P)                            \
+  if (g.kH == K && g.dH == S && g.padH == P) \
+    poolBwdStrip<K, S, P, true, true><<<grid, block, lds, s>>>(go.ptr(), data(indices), data(gradInput), g, units + extra);
+    POOL_STRIP_COMBOS(X)
+#undef X
+  } else if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
     g.maxStageRows = stageRows(g.tileRows);
     dim3 grid(g.nblk), block(dev::kBlock);
@@ -515,7 +772,22 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
     bool vec = g.W % 4 == 0 && aligned16(in.ptr());
     auto stageRows = [&](int rows) { return std::min(g.H, (rows - 1) * g.dH + g.kH); };
     auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.W * sizeof(float); };
-    if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
+    auto sbytes = [&](int rows) { return fwdStripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
+    if (stripFwdOk(g) && vec && aligned16(data(output)) &&
+        launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane)) {
+      g.nblk = (int)(planes * g.tilesPerPlane);
+      dim3 grid(g.nblk), block(dev::kBlock);
+      size_t lds = sbytes(g.tileRows);
+#define X(K, S, P)                                                                        \
+  if (g.kH == K && g.dH == S && g.padH == P) {                                           \
+    if (count_include_pad)                                                               \
+      avgPoolFwdStrip<K, S, P, true><<<grid, block, lds, s>>>(in.ptr(), data(output), g);  \
+    else                                                                                 \
+      avgPoolFwdStrip<K, S, P, false><<<grid, block, lds, s>>>(in.ptr(), data(output), g); \
+  }
+      POOL_STRIP_COMBOS(X)
+#undef X
+    } else if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
       dim3 grid(g.nblk), block(dev::kBlock);
       size_t lds = bytes(g.tileRows);
@@ -564,7 +836,26 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
   bool vec = g.oW % 4 == 0 && aligned16(go.ptr());
   auto stageRows = [&](int rows) { return std::min(g.oH, (rows + g.kH - 2) / g.dH + 2); };
   auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.oW * sizeof(float); };
-  if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
+  const int extra = bwdExtraRows(g);
+  const int spitch = g.oW + dev::kStripPadL;
+  auto sbytes = [&](int units) { return ((size_t)(units + extra) * spitch + dev::kStripPadL) * sizeof(float); };
+  int units = 0;
+  if (stripBwdOk(g) && vec && aligned16(data(gradInput)) &&
+      launch::pickBand(launch::ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
+    g.tileRows = units * g.dH;
+    g.nblk = (int)(planes * g.tilesPerPlane);
+    dim3 grid(g.nblk), block(dev::kBlock);
+    size_t lds = sbytes(units);
+#define X(K, S, P)                                                                                                    \
+  if (g.kH == K && g.dH == S && g.padH == P) {                                                                       \
+    if (count_include_pad)                                                                                           \
+      poolBwdStrip<K, S, P, false, true><<<grid, block, lds, s>>>(go.ptr(), nullptr, data(gradInput), g, units + extra);  \
+    else                                                                                                             \
+      poolBwdStrip<K, S, P, false, false><<<grid, block, lds, s>>>(go.ptr(), nullptr, data(gradInput), g, units + extra); \
+  }
+    POOL_STRIP_COMBOS(X)
+#undef X
+  } else if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
     dim3 grid(g.nblk), block(dev::kBlock);
     size_t lds = bytes(g.tileRows);

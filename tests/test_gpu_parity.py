@@ -201,6 +201,9 @@ POOL_CASES = [
     (4, 7, 32, 32, 3, 3, 1, 1, 1, 1, False),
     (1, 1, 5, 5, 2, 2, 1, 1, 1, 1, False),
     (1, 2, 300, 260, 3, 3, 2, 2, 1, 1, False),   # several row bands per plane
+    (2, 3, 48, 48, 3, 3, 2, 2, 0, 0, True),      # unpadded 3x3 s2, ceil mode: last window overhangs
+    (1, 2, 300, 264, 3, 3, 2, 2, 1, 1, False),   # strip kernels, several bands
+    (2, 2, 31, 40, 3, 3, 1, 1, 1, 1, False),     # 3x3 s1 strip with odd height
 ]
 
 
@@ -238,9 +241,10 @@ def test_maxpool_ties_bit_exact(T, case):
     _maxpool_run(T, case, _tied_input(case[:4], 20))
 
 
-@pytest.mark.parametrize("case", POOL_CASES[:6])
-def test_maxpool_direct_kernels(T, case):
-    with force_direct("THCUNN_POOL_FORCE_DIRECT"):
+@pytest.mark.parametrize("case", POOL_CASES[:6] + POOL_CASES[9:10])
+@pytest.mark.parametrize("mode", ["1", "2"])
+def test_maxpool_fallback_kernels(T, case, mode):
+    with force_direct("THCUNN_POOL_FORCE_DIRECT", mode):
         _maxpool_run(T, case, _tied_input(case[:4], 21, q=8))
 
 
@@ -295,11 +299,12 @@ def test_avgpool(T, case, include_pad):
     _avgpool_run(T, case, include_pad)
 
 
-@pytest.mark.parametrize("case", POOL_CASES[2:6])
+@pytest.mark.parametrize("case", POOL_CASES[:6])
 def test_avgpool_direct_and_noncontiguous(T, case):
-    with force_direct("THCUNN_POOL_FORCE_DIRECT"):
-        _avgpool_run(T, case, True)
-        _avgpool_run(T, case, False)
+    for mode in ("1", "2"):
+        with force_direct("THCUNN_POOL_FORCE_DIRECT", mode):
+            _avgpool_run(T, case, True)
+            _avgpool_run(T, case, False)
     rng = np.random.default_rng(31)
     _avgpool_run(T, case, True, xt=lambda a: T.CudaTensor.noncontiguous_from_numpy(a, rng))
 
@@ -317,7 +322,9 @@ def test_avgpool_reference_known_answer(T):
 
 
 # ------------------------------------------------------------------------- BN --
-BN_SHAPES = [(8, 16, 28, 28), (4, 3, 7, 5), (32, 64), (2, 5, 33), (3, 2, 4, 5, 6), (2, 2, 150, 120), (1, 3, 9000)]
+BN_SHAPES = [(8, 16, 28, 28), (4, 3, 7, 5), (32, 64), (2, 5, 33), (3, 2, 4, 5, 6), (2, 2, 150, 120), (1, 3, 9000),
+             # channel-resident kernels (C >= 96, a channel fits one workgroup's registers)
+             (64, 100, 28, 28), (40, 96, 20, 20), (33, 97, 12, 12), (4, 128, 14, 14), (57, 96, 24, 28)]
 
 
 def _bn_run(T, shape, affine, seed=40):
@@ -373,6 +380,14 @@ def _bn_run(T, shape, affine, seed=40):
 @pytest.mark.parametrize("affine", [True, False])
 def test_batchnorm(T, shape, affine):
     _bn_run(T, shape, affine)
+
+
+def test_batchnorm_chunked_path_on_resident_shape(T):
+    os.environ["THCUNN_BN_FORCE_CHUNKED"] = "1"
+    try:
+        _bn_run(T, (40, 96, 20, 20), True)
+    finally:
+        os.environ.pop("THCUNN_BN_FORCE_CHUNKED", None)
 
 
 def test_batchnorm_large_mean_and_zero_variance(T):

@@ -17,6 +17,9 @@
 //   updateGradInput    gradCol[k][n,l] = sum_o W[o][k] * gy[n][o][l] for a group
 //                      of images into `gradColumns`, then the col2im gather of
 //                      lib/THCUNN/im2col.h:63-102 over the group.
+#include <map>
+#include <mutex>
+
 #include "device_utils.h"
 #include "launch_utils.h"
 #include "thc_internal.h"
@@ -45,7 +48,7 @@ struct GemmArgs {
   float *c;         // forward: out; gradCol: gradCol of the group; gradWeight: partials
   const float *bias;
   int M, Ncols, R;  // GEMM extents: C is M x Ncols, reduction length R (per split)
-  int n0;           // first image of the group (gradCol) / images per split (gradWeight)
+  int n0;           // first image of the group (gradCol) / reduction tiles (of BK positions) per split (gradWeight)
   int nImages;      // images covered by this launch
   int mTiles;
   bool vecA;        // A rows may be fetched with 16-byte loads (extent % 4 == 0, aligned base)
@@ -131,10 +134,10 @@ convGemmKernel(GemmArgs p, ConvGeom g) {
   }
   // gradWeight: B column = k index (c, kh, kw), 16-lane groups walk consecutive positions
   const int gwR = t & 15, gwJ = t >> 4;  // reduction row within the tile, first of 8 columns (stride 16)
-  const int imgFirst = (MODE == kGradWeight) ? split * p.n0 : 0;
-  const int imgCount = (MODE == kGradWeight) ? min(p.n0, p.nImages - imgFirst) : 0;
-  const long Rlen = (MODE == kGradWeight) ? (long)imgCount * g.L : (long)p.R;
-  const int nkt = (int)((Rlen + BK - 1) / BK);
+  // gradWeight: split `split` reduces positions [rBegin, rEnd) of the N*L positions of the batch
+  const long rBegin = (MODE == kGradWeight) ? (long)split * p.n0 * BK : 0;
+  const long rEnd = (MODE == kGradWeight) ? min(rBegin + (long)p.n0 * BK, (long)p.nImages * g.L) : (long)p.R;
+  const int nkt = (int)((rEnd - rBegin + BK - 1) / BK);
 
   auto loadTiles = [&](int kt) {
     const int r0 = kt * BK;
@@ -190,27 +193,27 @@ convGemmKernel(GemmArgs p, ConvGeom g) {
       // gradWeight. A[m = o][r = (n,l)] = gy[n][o][l]: contiguous along r inside an image
       {
         int o = m0 + rowT;
-        long r = (long)r0 + redT8;
+        long r = rBegin + r0 + redT8;
         bool rowOk = o < p.M;
         int n = (int)(r / g.L);
         int l = (int)(r - (long)n * g.L);
-        if (p.vecA && rowOk && r + 8 <= Rlen) {
+        if (p.vecA && rowOk && r + 8 <= rEnd) {
           // with L % 4 == 0 a group of 4 never straddles an image
-          const float *s0 = p.a + ((long)(imgFirst + n) * g.Cout + o) * g.L + l;
+          const float *s0 = p.a + ((long)n * g.Cout + o) * g.L + l;
           float4 v0 = *reinterpret_cast<const float4 *>(s0);
           int l2 = l + 4, n2 = n;
           if (l2 >= g.L) {
             l2 -= g.L;
             ++n2;
           }
-          const float *s1 = p.a + ((long)(imgFirst + n2) * g.Cout + o) * g.L + l2;
+          const float *s1 = p.a + ((long)n2 * g.Cout + o) * g.L + l2;
           float4 v1 = *reinterpret_cast<const float4 *>(s1);
           ra[0] = v0.x, ra[1] = v0.y, ra[2] = v0.z, ra[3] = v0.w;
           ra[4] = v1.x, ra[5] = v1.y, ra[6] = v1.z, ra[7] = v1.w;
         } else {
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
-            ra[i] = (rowOk && r + i < Rlen) ? p.a[((long)(imgFirst + n) * g.Cout + o) * g.L + l] : 0.f;
+            ra[i] = (rowOk && r + i < rEnd) ? p.a[((long)n * g.Cout + o) * g.L + l] : 0.f;
             if (++l == g.L) {
               l = 0;
               ++n;
@@ -220,12 +223,12 @@ convGemmKernel(GemmArgs p, ConvGeom g) {
       }
       // B[r = (n,l)][j = k] = col[k][n,l]; lanes 0..15 of a group walk consecutive l
       {
-        long r = (long)r0 + gwR;
-        bool rOk = r < Rlen;
+        long r = rBegin + r0 + gwR;
+        bool rOk = r < rEnd;
         int n = rOk ? (int)(r / g.L) : 0;
         int l = rOk ? (int)(r - (long)n * g.L) : 0;
         int oh = l / g.oW, ow = l - oh * g.oW;
-        const float *xb = p.b + (long)(imgFirst + n) * g.Cin * g.H * g.W;
+        const float *xb = p.b + (long)n * g.Cin * g.H * g.W;
         int ih0g = oh * g.dH - g.padH, iw0g = ow * g.dW - g.padW;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -313,6 +316,217 @@ convGemmKernel(GemmArgs p, ConvGeom g) {
   }
 }
 
+// ---- forward implicit GEMM, second generation ---------------------------------
+// Same 128x128x16 tiling as convGemmKernel<kForward>, with the two costs that
+// kept the MFMA pipe at ~40 % removed:
+//  * operands sit in LDS as float4 groups of 4 consecutive k
+//    (As[kg][row], Bs[kg][col]); a lane fetches the operands of four MFMAs with
+//    one ds_read_b128 and the loaders store with ds_write_b128. Lane group
+//    g = lane / 32 of super-step s consumes k-group 2s + g, i.e. MFMA j contracts
+//    k = 8s + j (g = 0) with k = 8s + 4 + j (g = 1) - any pairing is valid as long
+//    as A and B agree.
+//  * the im2col gather is a buffer load: the image base is a scalar resource,
+//    the lane's position (n, oh, ow) is a fixed 32-bit byte offset, and the tap
+//    (c, kh, kw) of each k is wave-uniform, so it lives in scalar registers.
+//    A tap outside the image gets an out-of-range offset, for which the buffer
+//    unit returns 0 - the zero padding costs no branch.
+constexpr int FPITCH = BM + 8;  // float4 per k-group row: +8 keeps the 2 k-groups a lane pair writes in disjoint banks
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+struct FwdArgs {
+  const float *w;     // (M x K) row-major
+  const float *x;     // images n0 .. n0 + nImages - 1 of (N, Cin, H, W)
+  float *out;         // (nImages, M, L)
+  const float *bias;  // M or null
+  int M, Ncols;       // Ncols = nImages * L
+  int mTiles;
+  int xBytes;         // bytes of the nImages input images (< 2^31)
+  bool vecA;
+  // tail launch: tiles tile0 .. are each reduced by nSplit workgroups over ktPerSplit k-tiles;
+  // their 128x128 partial tiles go to `partial` and fwdTailFixupKernel folds them
+  int tile0, nSplit, ktPerSplit;
+  float *partial;
+};
+
+__global__ void __launch_bounds__(dev::kBlock)
+convFwdImplicitKernel(FwdArgs p, ConvGeom g) {
+  __shared__ float4 As[2][BK / 4][FPITCH];
+  __shared__ float4 Bs[2][BK / 4][FPITCH];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tileIdx = p.tile0 + blockIdx.x;
+  const int mTile = tileIdx % p.mTiles, nTile = tileIdx / p.mTiles;
+  const int m0 = mTile * BM, j0 = nTile * BN;
+  const int KK = g.kH * g.kW;
+
+  float16v acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // A loader: row (t >> 1), k = 8 * (t & 1) .. + 7
+  const int rowA = t >> 1, kA = (t & 1) * 8;
+  const bool rowOk = m0 + rowA < p.M;
+  const float *aSrc = p.w + (long)(m0 + rowA) * g.K + kA;
+  // B loader: column (t & 127) = one output position, k = 8 * (t >> 7) .. + 7 (wave-uniform)
+  const int colB = t & 127;
+  const int kB = __builtin_amdgcn_readfirstlane((t >> 7) * 8);
+  const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.xBytes, 0x00020000);
+  const int kOob = 0x7fffffff;  // beyond num_records: the load returns 0
+  int ih0 = 0, iw0 = 0, posOff = kOob;
+  {
+    long lg = (long)j0 + colB;
+    if (lg < (long)p.Ncols) {
+      int n = (int)(lg / g.L);
+      int l = (int)(lg - (long)n * g.L);
+      int oh = l / g.oW, ow = l - oh * g.oW;
+      ih0 = oh * g.dH - g.padH;
+      iw0 = ow * g.dW - g.padW;
+      posOff = ((n * g.Cin * g.H + ih0) * g.W + iw0) * 4;  // may be "negative": only used when the tap is inside
+    } else {
+      ih0 = -(1 << 28);  // every tap fails the bounds test
+    }
+  }
+
+  float4 ra[2], rb[2];
+  const int nktAll = (g.K + BK - 1) / BK;
+  const int ktBegin = blockIdx.y * p.ktPerSplit;
+  const int nkt = min(nktAll, ktBegin + p.ktPerSplit);  // this workgroup reduces k-tiles [ktBegin, nkt)
+
+  auto loadTiles = [&](int kt) {
+    const int k0 = kt * BK;
+    // ---- A
+    if (p.vecA && rowOk && k0 + kA + 8 <= g.K) {
+      ra[0] = reinterpret_cast<const float4 *>(aSrc + k0)[0];
+      ra[1] = reinterpret_cast<const float4 *>(aSrc + k0)[1];
+    } else {
+      float tmp[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) tmp[i] = (rowOk && k0 + kA + i < g.K) ? aSrc[k0 + i] : 0.f;
+      ra[0] = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
+      ra[1] = make_float4(tmp[4], tmp[5], tmp[6], tmp[7]);
+    }
+    // ---- B: scalar walk over the 8 taps of this wave
+    int k = k0 + kB;  // scalar
+    int c = k / KK, rem = k - c * KK;
+    int kh = rem / g.kW, kw = rem - kh * g.kW;
+    float tmp[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int ih = ih0 + kh, iw = iw0 + kw;
+      const bool ok = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W && (k + i) < g.K;
+      const int soff = ((c * g.H + kh) * g.W + kw) * 4;  // scalar
+      const int off = ok ? posOff + soff : kOob;
+      tmp[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
+      if (++kw == g.kW) {
+        kw = 0;
+        if (++kh == g.kH) {
+          kh = 0;
+          ++c;
+        }
+      }
+    }
+    rb[0] = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
+    rb[1] = make_float4(tmp[4], tmp[5], tmp[6], tmp[7]);
+  };
+  auto storeTiles = [&](int buf) {
+    As[buf][(t & 1) * 2][rowA] = ra[0];
+    As[buf][(t & 1) * 2 + 1][rowA] = ra[1];
+    Bs[buf][(t >> 7) * 2][colB] = rb[0];
+    Bs[buf][(t >> 7) * 2 + 1][colB] = rb[1];
+  };
+
+  loadTiles(ktBegin);
+  storeTiles(ktBegin & 1);
+  __syncthreads();
+  const int grp = lane >> 5, idx = lane & 31;
+  for (int kt = ktBegin; kt < nkt; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nkt) loadTiles(kt + 1);
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const float4 a0 = As[buf][2 * s + grp][wm * 64 + idx], a1 = As[buf][2 * s + grp][wm * 64 + 32 + idx];
+      const float4 b0 = Bs[buf][2 * s + grp][wn * 64 + idx], b1 = Bs[buf][2 * s + grp][wn * 64 + 32 + idx];
+      const float av0[4] = {a0.x, a0.y, a0.z, a0.w}, av1[4] = {a1.x, a1.y, a1.z, a1.w};
+      const float bv0[4] = {b0.x, b0.y, b0.z, b0.w}, bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv0[j], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv1[j], acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv0[j], acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv1[j], acc[1][1], 0, 0, 0);
+      }
+    }
+    if (kt + 1 < nkt) storeTiles(buf ^ 1);
+    __syncthreads();
+  }
+
+  // epilogue: lane holds column (lane & 31), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
+  const int rowHalf = grp * 4;
+  if (p.nSplit > 1) {
+    float *dst = p.partial + ((long)blockIdx.x * p.nSplit + blockIdx.y) * (BM * BN);
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+      for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          dst[(wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3)) * BN + wn * 64 + tj * 32 + idx] = acc[ti][tj][v];
+    return;
+  }
+#pragma unroll
+  for (int tj = 0; tj < 2; ++tj) {
+    const long col = (long)j0 + wn * 64 + tj * 32 + idx;
+    if (col >= p.Ncols) continue;
+    const int n = (int)(col / g.L);
+    const int l = (int)(col - (long)n * g.L);
+    float *dst = p.out + (long)n * p.M * g.L + l;
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
+        if (row < p.M) {
+          float val = acc[ti][tj][v];
+          if (p.bias) val += p.bias[row];
+          dst[(long)row * g.L] = val;
+        }
+      }
+  }
+}
+
+// out tile = bias + sum over the nSplit partial tiles (ascending split order).
+// grid = (tail tiles, BM*BN / 1024): a workgroup folds 1024 consecutive tile elements, 4 per lane.
+__global__ void __launch_bounds__(dev::kBlock)
+fwdTailFixupKernel(FwdArgs p, ConvGeom g) {
+  const int tileIdx = p.tile0 + blockIdx.x;
+  const int mTile = tileIdx % p.mTiles, nTile = tileIdx / p.mTiles;
+  const float *src = p.partial + (long)blockIdx.x * p.nSplit * (BM * BN);
+  const int e = (blockIdx.y * dev::kBlock + threadIdx.x) * 4;  // BN % 4 == 0: the 4 elements share a row
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s = 0; s < p.nSplit; ++s) {
+    const float4 q = *reinterpret_cast<const float4 *>(src + (long)s * (BM * BN) + e);
+    v.x += q.x, v.y += q.y, v.z += q.z, v.w += q.w;
+  }
+  const int r = e / BN, c = e - r * BN;
+  const int row = mTile * BM + r;
+  if (row >= p.M) return;
+  const float b = p.bias ? p.bias[row] : 0.f;
+  const float vals[4] = {v.x + b, v.y + b, v.z + b, v.w + b};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const long col = (long)nTile * BN + c + i;
+    if (col >= p.Ncols) break;
+    const int n = (int)(col / g.L);
+    const int l = (int)(col - (long)n * g.L);
+    p.out[((long)n * p.M + row) * g.L + l] = vals[i];
+  }
+}
+
 // gW[i] += scale * sum_s partial[s][i], s ascending
 __global__ void __launch_bounds__(dev::kBlock)
 foldPartialsKernel(const float *__restrict__ partial, float *__restrict__ dst, long count, int splits, float scale) {
@@ -324,24 +538,54 @@ foldPartialsKernel(const float *__restrict__ partial, float *__restrict__ dst, l
 }
 
 // gradBias[o] += scale * sum_{n,l} gy[n][o][l]   (lib/THCUNN/generic/SpatialConvolutionMM.cu:440-455)
-__global__ void __launch_bounds__(dev::kBlock)
+// One 1024-lane workgroup per output plane o streams its N runs of L floats.
+constexpr int kBiasBlock = 1024;
+template <bool VEC>
+__global__ void __launch_bounds__(kBiasBlock)
 gradBiasKernel(const float *__restrict__ gy, float *__restrict__ gradBias, int N, int Cout, int L, float scale) {
-  __shared__ float red[dev::kBlock / dev::kWave];
+  __shared__ float red[kBiasBlock / dev::kWave];
   const int o = blockIdx.x;
   float acc = 0.f;
-  const long total = (long)N * L;
-  for (long i = threadIdx.x; i < total; i += blockDim.x) {
-    int n = (int)(i / L);
-    int l = (int)(i - (long)n * L);
-    acc += gy[((long)n * Cout + o) * L + l];
+  if (VEC) {
+    const int L4 = L >> 2;
+    const int total4 = N * L4;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    for (int i = threadIdx.x; i < total4; i += kBiasBlock) {
+      int n = i / L4, l4 = i - n * L4;
+      float4 v = *reinterpret_cast<const float4 *>(gy + ((long)n * Cout + o) * L + (l4 << 2));
+      a0 += v.x, a1 += v.y, a2 += v.z, a3 += v.w;
+    }
+    acc = (a0 + a1) + (a2 + a3);
+  } else {
+    const long total = (long)N * L;
+    for (long i = threadIdx.x; i < total; i += kBiasBlock) {
+      int n = (int)(i / L);
+      int l = (int)(i - (long)n * L);
+      acc += gy[((long)n * Cout + o) * L + l];
+    }
   }
   acc = dev::waveSum(acc);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
   __syncthreads();
   if (threadIdx.x == 0) {
     float s = 0.f;
-    for (int w = 0; w < dev::kBlock / dev::kWave; ++w) s += red[w];
+    for (int w = 0; w < kBiasBlock / dev::kWave; ++w) s += red[w];
     gradBias[o] += scale * s;
+  }
+}
+
+// Wf[c][(o, kh', kw')] = W[o][(c, kH-1-kh', kW-1-kw')]: with these weights the
+// stride-1 gradInput is a plain forward convolution of gradOutput (padding k-1-pad).
+__global__ void __launch_bounds__(dev::kBlock)
+flipWeightKernel(const float *__restrict__ w, float *__restrict__ wf, int Cout, int Cin, int kH, int kW) {
+  const int KK = kH * kW;
+  const long total = (long)Cout * Cin * KK;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    int t = (int)(i % KK);
+    long r = i / KK;
+    int o = (int)(r % Cout);
+    int c = (int)(r / Cout);
+    wf[i] = w[((long)o * Cin + c) * KK + (KK - 1 - t)];
   }
 }
 
@@ -461,6 +705,100 @@ ConvCall convSetup(THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *
 
 inline unsigned tiles(long n, int b) { return (unsigned)((n + b - 1) / b); }
 
+// Workgroups of `kernel` (256 lanes, static LDS) the whole device holds at once.
+// kernel == nullptr: the number of CUs.
+int residentSlots(const void *kernel) {
+  static std::mutex mu;
+  static std::map<const void *, int> cache;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = cache.find(kernel);
+  if (it != cache.end()) return it->second;
+  int dev = 0, cus = 0, perCu = 1;
+  THC_HIP_CHECK(hipGetDevice(&dev));
+  THC_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  if (kernel) THC_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, kernel, dev::kBlock, 0));
+  int v = std::max(1, cus) * std::max(1, perCu);
+  cache[kernel] = v;
+  return v;
+}
+
+// Test switch: "1" routes the forward pass (and the stride-1 gradInput that
+// reuses it) through the first-generation kernels.
+bool forceGeneric() {
+  const char *e = getenv("THCUNN_CONV_FORCE_GENERIC");
+  return e && e[0] == '1';
+}
+
+// Plan of one implicit-GEMM forward launch. The 128x128 tiles are dealt to the
+// CUs in rounds; a last partial round would leave most CUs idle while a few
+// finish one more tile, so the tiles of that round are instead split along K
+// over all CUs (partials in scratch, folded by fwdTailFixupKernel in a fixed order).
+struct FwdPlan {
+  int mTiles, total, full, tail, nSplit, ktPerSplit;
+  long scratchFloats;
+};
+FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
+  FwdPlan pl{};
+  const int nkt = launch::ceilDiv(g.K, BK);
+  pl.mTiles = (int)tiles(M, BM);
+  pl.total = pl.mTiles * (int)tiles((long)nImages * g.L, BN);
+  const int cus = residentSlots(nullptr);
+  pl.tail = pl.total % cus;
+  int nSplit = (pl.tail > 0 && pl.total > cus) ? std::min(nkt / 4, cus / pl.tail) : 1;  // >= 4 k-tiles per split
+  if (nSplit < 2) {
+    pl.tail = 0;
+    nSplit = 1;
+  }
+  pl.full = pl.total - pl.tail;
+  pl.ktPerSplit = launch::ceilDiv(nkt, nSplit);
+  pl.nSplit = launch::ceilDiv(nkt, pl.ktPerSplit);
+  pl.scratchFloats = pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0;
+  return pl;
+}
+
+// out(nImages, M, L) = bias + W(M x K) * im2col(x); `partial` holds plan.scratchFloats floats
+void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *partial, const float *w, const float *x, float *out,
+                       const float *bias, int M, int nImages, const ConvGeom &g) {
+  FwdArgs p{};
+  p.w = w;
+  p.x = x;
+  p.out = out;
+  p.bias = bias;
+  p.M = M;
+  p.Ncols = nImages * g.L;
+  p.mTiles = pl.mTiles;
+  p.xBytes = (int)((long)nImages * g.Cin * g.H * g.W * sizeof(float));
+  p.vecA = (g.K % 4 == 0) && launch::aligned16(w);
+  p.nSplit = 1;
+  p.ktPerSplit = launch::ceilDiv(g.K, BK);
+  if (pl.full > 0) {
+    convFwdImplicitKernel<<<dim3(pl.full), dev::kBlock, 0, s>>>(p, g);
+    THC_HIP_CHECK(hipGetLastError());
+  }
+  if (pl.tail > 0) {
+    p.tile0 = pl.full;
+    p.ktPerSplit = pl.ktPerSplit;
+    p.nSplit = pl.nSplit;
+    p.partial = partial;
+    convFwdImplicitKernel<<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, g);
+    THC_HIP_CHECK(hipGetLastError());
+    fwdTailFixupKernel<<<dim3(pl.tail, BM * BN / (4 * dev::kBlock)), dev::kBlock, 0, s>>>(p, g);
+    THC_HIP_CHECK(hipGetLastError());
+  }
+}
+
+// Scratch of `floats` floats: the caller's buffer tensor (resized) or a stream-ordered temporary.
+float *scratchFloats(THCState *state, THCudaTensor *buffer, long floats, Temp &tmp, const char *name) {
+  if (floats <= 0) return nullptr;
+  if (buffer) {
+    resize(state, buffer, {floats});
+    if (!isContiguous(erase(buffer))) error("%s tensor has to be contiguous", name);
+    return data(buffer);
+  }
+  tmp = Temp(state->stream, (size_t)floats * sizeof(float));
+  return (float *)tmp.get();
+}
+
 }  // namespace
 
 extern "C" {
@@ -470,8 +808,7 @@ void THNN_CudaSpatialConvolutionMM_updateOutput(THCState *state, THCudaTensor *i
                                                 THCudaTensor *ones, int kW, int kH, int dW, int dH, int padW,
                                                 int padH) {
   THNN_ENTER
-  (void)columns;  // the implicit-im2col GEMM needs neither buffer; both are left untouched
-  (void)ones;
+  (void)ones;  // never read; `columns` is used (and resized) only as scratch for K-split tail tiles
   THC_ARG_CHECK(output != nullptr, 3, "output tensor expected");
   ConvCall call = convSetup(input, nullptr, weight, bias, "weight", kH, kW, dH, dW, padH, padW);
   ConvGeom &g = call.g;
@@ -485,7 +822,21 @@ void THNN_CudaSpatialConvolutionMM_updateOutput(THCState *state, THCudaTensor *i
   hipStream_t s = state->stream;
   // images per launch so that the flat column index n*L + l fits an int
   int group = (int)std::min<long>(g.N, std::max<long>(1, 0x7fffffffL / 2 / g.L));
-  for (int n0 = 0; n0 < g.N; n0 += group) {
+  const long imgBytes = (long)g.Cin * g.H * g.W * sizeof(float);
+  const bool implicit2 = !forceGeneric() && imgBytes < (1L << 30);
+  if (implicit2) group = (int)std::min<long>(group, std::max<long>(1, ((1L << 31) - 1 - 4096) / imgBytes));
+  if (implicit2) {
+    FwdPlan pl = planFwdImplicit(g.Cout, std::min(group, g.N), g);
+    Temp tmp;
+    float *partial = scratchFloats(state, columns, pl.scratchFloats, tmp, "columns");
+    for (int n0 = 0; n0 < g.N; n0 += group) {
+      int cnt = std::min(group, g.N - n0);
+      if (cnt != std::min(group, g.N)) pl = planFwdImplicit(g.Cout, cnt, g);  // last, smaller group: needs no more scratch
+      launchFwdImplicit(s, pl, partial, data(weight), in.ptr() + (long)n0 * g.Cin * g.H * g.W,
+                        data(output) + (long)n0 * g.Cout * g.L, bias ? data(bias) : nullptr, g.Cout, cnt, g);
+    }
+  }
+  for (int n0 = 0; !implicit2 && n0 < g.N; n0 += group) {
     int cnt = std::min(group, g.N - n0);
     GemmArgs p{};
     p.a = data(weight);
@@ -524,6 +875,35 @@ void THNN_CudaSpatialConvolutionMM_updateGradInput(THCState *state, THCudaTensor
   if (!isContiguous(erase(gradInput))) error("gradInput tensor has to be contiguous");
   if ((long)g.N * g.Cin == 0) return;
   hipStream_t s = state->stream;
+  // Stride 1: gradInput is a forward convolution of gradOutput with the flipped,
+  // transposed weights and padding k-1-pad, so it runs on the implicit-GEMM
+  // forward kernel and no gradient columns ever reach memory.
+  const long goImgBytes = (long)g.Cout * g.L * sizeof(float);
+  if (g.dH == 1 && g.dW == 1 && g.padH <= g.kH - 1 && g.padW <= g.kW - 1 && !forceGeneric() &&
+      goImgBytes < (1L << 30)) {
+    ConvGeom t = g;  // the transposed problem
+    t.Cin = g.Cout, t.Cout = g.Cin;
+    t.H = g.oH, t.W = g.oW, t.oH = g.H, t.oW = g.W;
+    t.padH = g.kH - 1 - g.padH, t.padW = g.kW - 1 - g.padW;
+    t.K = g.Cout * g.kH * g.kW;
+    t.L = g.H * g.W;
+    int group = (int)std::min<long>(g.N, std::max<long>(1, 0x7fffffffL / 2 / t.L));
+    group = (int)std::min<long>(group, std::max<long>(1, ((1L << 31) - 1 - 4096) / goImgBytes));
+    FwdPlan pl = planFwdImplicit(t.Cout, std::min(group, g.N), t);
+    const long wfFloats = ((long)g.Cout * g.K + 3) / 4 * 4;
+    Temp tmp;
+    float *buf = scratchFloats(state, gradColumns, wfFloats + pl.scratchFloats, tmp, "gradColumns");
+    flipWeightKernel<<<launch::directGrid((long)g.Cout * g.K, dev::kBlock), dev::kBlock, 0, s>>>(data(weight), buf, g.Cout,
+                                                                                                g.Cin, g.kH, g.kW);
+    THC_HIP_CHECK(hipGetLastError());
+    for (int n0 = 0; n0 < g.N; n0 += group) {
+      int cnt = std::min(group, g.N - n0);
+      if (cnt != std::min(group, g.N)) pl = planFwdImplicit(t.Cout, cnt, t);
+      launchFwdImplicit(s, pl, buf + wfFloats, buf, go.ptr() + (long)n0 * g.Cout * g.L,
+                        data(gradInput) + (long)n0 * g.Cin * g.H * g.W, nullptr, t.Cout, cnt, t);
+    }
+    return;
+  }
   // gradient columns of a group of images at a time (<= 64 MB so the buffer stays cache resident)
   const long perImg = (long)g.K * g.L;
   int group = (int)std::max<long>(1, std::min<long>(g.N, (64L << 20) / 4 / perImg));
@@ -577,12 +957,17 @@ void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTens
   if ((long)g.N * g.Cout * g.K == 0) return;
   hipStream_t s = state->stream;
 
-  // split the reduction over groups of images until the grid fills the chip
+  // Split the reduction over the N*L positions so that the grid fills the
+  // resident workgroup slots of the chip exactly once: with fewer, fatter
+  // splits some CUs would carry one workgroup more than others for the whole
+  // kernel.
+  if ((long)g.N * g.L >= 0x7fffffffL) error("SpatialConvolutionMM: batch too large");
   const int mT = (int)tiles(g.Cout, BM), nT = (int)tiles(g.K, BN);
-  int splits = (int)std::min<long>(g.N, std::max<long>(1, (2 * 256 + mT * nT - 1) / (mT * nT)));
-  int perSplit = launch::ceilDiv(g.N, splits);
-  perSplit = (int)std::min<long>(perSplit, std::max<long>(1, 0x7fffffffL / 2 / g.L));
-  splits = launch::ceilDiv(g.N, perSplit);
+  const int totalKt = launch::ceilDiv(g.N * g.L, BK);
+  const int slots = residentSlots((const void *)convGemmKernel<kGradWeight>);
+  int splits = std::max(1, std::min(totalKt, slots / (mT * nT)));
+  const int perSplit = launch::ceilDiv(totalKt, splits);
+  splits = launch::ceilDiv(totalKt, perSplit);
   const long count = (long)g.Cout * g.K;
   Temp tmp;
   float *partial;
@@ -612,7 +997,10 @@ void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTens
                                                                                    splits, scale);
   THC_HIP_CHECK(hipGetLastError());
   if (gradBias) {
-    gradBiasKernel<<<g.Cout, dev::kBlock, 0, s>>>(go.ptr(), data(gradBias), g.N, g.Cout, g.L, scale);
+    if (g.L % 4 == 0 && launch::aligned16(go.ptr()) && (long)g.N * (g.L / 4) < 0x7fffffffL)
+      gradBiasKernel<true><<<g.Cout, kBiasBlock, 0, s>>>(go.ptr(), data(gradBias), g.N, g.Cout, g.L, scale);
+    else
+      gradBiasKernel<false><<<g.Cout, kBiasBlock, 0, s>>>(go.ptr(), data(gradBias), g.N, g.Cout, g.L, scale);
     THC_HIP_CHECK(hipGetLastError());
   }
   THNN_LEAVE

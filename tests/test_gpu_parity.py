@@ -419,6 +419,10 @@ CONV_CASES = [
     (5, 1, 16, 19, 19, 5, 5, 2, 2, 0, 0),
     (3, 130, 136, 9, 9, 3, 3, 1, 1, 1, 1),   # Cout, K not multiples of the GEMM tile
     (2, 8, 200, 16, 16, 1, 1, 1, 1, 0, 0),
+    (5, 16, 8, 83, 83, 3, 3, 1, 1, 1, 1),    # more tiles than CUs: the last round is split along K
+    (3, 6, 10, 15, 17, 5, 3, 1, 1, 2, 0),    # rectangular kernel, stride 1: gradInput through the forward kernel
+    (2, 4, 6, 9, 9, 1, 1, 1, 1, 1, 1),       # pad > k-1: gradInput through gradient columns + col2im
+    (2, 8, 12, 70, 70, 3, 3, 1, 1, 1, 1),
 ]
 
 
@@ -456,6 +460,15 @@ def _conv_run(T, case, bias=True, weight4d=False, xt=None, scale=1.0, seed=50):
 @pytest.mark.parametrize("case", CONV_CASES)
 def test_convmm(T, case):
     _conv_run(T, case)
+
+
+def test_convmm_first_generation_kernels(T):
+    os.environ["THCUNN_CONV_FORCE_GENERIC"] = "1"
+    try:
+        _conv_run(T, CONV_CASES[0])
+        _conv_run(T, CONV_CASES[3])
+    finally:
+        os.environ.pop("THCUNN_CONV_FORCE_GENERIC", None)
 
 
 def test_convmm_variants(T):

@@ -38,9 +38,14 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 METRIC = "DW-conv fwd+bwd images/s + achieved HBM GB/s (% of peak), 1 MI355X"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/dwconv_cfg2_pmc.txt gives the runs and the copy-kernel scale factor);
-# None until a counter run exists for that kernel.
-MEASURED_TRAFFIC_BYTES = {}
+# (profiles/dwconv_cfg2_hbm_traffic.txt gives the runs and the copy-kernel scale
+# factors); workloads without a counter run report null.
+_KIB = 1024
+MEASURED_TRAFFIC_BYTES = {
+    ("cfg2", "dw_updateOutput"): int((50252.9 * 2.0 + 25088.0) * _KIB),
+    ("cfg2", "dw_updateGradInput"): int((12631.0 * 2.0 + 100352.0) * _KIB),
+    ("cfg2", "dw_accGradParameters"): int(((62768.0 + 189.0) * 2.0 + 1313.4 + 12.0) * _KIB),
+}
 
 
 class Hip:
@@ -288,7 +293,26 @@ def wl_conv(nsets):
                 desc=f"SpatialConvolutionMM fwd+gradInput+accGradParameters fp32 N={N} Cin={Ci} Cout={Co} {H}x{H} k3 s1 p1 bias")
 
 
-WORKLOADS = {"cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda n: wl_dw("cfg2", n), "cfg3": wl_bn, "cfg4": wl_pool,
+def wl_copy(nsets):
+    """Calibration: plain device-to-device copy of 128 MB (2 x 128 MB of HBM traffic per launch)."""
+    from cunn_amd import CudaTensor as CT
+    n = 32 * 1024 * 1024
+    src = np.arange(n, dtype=np.float32)
+    sets = [dict(a=CT.from_numpy(src), b=CT.with_size(n)) for _ in range(nsets)]
+
+    def calls(i):
+        t = sets[i]
+        return [("copy", lambda: t["b"].copy_from(t["a"]))]
+
+    def verify():
+        sets[0]["b"].copy_from(sets[0]["a"])
+        assert np.array_equal(sets[0]["b"].numpy(), src)
+
+    return dict(calls=calls, work={"copy": (2 * src.nbytes, "bytes")}, images=1, cpu=lambda reps: (1.0, 1, "n/a"),
+                verify=verify, bound="hbm", desc="float4 device-to-device copy of 128 MiB")
+
+
+WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda n: wl_dw("cfg2", n), "cfg3": wl_bn, "cfg4": wl_pool,
              "cfg5": wl_conv}
 
 
@@ -333,7 +357,7 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds):
     res = dict(workload=wl["desc"], images_per_s=wl["images"] / (ms_per_step * 1e-3), ms_per_step=ms_per_step,
                device_ms_per_step=float(sum(kern[n]["avg_ms"] for n in names)), roofline=roofline,
                kernels={n: {k: (round(v, 5) if isinstance(v, float) else v) for k, v in kern[n].items()} for n in names})
-    if cpu_seconds > 0:
+    if cpu_seconds > 0 and name != "copy":
         from oracle import oracle as O
         sec, imgs, sample = wl["cpu"](1)          # calibrate
         reps = max(1, min(50, int(cpu_seconds / max(sec, 1e-3))))
@@ -380,7 +404,7 @@ def main():
     if args.all:
         others = {}
         for name in sorted(WORKLOADS):
-            if name == args.workload:
+            if name == args.workload or name == "copy":
                 continue
             r = run_workload(name, max(20, args.steps // 4), max(5, args.warmup // 2), hip, stream,
                              args.sets, min(args.cpu_seconds, 8.0))

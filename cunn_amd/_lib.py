@@ -64,6 +64,7 @@ SHIM = {  # name: (restype, argtypes)
     "THCudaTensor_nElement": (C.c_ssize_t, [_T, _T]),
     "THCudaTensor_isContiguous": (_i, [_T, _T]),
     "THCudaTensor_fill": (None, [_T, _T, _f]),
+    "THCudaTensor_copy": (None, [_T, _T, _T]),
     "THCudaTensor_copyFromHost": (None, [_T, _T, _T]),
     "THCudaTensor_copyToHost": (None, [_T, _T, _T]),
     "THCudaLongTensor_new": (_T, [_T]),

@@ -256,6 +256,16 @@ Contiguous::Contiguous(THCState *state, const THCudaTensor *t) {
   ptr_ = (const float *)tmp_.get();
 }
 
+// dst[i] = src[i] over n4 float4s (+ tail): the plain streaming copy that bandwidth
+// figures of the other kernels are calibrated against
+__global__ void __launch_bounds__(256) copyKernel(const float *__restrict__ src, float *__restrict__ dst, long n) {
+  const long n4 = n >> 2;
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride)
+    reinterpret_cast<float4 *>(dst)[i] = reinterpret_cast<const float4 *>(src)[i];
+  for (long i = (n4 << 2) + (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) fillKernel(T *p, long n, T v) {
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
@@ -385,6 +395,25 @@ void THCudaTensor_fill(THCState *state, THCudaTensor *self, float value) {
   if (blocks > 16384) blocks = 16384;
   fillKernel<float><<<(unsigned)blocks, 256, 0, state->stream>>>(data(self), n, value);
   THC_HIP_CHECK(hipGetLastError());
+  THNN_LEAVE
+}
+void THCudaTensor_copy(THCState *state, THCudaTensor *self, THCudaTensor *src) {
+  THNN_ENTER
+  Tensor *d = erase(self), *f = erase(src);
+  ptrdiff_t n = numel(d);
+  if (n != numel(f)) error("copy: sizes do not match: %s vs %s", sizeDesc(d).c_str(), sizeDesc(f).c_str());
+  if (n == 0) return;
+  if (isContiguous(d) && isContiguous(f) && ((reinterpret_cast<uintptr_t>(data(self)) | reinterpret_cast<uintptr_t>(data(src))) & 15) == 0) {
+    long blocks = ((n >> 2) + 255) / 256;
+    blocks = blocks < 1 ? 1 : (blocks > 16384 ? 16384 : blocks);
+    copyKernel<<<(unsigned)blocks, 256, 0, state->stream>>>(data(src), data(self), n);
+    THC_HIP_CHECK(hipGetLastError());
+  } else {
+    // through a packed temporary: gather src, scatter into self
+    Temp tmp(state->stream, (size_t)n * sizeof(float));
+    stridedCopy(state->stream, f, tmp.get(), sizeof(float), true);
+    stridedCopy(state->stream, d, tmp.get(), sizeof(float), false);
+  }
   THNN_LEAVE
 }
 void THCudaTensor_copyFromHost(THCState *state, THCudaTensor *self, const float *src) {

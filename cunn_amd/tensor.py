@@ -178,6 +178,12 @@ class CudaTensor(_Base):
         check()
         return self
 
+    def copy_from(self, other):
+        """Device-to-device copy of another CudaTensor with the same number of elements."""
+        self._lib.THCudaTensor_copy(state(), self._h, other._h)
+        check()
+        return self
+
     def view(self, offset, size, stride):
         """A strided view sharing this tensor's storage (narrow/select/transpose by hand)."""
         sz, n = _longs(size)

@@ -119,6 +119,7 @@ long THCudaTensor_stride(THCState *state, const THCudaTensor *self, int dim);
 ptrdiff_t THCudaTensor_nElement(THCState *state, const THCudaTensor *self);
 int THCudaTensor_isContiguous(THCState *state, const THCudaTensor *self);
 void THCudaTensor_fill(THCState *state, THCudaTensor *self, float value);
+void THCudaTensor_copy(THCState *state, THCudaTensor *self, THCudaTensor *src); /* device to device, same nElement */
 /* host <-> device copies of the logical (size-ordered) contents; synchronous */
 void THCudaTensor_copyFromHost(THCState *state, THCudaTensor *self, const float *src);
 void THCudaTensor_copyToHost(THCState *state, THCudaTensor *self, float *dst);

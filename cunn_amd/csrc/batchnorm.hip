@@ -319,23 +319,6 @@ bnBackwardKernel(const float *__restrict__ x, const float *__restrict__ gy, floa
 constexpr int kResBlock = 1024;
 constexpr int kResWaves = kResBlock / dev::kWave;
 
-// Buffer-addressed 16-byte accesses: the channel base lives in a scalar
-// resource descriptor and each access carries only a 32-bit byte offset, so
-// the unrolled R-deep load/store sequences do not tie up a 64-bit address
-// register pair per access.
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t makeRsrc(const float *base, long bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)bytes, 0x00020000);
-}
-__device__ __forceinline__ float4 bufLoad4(__amdgpu_buffer_rsrc_t r, int byteOff) {
-  u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byteOff, 0, 0);
-  return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
-}
-__device__ __forceinline__ void bufStore4(__amdgpu_buffer_rsrc_t r, int byteOff, float4 f) {
-  u32x4 v = {__float_as_uint(f.x), __float_as_uint(f.y), __float_as_uint(f.z), __float_as_uint(f.w)};
-  __builtin_amdgcn_raw_buffer_store_b128(v, r, byteOff, 0, 0);
-}
-
 __device__ __forceinline__ float blockSum1024(float v, float *red) {
   const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
   v = dev::waveSum(v);
@@ -384,14 +367,14 @@ bnFwdResident(const float *__restrict__ x, float *__restrict__ y, const float *_
   const int ch = blockIdx.x;
   const int total4 = N * (L >> 2);
   const long span = ((long)(N - 1) * C * L + L) * 4;  // bytes from the channel's first to past its last element
-  const __amdgpu_buffer_rsrc_t xr = makeRsrc(x + (long)ch * L, span), yr = makeRsrc(y + (long)ch * L, span);
+  const __amdgpu_buffer_rsrc_t xr = dev::makeRsrc(x + (long)ch * L, span), yr = dev::makeRsrc(y + (long)ch * L, span);
   float4 v[R];
   {
     ResWalker wk(L, C);
 #pragma unroll
     for (int u = 0; u < R; ++u) {
       v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (u * kResBlock + (int)threadIdx.x < total4) v[u] = bufLoad4(xr, wk.offset());
+      if (u * kResBlock + (int)threadIdx.x < total4) v[u] = dev::bufLoad4(xr, wk.offset());
       wk.next();
     }
   }
@@ -427,7 +410,7 @@ bnFwdResident(const float *__restrict__ x, float *__restrict__ y, const float *_
       r.y = gamma * (v[u].y - mean) * invStd + beta;
       r.z = gamma * (v[u].z - mean) * invStd + beta;
       r.w = gamma * (v[u].w - mean) * invStd + beta;
-      bufStore4(yr, wk.offset(), r);
+      dev::bufStore4(yr, wk.offset(), r);
     }
     wk.next();
   }
@@ -450,8 +433,8 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
   const float stdVal = TRAIN ? stdSrc[ch] : 1.f / sqrtf(stdSrc[ch] + eps);
   const float weightVal = weight ? weight[ch] : 1.f;
   const long span = ((long)(N - 1) * C * L + L) * 4;
-  const __amdgpu_buffer_rsrc_t xr = makeRsrc(x + (long)ch * L, span), gr = makeRsrc(gy + (long)ch * L, span);
-  const __amdgpu_buffer_rsrc_t or_ = makeRsrc(gx ? gx + (long)ch * L : x, gx ? span : 0);
+  const __amdgpu_buffer_rsrc_t xr = dev::makeRsrc(x + (long)ch * L, span), gr = dev::makeRsrc(gy + (long)ch * L, span);
+  const __amdgpu_buffer_rsrc_t or_ = dev::makeRsrc(gx ? gx + (long)ch * L : x, gx ? span : 0);
   float4 d[R], xc[KEEPX ? R : 1];
   float s0 = 0.f, s1 = 0.f;
   {
@@ -463,8 +446,8 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
         xc[KEEPX ? u : 0] = make_float4(mean, mean, mean, mean);
         if (u * kResBlock + (int)threadIdx.x < total4) {
           const int off = wk.offset();
-          d[u] = bufLoad4(gr, off);
-          xc[KEEPX ? u : 0] = bufLoad4(xr, off);
+          d[u] = dev::bufLoad4(gr, off);
+          xc[KEEPX ? u : 0] = dev::bufLoad4(xr, off);
         }
         wk.next();
       }
@@ -481,7 +464,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
 #pragma unroll
       for (int u = 0; u < R; ++u) {
         d[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (u * kResBlock + (int)threadIdx.x < total4) d[u] = bufLoad4(gr, wk.offset());
+        if (u * kResBlock + (int)threadIdx.x < total4) d[u] = dev::bufLoad4(gr, wk.offset());
         wk.next();
       }
 #pragma unroll
@@ -491,7 +474,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
         for (int k = 0; k < 4; ++k) {
           q[k] = make_float4(mean, mean, mean, mean);
           if (u0 + k < R) {
-            if ((u0 + k) * kResBlock + (int)threadIdx.x < total4) q[k] = bufLoad4(xr, wx.offset());
+            if ((u0 + k) * kResBlock + (int)threadIdx.x < total4) q[k] = dev::bufLoad4(xr, wx.offset());
             wx.next();
           }
         }
@@ -528,7 +511,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
           } else {
             r.x = d[u].x * gradScale, r.y = d[u].y * gradScale, r.z = d[u].z * gradScale, r.w = d[u].w * gradScale;
           }
-          bufStore4(or_, wk.offset(), r);
+          dev::bufStore4(or_, wk.offset(), r);
         }
         wk.next();
       }
@@ -544,7 +527,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
           if (u0 + k < R) {
             if ((u0 + k) * kResBlock + (int)threadIdx.x < total4) {
               off[k] = wk.offset();
-              q[k] = bufLoad4(xr, off[k]);
+              q[k] = dev::bufLoad4(xr, off[k]);
             }
             wk.next();
           }
@@ -558,7 +541,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
             r.y = (g4.y - (q[k].y - mean) * projScale - gradMean) * gradScale;
             r.z = (g4.z - (q[k].z - mean) * projScale - gradMean) * gradScale;
             r.w = (g4.w - (q[k].w - mean) * projScale - gradMean) * gradScale;
-            bufStore4(or_, off[k], r);
+            dev::bufStore4(or_, off[k], r);
           }
         __asm__ volatile("" ::: "memory");
       }

@@ -44,6 +44,33 @@ __device__ __forceinline__ int xcdRemap(int bid, int nblk) {
   return xcd * q + (xcd < r ? xcd : r) + idx;
 }
 
+// Division of a non-negative int by a positive runtime divisor d through its
+// reciprocal magic = floor(2^32 / d) + 1 (magicOf): exact while i * d < 2^32, which
+// holds for every in-tile index here. A few integer instructions instead of the
+// ~25 of a generic 32-bit division. d == 1 has no 32-bit magic (it would be 2^32)
+// and is encoded as 0.
+__host__ __device__ __forceinline__ unsigned magicOf(int d) { return d == 1 ? 0u : 0xFFFFFFFFu / (unsigned)d + 1u; }
+__device__ __forceinline__ int fastDiv(int i, unsigned magic) {
+  return magic ? (int)__umulhi((unsigned)i, magic) : i;
+}
+
+// Buffer-addressed 16-byte accesses: the base lives in a scalar resource
+// descriptor, an access carries a 32-bit byte offset, and an offset at or beyond
+// the descriptor's size reads as 0 - out-of-image elements need no branch.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kBufOob = 0x7fffffff;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t makeRsrc(const void *base, long bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ float4 bufLoad4(__amdgpu_buffer_rsrc_t r, int byteOff) {
+  u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byteOff, 0, 0);
+  return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+}
+__device__ __forceinline__ void bufStore4(__amdgpu_buffer_rsrc_t r, int byteOff, float4 f) {
+  u32x4 v = {__float_as_uint(f.x), __float_as_uint(f.y), __float_as_uint(f.z), __float_as_uint(f.w)};
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, byteOff, 0, 0);
+}
+
 __device__ __forceinline__ int ceilDivPos(int a, int b) {  // ceil(a / b) for b > 0, any sign of a
   return (a >= 0) ? (a + b - 1) / b : -((-a) / b);
 }
@@ -71,17 +98,20 @@ __device__ __forceinline__ void loadRowsPadded(float *__restrict__ dst, const fl
   if (VEC) {
     const int W4 = W >> 2;
     const int total = nRows * W4;
+    const unsigned magic = magicOf(W4);
+    const __amdgpu_buffer_rsrc_t rs = makeRsrc(plane, (long)H * W * 4);
     for (int base = 0; base < total; base += kLoadBatch * nt) {
       float4 v[kLoadBatch];
       int off[kLoadBatch];
 #pragma unroll
       for (int u = 0; u < kLoadBatch; ++u) {
-        int i = base + u * nt + tid;
-        int r = i / W4, c4 = i - r * W4;
-        int gr = r0 + r;
+        const int i = base + u * nt + tid;
+        const int r = fastDiv(i, magic), c4 = i - r * W4;
+        const int gr = r0 + r;
+        const bool ok = i < total && (unsigned)gr < (unsigned)H;
         off[u] = (i < total) ? r * pitch + padL + (c4 << 2) : -1;
-        v[u] = make_float4(fill, fill, fill, fill);
-        if (i < total && gr >= 0 && gr < H) v[u] = reinterpret_cast<const float4 *>(plane + (long)gr * W)[c4];
+        v[u] = bufLoad4(rs, ok ? (gr * W + (c4 << 2)) * 4 : kBufOob);
+        if (fill != 0.f && !ok) v[u] = make_float4(fill, fill, fill, fill);
       }
 #pragma unroll
       for (int u = 0; u < kLoadBatch; ++u)
@@ -121,14 +151,11 @@ __device__ __forceinline__ void loadFlat(T *__restrict__ dst, const T *__restric
   const int tid = threadIdx.x, nt = blockDim.x;
   if (VEC && sizeof(T) == 4) {
     const int n4 = count >> 2;
+    const __amdgpu_buffer_rsrc_t rs = makeRsrc(src, (long)count * 4);
     for (int base = 0; base < n4; base += kLoadBatch * nt) {
       float4 v[kLoadBatch];
 #pragma unroll
-      for (int u = 0; u < kLoadBatch; ++u) {
-        int i = base + u * nt + tid;
-        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (i < n4) v[u] = reinterpret_cast<const float4 *>(src)[i];
-      }
+      for (int u = 0; u < kLoadBatch; ++u) v[u] = bufLoad4(rs, (base + u * nt + tid) * 16);  // past the end reads 0
 #pragma unroll
       for (int u = 0; u < kLoadBatch; ++u) {
         int i = base + u * nt + tid;
@@ -166,17 +193,20 @@ __device__ __forceinline__ void loadRowsSplit(float *__restrict__ dst, const flo
   const int W4 = W >> 2;
   const int oddOff = (W >> 1) + 8;
   const int total = nRows * W4;
+  const unsigned magic = magicOf(W4);
+  const __amdgpu_buffer_rsrc_t rs = makeRsrc(plane, (long)H * W * 4);
   for (int base = 0; base < total; base += kLoadBatch * nt) {
     float4 v[kLoadBatch];
     int off[kLoadBatch];
 #pragma unroll
     for (int u = 0; u < kLoadBatch; ++u) {
-      int i = base + u * nt + tid;
-      int r = i / W4, c4 = i - r * W4;
-      int gr = r0 + r;
+      const int i = base + u * nt + tid;
+      const int r = fastDiv(i, magic), c4 = i - r * W4;
+      const int gr = r0 + r;
+      const bool ok = i < total && (unsigned)gr < (unsigned)H;
       off[u] = (i < total) ? r * pitch + 4 + (c4 << 1) : -1;
-      v[u] = make_float4(fill, fill, fill, fill);
-      if (i < total && gr >= 0 && gr < H) v[u] = reinterpret_cast<const float4 *>(plane + (long)gr * W)[c4];
+      v[u] = bufLoad4(rs, ok ? (gr * W + (c4 << 2)) * 4 : kBufOob);
+      if (fill != 0.f && !ok) v[u] = make_float4(fill, fill, fill, fill);
     }
 #pragma unroll
     for (int u = 0; u < kLoadBatch; ++u)

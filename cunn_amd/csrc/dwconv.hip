@@ -20,6 +20,13 @@ using namespace thc;
 
 namespace {
 
+struct Strides4 {
+  long s0, s1, s2, s3;
+};
+struct Strides2 {
+  long s0, s1;
+};
+
 struct DwGeom {
   int N, C, M, H, W, oH, oW;
   int kH, kW, dH, dW, padH, padW;
@@ -28,14 +35,39 @@ struct DwGeom {
   int pitch, padL;    // LDS row pitch / left zero pad of the staged input band
   int nblk;           // grid size
   int nslots;         // N * tilesPerPlane (accGradParameters partials per (c,j) and tap)
+  unsigned magicTiles, magicC;  // dev::magicOf(tilesPerPlane), dev::magicOf(C): used by the strip kernels
 };
 
-struct Strides4 {
-  long s0, s1, s2, s3;
+// (plane, tile, channel) of a workgroup of the strip kernels
+struct BlockPos {
+  int plane, tile, c;
 };
-struct Strides2 {
-  long s0, s1;
-};
+__device__ __forceinline__ BlockPos blockPos(const DwGeom &g) {
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  BlockPos b;
+  b.plane = g.tilesPerPlane == 1 ? bid : dev::fastDiv(bid, g.magicTiles);
+  b.tile = bid - b.plane * g.tilesPerPlane;
+  b.c = b.plane - dev::fastDiv(b.plane, g.magicC) * g.C;
+  return b;
+}
+
+// The KS*KS taps of (multiplier j, channel c) into registers; one wide scalar
+// load when the kernel plane is contiguous.
+template <int KS>
+__device__ __forceinline__ void loadTaps(const float *__restrict__ weight, const Strides4 &ws, int j, int c,
+                                         float (&w)[KS * KS]) {
+  const float *wp = weight + j * ws.s0 + c * ws.s1;
+  if (ws.s3 == 1 && ws.s2 == KS) {
+#pragma unroll
+    for (int t = 0; t < KS * KS; ++t) w[t] = wp[t];
+  } else {
+#pragma unroll
+    for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+      for (int kw = 0; kw < KS; ++kw) w[kh * KS + kw] = wp[kh * ws.s2 + kw * ws.s3];
+  }
+}
+
 
 // ------------------------------------------------------------------ forward --
 // KS/ST > 0: square kernel / stride known at compile time (taps in registers,
@@ -353,9 +385,8 @@ dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strid
   using S = dev::Strip<KS, ST, KS / 2>;
   constexpr int PAD = KS / 2, NW = S::NW;
   extern __shared__ float smem[];
-  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
-  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
-  const int c = plane % g.C;
+  const BlockPos bp = blockPos(g);
+  const int plane = bp.plane, tile = bp.tile, c = bp.c;
   const int oh0 = tile * g.tileRows;
   const int nOut = min(g.tileRows, g.oH - oh0);
   const int nIn = (nOut - 1) * ST + KS;
@@ -363,17 +394,15 @@ dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strid
   S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
   __syncthreads();
   const int oW4 = g.oW >> 2;
+  const unsigned magicOw4 = dev::magicOf(oW4);
   const int total = nOut * oW4;
   for (int j = 0; j < g.M; ++j) {
     float w[KS * KS];
-#pragma unroll
-    for (int kh = 0; kh < KS; ++kh)
-#pragma unroll
-      for (int kw = 0; kw < KS; ++kw) w[kh * KS + kw] = weight[j * ws.s0 + c * ws.s1 + kh * ws.s2 + kw * ws.s3];
+    loadTaps<KS>(weight, ws, j, c, w);
     const float b = bias ? bias[j * bs.s0 + c * bs.s1] : 0.f;
     float *o = out + (((long)plane * g.M + j) * g.oH + oh0) * g.oW;
     for (int i = threadIdx.x; i < total; i += blockDim.x) {
-      const int r = i / oW4, b4 = i - r * oW4;
+      const int r = dev::fastDiv(i, magicOw4), b4 = i - r * oW4;
       const float *p = smem + r * ST * pitch;
       float acc[4] = {b, b, b, b};
 #pragma unroll
@@ -406,9 +435,8 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
   constexpr int OFF = ((dev::kStripPadL + QW0) % 4 + 4) % 4;
   constexpr int ALIGN = (CPB % 4 == 0) ? 4 : 2;
   extern __shared__ float smem[];
-  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
-  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
-  const int c = plane % g.C;
+  const BlockPos bp = blockPos(g);
+  const int plane = bp.plane, tile = bp.tile, c = bp.c;
   const int h0 = tile * g.tileRows;  // multiple of ST
   const int nRows = min(g.tileRows, g.H - h0);
   const int pitch = g.oW + dev::kStripPadL;
@@ -419,11 +447,12 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
                               dev::kStripPadL);
   __syncthreads();
   const int W4 = g.W >> 2;
+  const unsigned magicW4 = dev::magicOf(W4);
   const int nA = (nRows + ST - 1) / ST;
   const int total = nA * W4;
   float *o = gradIn + ((long)plane * g.H + h0) * g.W;
   for (int i = threadIdx.x; i < total; i += blockDim.x) {
-    const int a = i / W4, b = i - a * W4;
+    const int a = dev::fastDiv(i, magicW4), b = i - a * W4;
     float acc[ST][4];
 #pragma unroll
     for (int dy = 0; dy < ST; ++dy)
@@ -431,10 +460,7 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
       for (int dx = 0; dx < 4; ++dx) acc[dy][dx] = 0.f;
     for (int j = 0; j < g.M; ++j) {
       float w[KS * KS];
-#pragma unroll
-      for (int kh = 0; kh < KS; ++kh)
-#pragma unroll
-        for (int kw = 0; kw < KS; ++kw) w[kh * KS + kw] = weight[j * ws.s0 + c * ws.s1 + kh * ws.s2 + kw * ws.s3];
+      loadTaps<KS>(weight, ws, j, c, w);
       const float *gj = smem + (size_t)j * (stageRows * pitch + dev::kStripPadL) + dev::kStripPadL + QW0 + b * CPB;
 #pragma unroll
       for (int qh = QH0; qh <= QH1; ++qh) {
@@ -474,9 +500,9 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
   constexpr int nWaves = dev::kBlock / dev::kWave;
   extern __shared__ float smem[];
   __shared__ float red[nWaves][T];
-  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
-  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
-  const int n = plane / g.C, c = plane - n * g.C;
+  const BlockPos bp = blockPos(g);
+  const int plane = bp.plane, tile = bp.tile, c = bp.c;
+  const int n = dev::fastDiv(plane, g.magicC);
   const int oh0 = tile * g.tileRows;
   const int nOut = min(g.tileRows, g.oH - oh0);
   const int nIn = (nOut - 1) * ST + KS;
@@ -484,6 +510,7 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
   float *gs = smem + S::floats((g.tileRows - 1) * ST + KS, g.W);  // multiple of 4 floats
   S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
   const int oW4 = g.oW >> 2;
+  const unsigned magicOw4 = dev::magicOf(oW4);
   const int total = nOut * oW4;
   const int slot = n * g.tilesPerPlane + tile;
   const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
@@ -495,7 +522,7 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
 #pragma unroll
     for (int t = 0; t < T; ++t) acc[t] = 0.f;
     for (int i = threadIdx.x; i < total; i += blockDim.x) {
-      const int r = i / oW4, b4 = i - r * oW4;
+      const int r = dev::fastDiv(i, magicOw4), b4 = i - r * oW4;
       const float *p = smem + r * ST * pitch;
       const float4 gy4 = *reinterpret_cast<const float4 *>(gs + r * g.oW + b4 * 4);
       const float gy[4] = {gy4.x, gy4.y, gy4.z, gy4.w};
@@ -603,6 +630,7 @@ DwCall dwSetup(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, T
   g.oH = (g.H + 2 * padH - kH) / dH + 1;
   g.oW = (g.W + 2 * padW - kW) / dW + 1;
   g.tileRows = g.tilesPerPlane = g.pitch = g.padL = g.nblk = g.nslots = 0;
+  g.magicTiles = g.magicC = 0;
   return call;
 }
 
@@ -728,10 +756,12 @@ void THNN_CudaSpatialDepthWiseConvolution_updateOutput(THCState *state, THCudaTe
   };
   if (stripGeometry(g) && vec && aligned16(data(output))) {
     auto sbytes = [&](int rows) { return stripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
-    if (launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane)) {
+    auto staged = [&](int rows) { return (size_t)((rows - 1) * g.dH + g.kH) * g.W; };
+    if (launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane, staged)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
       size_t lds = sbytes(g.tileRows);
       dim3 grid(g.nblk), block(dev::kBlock);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane), g.magicC = dev::magicOf(g.C);
       DW_STRIP_DISPATCH(dwFwdStrip, in.ptr(), data(weight), strides4(weight), bptr, strides2(bias), data(output), g);
       THC_HIP_CHECK(hipGetLastError());
       return;
@@ -791,6 +821,7 @@ void THNN_CudaSpatialDepthWiseConvolution_updateGradInput(THCState *state, THCud
       g.nblk = (int)(planes * g.tilesPerPlane);
       size_t lds = sbytes(units);
       dim3 grid(g.nblk), block(dev::kBlock);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane), g.magicC = dev::magicOf(g.C);
       DW_STRIP_DISPATCH(dwGradInputStrip, go.ptr(), data(weight), strides4(weight), data(gradInput), g, units + extra);
       THC_HIP_CHECK(hipGetLastError());
       return;
@@ -844,7 +875,8 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
                            : (size_t)roundUp(((rows - 1) * g.dH + g.kH) * g.pitch + g.padL, 4);
     return (band + (size_t)rows * g.oW) * sizeof(float);
   };
-  if (haveKernel && !forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
+  auto staged = [&](int rows) { return useStrip ? (size_t)((rows - 1) * g.dH + g.kH) * g.W : (size_t)0; };
+  if (haveKernel && !forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane, staged)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
     g.nslots = g.N * g.tilesPerPlane;
     size_t lds = bytes(g.tileRows);
@@ -867,6 +899,7 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
     bool vecg = aligned16(go.ptr()) && (g.oW % 4 == 0 || (g.tilesPerPlane == 1 && ((long)g.oH * g.oW) % 4 == 0));
     if (useStrip) {
       dim3 grid(g.nblk), block(dev::kBlock);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane), g.magicC = dev::magicOf(g.C);
       DW_STRIP_DISPATCH(dwAccGradStrip, in.ptr(), go.ptr(), partial, g);
     } else {
       if (ks == 3 && st == 1) launchAcc1<3, 1>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);

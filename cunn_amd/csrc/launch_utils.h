@@ -23,11 +23,24 @@ inline int ceilDiv(int a, int b) { return (a + b - 1) / b; }
 // Splits `produced` rows of a plane into equal bands. bytes(rows) is the LDS a
 // band of that many rows needs. Returns false when a one-row band exceeds the
 // LDS limit or the grid would not fit an int.
-template <typename BytesFn>
-bool pickBand(int produced, long planes, BytesFn bytes, int *tileRows, int *tilesPerPlane) {
+//
+// The staging loaders keep kLoadBatch 16-byte loads per lane in flight; a band
+// that needs one load more than a whole number of batches pays a full extra
+// memory round trip for it. stagedFloats(rows) (optional) is the number of
+// floats a band stages: bands are shrunk until they fit one batch of a
+// 256-lane workgroup (4096 floats) when that still leaves >= 4 rows.
+constexpr int kBatchFloats = 4 * 4 * 256;
+
+template <typename BytesFn, typename StagedFn>
+bool pickBand(int produced, long planes, BytesFn bytes, int *tileRows, int *tilesPerPlane, StagedFn stagedFloats) {
   if (produced < 1 || bytes(1) > kLdsMax) return false;
   int rows = produced;
   while (rows > 1 && bytes(rows) > kLdsBudget) rows = (rows + 1) / 2;
+  {
+    int r = rows;
+    while (r > 4 && stagedFloats(r) > (size_t)kBatchFloats) --r;
+    if (stagedFloats(r) <= (size_t)kBatchFloats) rows = r;
+  }
   while (rows > 4 && planes * ceilDiv(produced, rows) < kMinBlocks) rows = (rows + 1) / 2;
   int t = ceilDiv(produced, rows);
   rows = ceilDiv(produced, t);
@@ -35,6 +48,11 @@ bool pickBand(int produced, long planes, BytesFn bytes, int *tileRows, int *tile
   *tileRows = rows;
   *tilesPerPlane = t;
   return true;
+}
+
+template <typename BytesFn>
+bool pickBand(int produced, long planes, BytesFn bytes, int *tileRows, int *tilesPerPlane) {
+  return pickBand(produced, planes, bytes, tileRows, tilesPerPlane, [](int) { return (size_t)0; });
 }
 
 inline unsigned directGrid(long total, int block) {

@@ -25,7 +25,16 @@ struct PoolGeom {
   int kH, kW, dH, dW, padH, padW, dilH, dilW;
   int tileRows, tilesPerPlane, nblk;
   int maxStageRows;  // rows of the staged tensor per band (upper bound)
+  unsigned magicTiles;  // dev::magicOf(tilesPerPlane), used by the strip kernels
+  int constDiv;         // average pooling: every window has the divisor kH*kW (no window is clipped)
 };
+
+// (plane, tile) of a workgroup of the strip kernels
+__device__ __forceinline__ void blockPos(const PoolGeom &g, int &plane, int &tile) {
+  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  plane = g.tilesPerPlane == 1 ? bid : dev::fastDiv(bid, g.magicTiles);
+  tile = bid - plane * g.tilesPerPlane;
+}
 
 // ----------------------------------------------------------- max: forward ----
 template <int KS, int ST, bool VEC>
@@ -307,8 +316,8 @@ maxPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, long *__r
   using S = dev::Strip<KS, ST, PAD>;
   constexpr int NW = S::NW;
   extern __shared__ float smem[];
-  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
-  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  int plane, tile;
+  blockPos(g, plane, tile);
   const int ph0 = tile * g.tileRows;
   const int nOut = min(g.tileRows, g.oH - ph0);
   const int nIn = (nOut - 1) * ST + KS;
@@ -316,10 +325,11 @@ maxPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, long *__r
   S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, ph0 * ST - PAD, nIn, -FLT_MAX);
   __syncthreads();
   const int oW4 = g.oW >> 2;
+  const unsigned magicOw4 = dev::magicOf(oW4);
   const int total = nOut * oW4;
   const long obase = ((long)plane * g.oH + ph0) * g.oW;
   for (int i = threadIdx.x; i < total; i += blockDim.x) {
-    const int r = i / oW4, b4 = i - r * oW4;
+    const int r = dev::fastDiv(i, magicOw4), b4 = i - r * oW4;
     const float *p = smem + r * ST * pitch;
     float mv[4] = {-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
     int mi[4] = {-1, -1, -1, -1};
@@ -353,8 +363,8 @@ avgPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, PoolGeom 
   using S = dev::Strip<KS, ST, PAD>;
   constexpr int NW = S::NW;
   extern __shared__ float smem[];
-  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
-  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  int plane, tile;
+  blockPos(g, plane, tile);
   const int ph0 = tile * g.tileRows;
   const int nOut = min(g.tileRows, g.oH - ph0);
   const int nIn = (nOut - 1) * ST + KS;
@@ -362,10 +372,11 @@ avgPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, PoolGeom 
   S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, ph0 * ST - PAD, nIn, 0.f);
   __syncthreads();
   const int oW4 = g.oW >> 2;
+  const unsigned magicOw4 = dev::magicOf(oW4);
   const int total = nOut * oW4;
   const long obase = ((long)plane * g.oH + ph0) * g.oW;
   for (int i = threadIdx.x; i < total; i += blockDim.x) {
-    const int r = i / oW4, b4 = i - r * oW4;
+    const int r = dev::fastDiv(i, magicOw4), b4 = i - r * oW4;
     const float *p = smem + r * ST * pitch;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -378,10 +389,15 @@ avgPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, PoolGeom 
         for (int q = 0; q < 4; ++q) acc[q] += win[q * ST + kw];
     }
     float res[4];
+    if (g.constDiv) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      int hs, he, ws, we;
-      res[q] = acc[q] / avgDivisor<INCLUDE_PAD>(ph0 + r, b4 * 4 + q, g, hs, he, ws, we);
+      for (int q = 0; q < 4; ++q) res[q] = acc[q] / (float)(KS * KS);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        int hs, he, ws, we;
+        res[q] = acc[q] / avgDivisor<INCLUDE_PAD>(ph0 + r, b4 * 4 + q, g, hs, he, ws, we);
+      }
     }
     *reinterpret_cast<float4 *>(out + obase + (long)r * g.oW + b4 * 4) = make_float4(res[0], res[1], res[2], res[3]);
   }
@@ -403,8 +419,8 @@ poolBwdStrip(const float *__restrict__ gradOut, const long *__restrict__ indices
   constexpr int OFF = ((dev::kStripPadL + QW0) % 4 + 4) % 4;
   constexpr int ALIGN = (CPB % 4 == 0) ? 4 : 2;
   extern __shared__ float smem[];
-  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
-  const int plane = bid / g.tilesPerPlane, tile = bid - plane * g.tilesPerPlane;
+  int plane, tile;
+  blockPos(g, plane, tile);
   const int h0 = tile * g.tileRows;  // multiple of ST
   const int nRows = min(g.tileRows, g.H - h0);
   const int pitch = g.oW + dev::kStripPadL;
@@ -417,8 +433,9 @@ poolBwdStrip(const float *__restrict__ gradOut, const long *__restrict__ indices
     dev::loadRowsPadded<true>(gs, gp, g.oH, g.oW, ph0, stageRows, pitch, dev::kStripPadL, 0.f);
     const long *ip = indices + (long)plane * g.oH * g.oW;
     const int cnt = stageRows * pitch + dev::kStripPadL;
+    const unsigned magicPitch = dev::magicOf(pitch);
     for (int i = threadIdx.x; i < cnt; i += blockDim.x) {
-      int r = i / pitch, cc = i - r * pitch - dev::kStripPadL;
+      int r = dev::fastDiv(i, magicPitch), cc = i - r * pitch - dev::kStripPadL;
       int ph = ph0 + r;
       int v = -2;
       if (cc >= 0 && r < stageRows && ph >= 0 && ph < g.oH) v = (int)(ip[(long)ph * g.oW + cc] - TH_INDEX_BASE);
@@ -426,24 +443,27 @@ poolBwdStrip(const float *__restrict__ gradOut, const long *__restrict__ indices
     }
   } else {
     const int cnt = stageRows * pitch + dev::kStripPadL;
+    const unsigned magicPitch = dev::magicOf(pitch);
     for (int i = threadIdx.x; i < cnt; i += blockDim.x) {
-      int r = i / pitch, cc = i - r * pitch - dev::kStripPadL;
+      int r = dev::fastDiv(i, magicPitch), cc = i - r * pitch - dev::kStripPadL;
       int ph = ph0 + r;
       float v = 0.f;
       if (cc >= 0 && r < stageRows && ph >= 0 && ph < g.oH) {
         int hs, he, ws, we;
-        v = gp[(long)ph * g.oW + cc] / avgDivisor<INCLUDE_PAD>(ph, cc, g, hs, he, ws, we);
+        const float gyv = gp[(long)ph * g.oW + cc];
+        v = g.constDiv ? gyv / (float)(KS * KS) : gyv / avgDivisor<INCLUDE_PAD>(ph, cc, g, hs, he, ws, we);
       }
       gs[i] = v;
     }
   }
   __syncthreads();
   const int W4 = g.W >> 2;
+  const unsigned magicW4 = dev::magicOf(W4);
   const int nA = (nRows + ST - 1) / ST;
   const int total = nA * W4;
   float *o = gradIn + ((long)plane * g.H + h0) * g.W;
   for (int i = threadIdx.x; i < total; i += blockDim.x) {
-    const int a = i / W4, b = i - a * W4;
+    const int a = dev::fastDiv(i, magicW4), b = i - a * W4;
     float acc[ST][4];
 #pragma unroll
     for (int dy = 0; dy < ST; ++dy)
@@ -491,6 +511,14 @@ int forcedPath() {
   return e ? atoi(e) : 0;
 }
 bool forceDirect() { return forcedPath() == 1; }
+
+// 1 when no window of the average pooling is clipped, i.e. every divisor is kH*kW:
+// windows inside the padded extent (count_include_pad) or inside the image itself.
+int avgConstDivisor(const PoolGeom &g, bool include_pad) {
+  int lastH = (g.oH - 1) * g.dH - g.padH + g.kH, lastW = (g.oW - 1) * g.dW - g.padW + g.kW;  // one past the last window
+  if (include_pad) return lastH <= g.H + g.padH && lastW <= g.W + g.padW;
+  return g.padH == 0 && g.padW == 0 && lastH <= g.H && lastW <= g.W;
+}
 
 // (KS, ST, PAD) combinations the strip kernels are instantiated for
 #define POOL_STRIP_COMBOS(X) X(3, 2, 1) X(2, 2, 0) X(3, 2, 0) X(3, 1, 1)
@@ -601,6 +629,8 @@ PoolCall poolSetup(THCudaTensor *input, THCudaTensor *gradOutput, THCudaLongTens
   g.H = (int)nInputRows, g.W = (int)nInputCols, g.oH = (int)nOutputRows, g.oW = (int)nOutputCols;
   g.kH = kH, g.kW = kW, g.dH = dH, g.dW = dW, g.padH = padH, g.padW = padW, g.dilH = dilH, g.dilW = dilW;
   g.tileRows = g.tilesPerPlane = g.nblk = g.maxStageRows = 0;
+  g.magicTiles = 0;
+  g.constDiv = 0;
   return c;
 }
 
@@ -636,9 +666,11 @@ void maxPoolUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *out
     auto stageRows = [&](int rows) { return std::min(g.H, (rows - 1) * g.dH + (g.kH - 1) * g.dilH + 1); };
     auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.W * sizeof(float); };
     auto sbytes = [&](int rows) { return fwdStripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
+    auto staged = [&](int rows) { return (size_t)((rows - 1) * g.dH + g.kH) * g.W; };
     if (stripFwdOk(g) && vec && aligned16(data(output)) && aligned16(data(indices)) &&
-        launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane)) {
+        launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane, staged)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane);
       dim3 grid(g.nblk), block(dev::kBlock);
       size_t lds = sbytes(g.tileRows);
 #define X(K, S, P)                                  \
@@ -648,6 +680,7 @@ void maxPoolUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *out
 #undef X
     } else if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane);
       if (vec)
         launchMaxFwd<true>(s, bytes(g.tileRows), in.ptr(), data(output), data(indices), g);
       else
@@ -692,6 +725,7 @@ void maxPoolUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *
       launch::pickBand(launch::ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
     g.tileRows = units * g.dH;
     g.nblk = (int)(planes * g.tilesPerPlane);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane);
     dim3 grid(g.nblk), block(dev::kBlock);
     size_t lds = sbytes(units);
 #define X(K, S, P)                            \
@@ -701,6 +735,7 @@ void maxPoolUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *
 #undef X
   } else if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane);
     g.maxStageRows = stageRows(g.tileRows);
     dim3 grid(g.nblk), block(dev::kBlock);
     if (vec)
@@ -763,6 +798,7 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
   THC_ARG_CHECK(output != nullptr, 3, "output tensor expected");
   PoolCall call = poolSetup(input, nullptr, nullptr, kH, kW, dH, dW, padH, padW, 1, 1, ceil_mode, false);
   PoolGeom &g = call.g;
+  g.constDiv = avgConstDivisor(g, count_include_pad);
   Contiguous in(state, input);
   resize(state, output, {call.N, call.C, g.oH, g.oW});
   if (!isContiguous(erase(output))) error("output tensor has to be contiguous");
@@ -773,9 +809,11 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
     auto stageRows = [&](int rows) { return std::min(g.H, (rows - 1) * g.dH + g.kH); };
     auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.W * sizeof(float); };
     auto sbytes = [&](int rows) { return fwdStripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
+    auto staged = [&](int rows) { return (size_t)((rows - 1) * g.dH + g.kH) * g.W; };
     if (stripFwdOk(g) && vec && aligned16(data(output)) &&
-        launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane)) {
+        launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane, staged)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane);
       dim3 grid(g.nblk), block(dev::kBlock);
       size_t lds = sbytes(g.tileRows);
 #define X(K, S, P)                                                                        \
@@ -789,6 +827,7 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
 #undef X
     } else if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane);
       dim3 grid(g.nblk), block(dev::kBlock);
       size_t lds = bytes(g.tileRows);
       if (count_include_pad) {
@@ -824,6 +863,7 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
   THC_ARG_CHECK(gradInput != nullptr, 4, "gradInput tensor expected");
   PoolCall call = poolSetup(input, gradOutput, nullptr, kH, kW, dH, dW, padH, padW, 1, 1, ceil_mode, false);
   PoolGeom &g = call.g;
+  g.constDiv = avgConstDivisor(g, count_include_pad);
   Contiguous go(state, gradOutput);
   if (call.batch)
     resize(state, gradInput, {call.N, call.C, g.H, g.W});
@@ -844,6 +884,7 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
       launch::pickBand(launch::ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
     g.tileRows = units * g.dH;
     g.nblk = (int)(planes * g.tilesPerPlane);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane);
     dim3 grid(g.nblk), block(dev::kBlock);
     size_t lds = sbytes(units);
 #define X(K, S, P)                                                                                                    \
@@ -857,6 +898,7 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
 #undef X
   } else if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
+      g.magicTiles = dev::magicOf(g.tilesPerPlane);
     dim3 grid(g.nblk), block(dev::kBlock);
     size_t lds = bytes(g.tileRows);
     if (count_include_pad) {

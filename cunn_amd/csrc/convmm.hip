@@ -347,8 +347,34 @@ struct FwdArgs {
   // their 128x128 partial tiles go to `partial` and fwdTailFixupKernel folds them
   int tile0, nSplit, ktPerSplit;
   float *partial;
+  const int2 *taps;   // FAST kernel: per k (padded to a multiple of BK) {byte offset of tap (c,kh,kw), kh << 16 | kw}
 };
 
+// taps[k] = {((c*H + kh)*W + kw) * 4, kh << 16 | kw} for k = (c*kH + kh)*kW + kw < K; beyond K a row offset
+// that fails every bounds test. Built once per call: the FAST forward kernel reads 8 consecutive entries
+// per wave and k-tile with scalar loads instead of dividing k by kH*kW and kW in every lane.
+__global__ void __launch_bounds__(dev::kBlock)
+buildTapTableKernel(int2 *taps, int entries, ConvGeom g) {
+  const int KK = g.kH * g.kW;
+  for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < entries; k += gridDim.x * blockDim.x) {
+    int2 e;
+    if (k < g.K) {
+      int c = k / KK, rem = k - c * KK;
+      int kh = rem / g.kW, kw = rem - kh * g.kW;
+      e.x = ((c * g.H + kh) * g.W + kw) * 4;
+      e.y = (kh << 16) | kw;
+    } else {
+      e.x = 0;
+      e.y = 0x4000 << 16;
+    }
+    taps[k] = e;
+  }
+}
+
+// FAST: K % BK == 0, 16-byte loadable weight rows and a tap table - the loaders are
+// branch-free (rows past M are clamped and discarded in the epilogue, columns past the
+// batch and taps outside the image read 0 through the buffer bounds check).
+template <bool FAST>
 __global__ void __launch_bounds__(dev::kBlock)
 convFwdImplicitKernel(FwdArgs p, ConvGeom g) {
   __shared__ float4 As[2][BK / 4][FPITCH];
@@ -371,7 +397,7 @@ convFwdImplicitKernel(FwdArgs p, ConvGeom g) {
   // A loader: row (t >> 1), k = 8 * (t & 1) .. + 7
   const int rowA = t >> 1, kA = (t & 1) * 8;
   const bool rowOk = m0 + rowA < p.M;
-  const float *aSrc = p.w + (long)(m0 + rowA) * g.K + kA;
+  const float *aSrc = p.w + (long)(FAST ? min(m0 + rowA, p.M - 1) : m0 + rowA) * g.K + kA;
   // B loader: column (t & 127) = one output position, k = 8 * (t >> 7) .. + 7 (wave-uniform)
   const int colB = t & 127;
   const int kB = __builtin_amdgcn_readfirstlane((t >> 7) * 8);
@@ -392,52 +418,72 @@ convFwdImplicitKernel(FwdArgs p, ConvGeom g) {
     }
   }
 
-  float4 ra[2], rb[2];
+  float4 ra0, ra1, rb0, rb1;
   const int nktAll = (g.K + BK - 1) / BK;
   const int ktBegin = blockIdx.y * p.ktPerSplit;
   const int nkt = min(nktAll, ktBegin + p.ktPerSplit);  // this workgroup reduces k-tiles [ktBegin, nkt)
 
   auto loadTiles = [&](int kt) {
     const int k0 = kt * BK;
-    // ---- A
-    if (p.vecA && rowOk && k0 + kA + 8 <= g.K) {
-      ra[0] = reinterpret_cast<const float4 *>(aSrc + k0)[0];
-      ra[1] = reinterpret_cast<const float4 *>(aSrc + k0)[1];
+    if constexpr (FAST) {
+      ra0 = reinterpret_cast<const float4 *>(aSrc + k0)[0];
+      ra1 = reinterpret_cast<const float4 *>(aSrc + k0)[1];
+      // the 8 taps of this wave and k-tile: 16 consecutive dwords at a wave-uniform address -> one scalar load
+      const int4 *tp = reinterpret_cast<const int4 *>(p.taps + k0 + kB);
+      const int4 e01 = tp[0], e23 = tp[1], e45 = tp[2], e67 = tp[3];
+      float t0, t1, t2, t3, t4, t5, t6, t7;
+#define FWD_TAP(EX, EY, DST)                                                                                   \
+  {                                                                                                            \
+    const int ih = ih0 + ((EY) >> 16), iw = iw0 + ((EY)&0xffff);                                               \
+    const bool ok = ((unsigned)ih < (unsigned)g.H) & ((unsigned)iw < (unsigned)g.W);                           \
+    DST = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, ok ? posOff + (EX) : kOob, 0, 0)); \
+  }
+      FWD_TAP(e01.x, e01.y, t0) FWD_TAP(e01.z, e01.w, t1) FWD_TAP(e23.x, e23.y, t2) FWD_TAP(e23.z, e23.w, t3)
+      FWD_TAP(e45.x, e45.y, t4) FWD_TAP(e45.z, e45.w, t5) FWD_TAP(e67.x, e67.y, t6) FWD_TAP(e67.z, e67.w, t7)
+#undef FWD_TAP
+      rb0 = make_float4(t0, t1, t2, t3);
+      rb1 = make_float4(t4, t5, t6, t7);
     } else {
+      // ---- A
+      if (p.vecA && rowOk && k0 + kA + 8 <= g.K) {
+        ra0 = reinterpret_cast<const float4 *>(aSrc + k0)[0];
+        ra1 = reinterpret_cast<const float4 *>(aSrc + k0)[1];
+      } else {
+        float tmp[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) tmp[i] = (rowOk && k0 + kA + i < g.K) ? aSrc[k0 + i] : 0.f;
+        ra0 = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
+        ra1 = make_float4(tmp[4], tmp[5], tmp[6], tmp[7]);
+      }
+      // ---- B: scalar walk over the 8 taps of this wave
+      int k = k0 + kB;  // scalar
+      int c = k / KK, rem = k - c * KK;
+      int kh = rem / g.kW, kw = rem - kh * g.kW;
       float tmp[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) tmp[i] = (rowOk && k0 + kA + i < g.K) ? aSrc[k0 + i] : 0.f;
-      ra[0] = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
-      ra[1] = make_float4(tmp[4], tmp[5], tmp[6], tmp[7]);
-    }
-    // ---- B: scalar walk over the 8 taps of this wave
-    int k = k0 + kB;  // scalar
-    int c = k / KK, rem = k - c * KK;
-    int kh = rem / g.kW, kw = rem - kh * g.kW;
-    float tmp[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int ih = ih0 + kh, iw = iw0 + kw;
-      const bool ok = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W && (k + i) < g.K;
-      const int soff = ((c * g.H + kh) * g.W + kw) * 4;  // scalar
-      const int off = ok ? posOff + soff : kOob;
-      tmp[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
-      if (++kw == g.kW) {
-        kw = 0;
-        if (++kh == g.kH) {
-          kh = 0;
-          ++c;
+      for (int i = 0; i < 8; ++i) {
+        const int ih = ih0 + kh, iw = iw0 + kw;
+        const bool ok = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W && (k + i) < g.K;
+        const int soff = ((c * g.H + kh) * g.W + kw) * 4;  // scalar
+        const int off = ok ? posOff + soff : kOob;
+        tmp[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
+        if (++kw == g.kW) {
+          kw = 0;
+          if (++kh == g.kH) {
+            kh = 0;
+            ++c;
+          }
         }
       }
+      rb0 = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
+      rb1 = make_float4(tmp[4], tmp[5], tmp[6], tmp[7]);
     }
-    rb[0] = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
-    rb[1] = make_float4(tmp[4], tmp[5], tmp[6], tmp[7]);
   };
   auto storeTiles = [&](int buf) {
-    As[buf][(t & 1) * 2][rowA] = ra[0];
-    As[buf][(t & 1) * 2 + 1][rowA] = ra[1];
-    Bs[buf][(t >> 7) * 2][colB] = rb[0];
-    Bs[buf][(t >> 7) * 2 + 1][colB] = rb[1];
+    As[buf][(t & 1) * 2][rowA] = ra0;
+    As[buf][(t & 1) * 2 + 1][rowA] = ra1;
+    Bs[buf][(t >> 7) * 2][colB] = rb0;
+    Bs[buf][(t >> 7) * 2 + 1][colB] = rb1;
   };
 
   loadTiles(ktBegin);
@@ -735,7 +781,8 @@ bool forceGeneric() {
 // over all CUs (partials in scratch, folded by fwdTailFixupKernel in a fixed order).
 struct FwdPlan {
   int mTiles, total, full, tail, nSplit, ktPerSplit;
-  long scratchFloats;
+  int tapEntries;      // > 0: the FAST kernel applies; entries of the tap table at the start of the scratch
+  long scratchFloats;  // tap table (2 ints per entry) followed by the tail partials
 };
 FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
   FwdPlan pl{};
@@ -752,14 +799,23 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
   pl.full = pl.total - pl.tail;
   pl.ktPerSplit = launch::ceilDiv(nkt, nSplit);
   pl.nSplit = launch::ceilDiv(nkt, pl.ktPerSplit);
-  pl.scratchFloats = pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0;
+  pl.tapEntries = (g.K % BK == 0 && g.K % 4 == 0 && g.kH < 0x4000 && g.kW < 0x4000) ? nkt * BK : 0;
+  pl.scratchFloats = 2L * pl.tapEntries + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0);
   return pl;
 }
 
-// out(nImages, M, L) = bias + W(M x K) * im2col(x); `partial` holds plan.scratchFloats floats
-void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *partial, const float *w, const float *x, float *out,
+// out(nImages, M, L) = bias + W(M x K) * im2col(x); `scratch` holds plan.scratchFloats floats
+void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const float *w, const float *x, float *out,
                        const float *bias, int M, int nImages, const ConvGeom &g) {
+  const bool fast = pl.tapEntries > 0 && launch::aligned16(w) && launch::aligned16(scratch);
+  float *partial = scratch + 2L * pl.tapEntries;
+  if (fast) {
+    buildTapTableKernel<<<launch::directGrid(pl.tapEntries, dev::kBlock), dev::kBlock, 0, s>>>(
+        reinterpret_cast<int2 *>(scratch), pl.tapEntries, g);
+    THC_HIP_CHECK(hipGetLastError());
+  }
   FwdArgs p{};
+  p.taps = reinterpret_cast<const int2 *>(scratch);
   p.w = w;
   p.x = x;
   p.out = out;
@@ -772,7 +828,10 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *partial, const f
   p.nSplit = 1;
   p.ktPerSplit = launch::ceilDiv(g.K, BK);
   if (pl.full > 0) {
-    convFwdImplicitKernel<<<dim3(pl.full), dev::kBlock, 0, s>>>(p, g);
+    if (fast)
+      convFwdImplicitKernel<true><<<dim3(pl.full), dev::kBlock, 0, s>>>(p, g);
+    else
+      convFwdImplicitKernel<false><<<dim3(pl.full), dev::kBlock, 0, s>>>(p, g);
     THC_HIP_CHECK(hipGetLastError());
   }
   if (pl.tail > 0) {
@@ -780,7 +839,10 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *partial, const f
     p.ktPerSplit = pl.ktPerSplit;
     p.nSplit = pl.nSplit;
     p.partial = partial;
-    convFwdImplicitKernel<<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, g);
+    if (fast)
+      convFwdImplicitKernel<true><<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, g);
+    else
+      convFwdImplicitKernel<false><<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, g);
     THC_HIP_CHECK(hipGetLastError());
     fwdTailFixupKernel<<<dim3(pl.tail, BM * BN / (4 * dev::kBlock)), dev::kBlock, 0, s>>>(p, g);
     THC_HIP_CHECK(hipGetLastError());
@@ -828,11 +890,11 @@ void THNN_CudaSpatialConvolutionMM_updateOutput(THCState *state, THCudaTensor *i
   if (implicit2) {
     FwdPlan pl = planFwdImplicit(g.Cout, std::min(group, g.N), g);
     Temp tmp;
-    float *partial = scratchFloats(state, columns, pl.scratchFloats, tmp, "columns");
+    float *scratch = scratchFloats(state, columns, pl.scratchFloats, tmp, "columns");
     for (int n0 = 0; n0 < g.N; n0 += group) {
       int cnt = std::min(group, g.N - n0);
       if (cnt != std::min(group, g.N)) pl = planFwdImplicit(g.Cout, cnt, g);  // last, smaller group: needs no more scratch
-      launchFwdImplicit(s, pl, partial, data(weight), in.ptr() + (long)n0 * g.Cin * g.H * g.W,
+      launchFwdImplicit(s, pl, scratch, data(weight), in.ptr() + (long)n0 * g.Cin * g.H * g.W,
                         data(output) + (long)n0 * g.Cout * g.L, bias ? data(bias) : nullptr, g.Cout, cnt, g);
     }
   }

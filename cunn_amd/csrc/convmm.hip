@@ -573,6 +573,166 @@ fwdTailFixupKernel(FwdArgs p, ConvGeom g) {
   }
 }
 
+// ---- weight gradient, second generation ------------------------------------------
+// partial[split][o][k] = sum over the split's positions r = (n, l) of gy[n][o][l] * col[k][n,l].
+// Same MFMA core and float4 operand layout as the forward kernel, with the reduction
+// running over positions: 4 consecutive l of one gradOutput row are already a float4
+// in memory (L % 4 == 0), so the A tile goes from 16-byte buffer loads to
+// ds_write_b128 without a transpose. For the B tile a lane owns one position of the
+// k-tile and 8 columns k; the columns never change, so their taps (c, kh, kw) are
+// resolved once into registers and each k-tile costs one position decomposition per
+// lane. 16 consecutive lanes gather 16 consecutive positions (64-byte runs of x).
+constexpr int GPITCH = BN + 4;  // float4 per position-group row of Bs: the 4 groups of a wave's scalar stores hit disjoint banks
+
+struct GradWeightArgs {
+  const float *gy;  // (N, M, L)
+  const float *x;   // (N, Cin, H, W)
+  float *partial;   // (splits, M, Ncols)
+  int M, Ncols;     // Cout, K
+  int mTiles, nTiles;
+  int totalKt, ktPerSplit;  // k-tiles of BK positions over the N*L positions; per split
+  int gyBytes, xBytes;      // < 2^31
+  unsigned magicOW;
+};
+
+__global__ void __launch_bounds__(dev::kBlock)
+convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
+  __shared__ float4 As[2][BK / 4][FPITCH];
+  __shared__ float4 Bs[2][BK / 4][GPITCH];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  // workgroups that reduce the same positions (one split) are neighbours in the remapped order: same XCD, same L2
+  const int tilesPerSplit = p.mTiles * p.nTiles;
+  const int bid = dev::xcdRemap(blockIdx.x, gridDim.x);
+  const int split = bid / tilesPerSplit, tileIdx = bid - split * tilesPerSplit;
+  const int mTile = tileIdx % p.mTiles, nTile = tileIdx / p.mTiles;
+  const int m0 = mTile * BM, j0 = nTile * BN;
+  const int ktBegin = split * p.ktPerSplit;
+  const int ktEnd = min(p.totalKt, ktBegin + p.ktPerSplit);
+  const int kOob = 0x7fffffff;
+
+  float16v acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // ---- A loader: row o = t >> 1, positions 8 * (t & 1) .. + 7 of the k-tile as two float4
+  const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc((void *)p.gy, 0, p.gyBytes, 0x00020000);
+  const int rowA = t >> 1;
+  const int rowOffA = min(m0 + rowA, p.M - 1) * g.L * 4;  // rows past M are clamped and dropped in the epilogue
+  const int imgStrideA = p.M * g.L * 4;
+  int nA, lA;
+  {
+    const long r = (long)ktBegin * BK + (t & 1) * 8;
+    nA = (int)(r / g.L);
+    lA = (int)(r - (long)nA * g.L);
+  }
+  // ---- B loader: position t & 15 of the k-tile, columns (t >> 4) + 16 i
+  const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.xBytes, 0x00020000);
+  const int rB = t & 15, cB = t >> 4;
+  int tapOff[8], tapHW[8];
+  {
+    const int KK = g.kH * g.kW;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int k = j0 + cB + 16 * i;
+      const int c = k / KK, rem = k - c * KK;
+      const int kh = rem / g.kW, kw = rem - kh * g.kW;
+      tapOff[i] = ((c * g.H + kh) * g.W + kw) * 4;
+      tapHW[i] = k < p.Ncols ? (kh << 16) | kw : 0x4000 << 16;  // columns past K fail the row test
+    }
+  }
+  int nB, lB;
+  {
+    const long r = (long)ktBegin * BK + rB;
+    nB = (int)(r / g.L);
+    lB = (int)(r - (long)nB * g.L);
+  }
+  const int imgStrideB = g.Cin * g.H * g.W * 4;
+
+  float4 ra0, ra1;
+  float rb[8];
+  // loads the k-tile the position counters stand on, then advances them by BK (L >= BK: one wrap at most)
+  auto loadTiles = [&]() {
+    {
+      int n1 = nA, l1 = lA + 4;
+      if (l1 >= g.L) l1 -= g.L, ++n1;
+      const int o0 = nA < g.N ? nA * imgStrideA + rowOffA + lA * 4 : kOob;
+      const int o1 = n1 < g.N ? n1 * imgStrideA + rowOffA + l1 * 4 : kOob;
+      ra0 = dev::bufLoad4(gr, o0);
+      ra1 = dev::bufLoad4(gr, o1);
+      lA += BK;
+      if (lA >= g.L) lA -= g.L, ++nA;
+    }
+    {
+      const int oh = dev::fastDiv(lB, p.magicOW), ow = lB - oh * g.oW;
+      const int ih0 = nB < g.N ? oh * g.dH - g.padH : -(1 << 28);
+      const int iw0 = ow * g.dW - g.padW;
+      const int posOff = nB * imgStrideB + (ih0 * g.W + iw0) * 4;  // only used when the tap is inside the image
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int ih = ih0 + (tapHW[i] >> 16), iw = iw0 + (tapHW[i] & 0xffff);
+        const bool ok = ((unsigned)ih < (unsigned)g.H) & ((unsigned)iw < (unsigned)g.W);
+        rb[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, ok ? posOff + tapOff[i] : kOob, 0, 0));
+      }
+      lB += BK;
+      if (lB >= g.L) lB -= g.L, ++nB;
+    }
+  };
+  auto storeTiles = [&](int buf) {
+    As[buf][(t & 1) * 2][rowA] = ra0;
+    As[buf][(t & 1) * 2 + 1][rowA] = ra1;
+    float *b = reinterpret_cast<float *>(&Bs[buf][rB >> 2][cB]) + (rB & 3);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) b[64 * i] = rb[i];  // column + 16 = 16 float4 further
+  };
+
+  if (ktBegin < ktEnd) {
+    loadTiles();
+    storeTiles(0);
+  }
+  __syncthreads();
+  const int grp = lane >> 5, idx = lane & 31;
+  for (int kt = ktBegin; kt < ktEnd; ++kt) {
+    const int buf = (kt - ktBegin) & 1;
+    if (kt + 1 < ktEnd) loadTiles();
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const float4 a0 = As[buf][2 * s + grp][wm * 64 + idx], a1 = As[buf][2 * s + grp][wm * 64 + 32 + idx];
+      const float4 b0 = Bs[buf][2 * s + grp][wn * 64 + idx], b1 = Bs[buf][2 * s + grp][wn * 64 + 32 + idx];
+      const float av0[4] = {a0.x, a0.y, a0.z, a0.w}, av1[4] = {a1.x, a1.y, a1.z, a1.w};
+      const float bv0[4] = {b0.x, b0.y, b0.z, b0.w}, bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv0[j], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv1[j], acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv0[j], acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv1[j], acc[1][1], 0, 0, 0);
+      }
+    }
+    if (kt + 1 < ktEnd) storeTiles(buf ^ 1);
+    __syncthreads();
+  }
+
+  // lane holds column (lane & 31), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
+  float *dst = p.partial + (long)split * p.M * p.Ncols;
+#pragma unroll
+  for (int tj = 0; tj < 2; ++tj) {
+    const int col = j0 + wn * 64 + tj * 32 + idx;
+    if (col >= p.Ncols) continue;
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + grp * 4 + (v & 3);
+        if (row < p.M) dst[(long)row * p.Ncols + col] = acc[ti][tj][v];
+      }
+  }
+}
+
 // gW[i] += scale * sum_s partial[s][i], s ascending
 __global__ void __launch_bounds__(dev::kBlock)
 foldPartialsKernel(const float *__restrict__ partial, float *__restrict__ dst, long count, int splits, float scale) {
@@ -1026,7 +1186,12 @@ void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTens
   if ((long)g.N * g.L >= 0x7fffffffL) error("SpatialConvolutionMM: batch too large");
   const int mT = (int)tiles(g.Cout, BM), nT = (int)tiles(g.K, BN);
   const int totalKt = launch::ceilDiv(g.N * g.L, BK);
-  const int slots = residentSlots((const void *)convGemmKernel<kGradWeight>);
+  // second-generation kernel: gradOutput rows loadable as float4 groups, 32-bit byte offsets into both operands
+  const long gyBytes = (long)g.N * g.Cout * g.L * 4, xBytes = (long)g.N * g.Cin * g.H * g.W * 4;
+  const bool fast = !forceGeneric() && g.L % 4 == 0 && g.L >= BK && launch::aligned16(go.ptr()) &&
+                    gyBytes < 0x7fffffffL && xBytes < 0x7fffffffL && g.kH < 0x4000 && g.kW < 0x4000 &&
+                    (long)g.L * g.oW < 0x7fffffffL;
+  const int slots = residentSlots(fast ? (const void *)convGradWeightKernel : (const void *)convGemmKernel<kGradWeight>);
   int splits = std::max(1, std::min(totalKt, slots / (mT * nT)));
   const int perSplit = launch::ceilDiv(totalKt, splits);
   splits = launch::ceilDiv(totalKt, perSplit);
@@ -1041,19 +1206,36 @@ void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTens
     tmp = Temp(s, (size_t)splits * count * sizeof(float));
     partial = (float *)tmp.get();
   }
-  GemmArgs p{};
-  p.a = go.ptr();
-  p.b = in.ptr();
-  p.c = partial;
-  p.M = g.Cout;
-  p.Ncols = g.K;
-  p.R = 0;
-  p.n0 = perSplit;
-  p.nImages = g.N;
-  p.mTiles = mT;
-  p.vecA = (g.L % 4 == 0) && launch::aligned16(p.a);
-  dim3 grid(mT * nT, splits);
-  convGemmKernel<kGradWeight><<<grid, dev::kBlock, 0, s>>>(p, g);
+  if (fast) {
+    GradWeightArgs q{};
+    q.gy = go.ptr();
+    q.x = in.ptr();
+    q.partial = partial;
+    q.M = g.Cout;
+    q.Ncols = g.K;
+    q.mTiles = mT;
+    q.nTiles = nT;
+    q.totalKt = totalKt;
+    q.ktPerSplit = perSplit;
+    q.gyBytes = (int)gyBytes;
+    q.xBytes = (int)xBytes;
+    q.magicOW = dev::magicOf(g.oW);
+    convGradWeightKernel<<<dim3(mT * nT * splits), dev::kBlock, 0, s>>>(q, g);
+  } else {
+    GemmArgs p{};
+    p.a = go.ptr();
+    p.b = in.ptr();
+    p.c = partial;
+    p.M = g.Cout;
+    p.Ncols = g.K;
+    p.R = 0;
+    p.n0 = perSplit;
+    p.nImages = g.N;
+    p.mTiles = mT;
+    p.vecA = (g.L % 4 == 0) && launch::aligned16(p.a);
+    dim3 grid(mT * nT, splits);
+    convGemmKernel<kGradWeight><<<grid, dev::kBlock, 0, s>>>(p, g);
+  }
   THC_HIP_CHECK(hipGetLastError());
   foldPartialsKernel<<<launch::directGrid(count, dev::kBlock), dev::kBlock, 0, s>>>(partial, data(gradWeight), count,
                                                                                    splits, scale);

@@ -19,6 +19,7 @@
 //                      lib/THCUNN/im2col.h:63-102 over the group.
 #include <map>
 #include <mutex>
+#include <type_traits>
 
 #include "device_utils.h"
 #include "launch_utils.h"
@@ -342,39 +343,99 @@ struct FwdArgs {
   int M, Ncols;       // Ncols = nImages * L
   int mTiles;
   int xBytes;         // bytes of the nImages input images (< 2^31)
+  int wBytes;         // padded kernel: bytes of the weights (< 2^31)
   bool vecA;
   // tail launch: tiles tile0 .. are each reduced by nSplit workgroups over ktPerSplit k-tiles;
   // their 128x128 partial tiles go to `partial` and fwdTailFixupKernel folds them
   int tile0, nSplit, ktPerSplit;
   float *partial;
-  const int2 *taps;   // FAST kernel: per k (padded to a multiple of BK) {byte offset of tap (c,kh,kw), kh << 16 | kw}
+  const int *taps;    // padded kernel: byte offset of tap (c, kh, kw) inside a (zero-padded) image, per k
 };
 
-// taps[k] = {((c*H + kh)*W + kw) * 4, kh << 16 | kw} for k = (c*kH + kh)*kW + kw < K; beyond K a row offset
-// that fails every bounds test. Built once per call: the FAST forward kernel reads 8 consecutive entries
-// per wave and k-tile with scalar loads instead of dividing k by kH*kW and kW in every lane.
-__global__ void __launch_bounds__(dev::kBlock)
-buildTapTableKernel(int2 *taps, int entries, ConvGeom g) {
-  const int KK = g.kH * g.kW;
-  for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < entries; k += gridDim.x * blockDim.x) {
-    int2 e;
-    if (k < g.K) {
-      int c = k / KK, rem = k - c * KK;
-      int kh = rem / g.kW, kw = rem - kh * g.kW;
-      e.x = ((c * g.H + kh) * g.W + kw) * 4;
-      e.y = (kh << 16) | kw;
-    } else {
-      e.x = 0;
-      e.y = 0x4000 << 16;
-    }
-    taps[k] = e;
+// Epilogue shared by the forward kernels: a lane holds column (lane & 31) and rows
+// 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 accumulator tile. Split workgroups store their
+// partial tile, the others add the bias and store to out(n, row, l).
+__device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g, const float16v (&acc)[2][2], int bx,
+                                            int by, int m0, int j0, int wm, int wn, int grp, int idx) {
+  const int rowHalf = grp * 4;
+  if (p.nSplit > 1) {
+    float *dst = p.partial + ((long)bx * p.nSplit + by) * (BM * BN);
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+      for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          dst[(wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3)) * BN + wn * 64 + tj * 32 + idx] = acc[ti][tj][v];
+    return;
+  }
+#pragma unroll
+  for (int tj = 0; tj < 2; ++tj) {
+    const long col = (long)j0 + wn * 64 + tj * 32 + idx;
+    if (col >= p.Ncols) continue;
+    const int n = (int)(col / g.L);
+    const int l = (int)(col - (long)n * g.L);
+    float *dst = p.out + (long)n * p.M * g.L + l;
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
+        if (row < p.M) {
+          float val = acc[ti][tj][v];
+          if (p.bias) val += p.bias[row];
+          dst[(long)row * g.L] = val;
+        }
+      }
   }
 }
 
-// FAST: K % BK == 0, 16-byte loadable weight rows and a tap table - the loaders are
-// branch-free (rows past M are clamped and discarded in the epilogue, columns past the
-// batch and taps outside the image read 0 through the buffer bounds check).
-template <bool FAST>
+// taps[k] = ((c*H + kh)*W + kw) * 4 for k = (c*kH + kh)*kW + kw; g is the geometry of the padded images.
+__global__ void __launch_bounds__(dev::kBlock)
+buildTapTableKernel(int *taps, int entries, ConvGeom g) {
+  const int KK = g.kH * g.kW;
+  for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < entries; k += gridDim.x * blockDim.x) {
+    const int c = k / KK, rem = k - c * KK;
+    const int kh = rem / g.kW, kw = rem - kh * g.kW;
+    taps[k] = ((c * g.H + kh) * g.W + kw) * 4;
+  }
+}
+
+// xp(nc, H + 2 padH, W + 2 padW) = x(nc, H, W) inside a zero border. grid = (planes, chunks of a plane);
+// VEC: a lane produces 4 consecutive floats of the bordered plane with one 16-byte store
+// (plane size a multiple of 4 floats, 16-byte aligned destination).
+template <bool VEC>
+__global__ void __launch_bounds__(dev::kBlock)
+padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int padH, int padW) {
+  const int Hp = H + 2 * padH, Wp = W + 2 * padW;
+  const unsigned magic = dev::magicOf(Wp);
+  const float *src = x + (long)blockIdx.x * H * W;
+  float *dst = xp + (long)blockIdx.x * Hp * Wp;
+  auto fetch = [&](int j) {
+    const int hp = dev::fastDiv(j, magic), wp = j - hp * Wp;
+    const int h = hp - padH, w = wp - padW;
+    return (((unsigned)h < (unsigned)H) & ((unsigned)w < (unsigned)W)) ? src[h * W + w] : 0.f;
+  };
+  const int i = blockIdx.y * dev::kBlock + threadIdx.x;
+  if (VEC) {
+    if (i * 4 < Hp * Wp)
+      *reinterpret_cast<float4 *>(dst + i * 4) = make_float4(fetch(i * 4), fetch(i * 4 + 1), fetch(i * 4 + 2), fetch(i * 4 + 3));
+  } else {
+    if (i < Hp * Wp) dst[i] = fetch(i);
+  }
+}
+
+void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int H, int W, int padH, int padW) {
+  const int plane = (H + 2 * padH) * (W + 2 * padW);
+  if (launch::ceilDiv(plane, dev::kBlock) > 65535) error("SpatialConvolutionMM: image plane too large");
+  if (plane % 4 == 0 && launch::aligned16(xp))
+    padPlanesKernel<true><<<dim3((unsigned)planes, launch::ceilDiv(plane / 4, dev::kBlock)), dev::kBlock, 0, s>>>(x, xp, H, W, padH, padW);
+  else
+    padPlanesKernel<false><<<dim3((unsigned)planes, launch::ceilDiv(plane, dev::kBlock)), dev::kBlock, 0, s>>>(x, xp, H, W, padH, padW);
+  THC_HIP_CHECK(hipGetLastError());
+}
+
+// Generic forward kernel: any K, any alignment; taps and bounds resolved in the loop.
 __global__ void __launch_bounds__(dev::kBlock)
 convFwdImplicitKernel(FwdArgs p, ConvGeom g) {
   __shared__ float4 As[2][BK / 4][FPITCH];
@@ -397,7 +458,7 @@ convFwdImplicitKernel(FwdArgs p, ConvGeom g) {
   // A loader: row (t >> 1), k = 8 * (t & 1) .. + 7
   const int rowA = t >> 1, kA = (t & 1) * 8;
   const bool rowOk = m0 + rowA < p.M;
-  const float *aSrc = p.w + (long)(FAST ? min(m0 + rowA, p.M - 1) : m0 + rowA) * g.K + kA;
+  const float *aSrc = p.w + (long)(m0 + rowA) * g.K + kA;
   // B loader: column (t & 127) = one output position, k = 8 * (t >> 7) .. + 7 (wave-uniform)
   const int colB = t & 127;
   const int kB = __builtin_amdgcn_readfirstlane((t >> 7) * 8);
@@ -425,59 +486,39 @@ convFwdImplicitKernel(FwdArgs p, ConvGeom g) {
 
   auto loadTiles = [&](int kt) {
     const int k0 = kt * BK;
-    if constexpr (FAST) {
+    // ---- A
+    if (p.vecA && rowOk && k0 + kA + 8 <= g.K) {
       ra0 = reinterpret_cast<const float4 *>(aSrc + k0)[0];
       ra1 = reinterpret_cast<const float4 *>(aSrc + k0)[1];
-      // the 8 taps of this wave and k-tile: 16 consecutive dwords at a wave-uniform address -> one scalar load
-      const int4 *tp = reinterpret_cast<const int4 *>(p.taps + k0 + kB);
-      const int4 e01 = tp[0], e23 = tp[1], e45 = tp[2], e67 = tp[3];
-      float t0, t1, t2, t3, t4, t5, t6, t7;
-#define FWD_TAP(EX, EY, DST)                                                                                   \
-  {                                                                                                            \
-    const int ih = ih0 + ((EY) >> 16), iw = iw0 + ((EY)&0xffff);                                               \
-    const bool ok = ((unsigned)ih < (unsigned)g.H) & ((unsigned)iw < (unsigned)g.W);                           \
-    DST = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, ok ? posOff + (EX) : kOob, 0, 0)); \
-  }
-      FWD_TAP(e01.x, e01.y, t0) FWD_TAP(e01.z, e01.w, t1) FWD_TAP(e23.x, e23.y, t2) FWD_TAP(e23.z, e23.w, t3)
-      FWD_TAP(e45.x, e45.y, t4) FWD_TAP(e45.z, e45.w, t5) FWD_TAP(e67.x, e67.y, t6) FWD_TAP(e67.z, e67.w, t7)
-#undef FWD_TAP
-      rb0 = make_float4(t0, t1, t2, t3);
-      rb1 = make_float4(t4, t5, t6, t7);
     } else {
-      // ---- A
-      if (p.vecA && rowOk && k0 + kA + 8 <= g.K) {
-        ra0 = reinterpret_cast<const float4 *>(aSrc + k0)[0];
-        ra1 = reinterpret_cast<const float4 *>(aSrc + k0)[1];
-      } else {
-        float tmp[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) tmp[i] = (rowOk && k0 + kA + i < g.K) ? aSrc[k0 + i] : 0.f;
-        ra0 = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
-        ra1 = make_float4(tmp[4], tmp[5], tmp[6], tmp[7]);
-      }
-      // ---- B: scalar walk over the 8 taps of this wave
-      int k = k0 + kB;  // scalar
-      int c = k / KK, rem = k - c * KK;
-      int kh = rem / g.kW, kw = rem - kh * g.kW;
       float tmp[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int ih = ih0 + kh, iw = iw0 + kw;
-        const bool ok = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W && (k + i) < g.K;
-        const int soff = ((c * g.H + kh) * g.W + kw) * 4;  // scalar
-        const int off = ok ? posOff + soff : kOob;
-        tmp[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
-        if (++kw == g.kW) {
-          kw = 0;
-          if (++kh == g.kH) {
-            kh = 0;
-            ++c;
-          }
+      for (int i = 0; i < 8; ++i) tmp[i] = (rowOk && k0 + kA + i < g.K) ? aSrc[k0 + i] : 0.f;
+      ra0 = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
+      ra1 = make_float4(tmp[4], tmp[5], tmp[6], tmp[7]);
+    }
+    // ---- B: scalar walk over the 8 taps of this wave
+    int k = k0 + kB;  // scalar
+    int c = k / KK, rem = k - c * KK;
+    int kh = rem / g.kW, kw = rem - kh * g.kW;
+    float tmp[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int ih = ih0 + kh, iw = iw0 + kw;
+      const bool ok = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W && (k + i) < g.K;
+      const int soff = ((c * g.H + kh) * g.W + kw) * 4;  // scalar
+      const int off = ok ? posOff + soff : kOob;
+      tmp[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
+      if (++kw == g.kW) {
+        kw = 0;
+        if (++kh == g.kH) {
+          kh = 0;
+          ++c;
         }
       }
-      rb0 = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
-      rb1 = make_float4(tmp[4], tmp[5], tmp[6], tmp[7]);
     }
+    rb0 = make_float4(tmp[0], tmp[1], tmp[2], tmp[3]);
+    rb1 = make_float4(tmp[4], tmp[5], tmp[6], tmp[7]);
   };
   auto storeTiles = [&](int buf) {
     As[buf][(t & 1) * 2][rowA] = ra0;
@@ -510,39 +551,136 @@ convFwdImplicitKernel(FwdArgs p, ConvGeom g) {
     if (kt + 1 < nkt) storeTiles(buf ^ 1);
     __syncthreads();
   }
+  fwdEpilogue(p, g, acc, blockIdx.x, blockIdx.y, m0, j0, wm, wn, grp, idx);
+}
 
-  // epilogue: lane holds column (lane & 31), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
-  const int rowHalf = grp * 4;
-  if (p.nSplit > 1) {
-    float *dst = p.partial + ((long)blockIdx.x * p.nSplit + blockIdx.y) * (BM * BN);
+// Forward kernel for images that carry their zero border in memory (padH = padW = 0 in g,
+// K % BK == 0, 16-byte loadable weight rows). On this part every ordinary vector-ALU
+// instruction takes issue time away from the MFMA pipe, so the main loop has none:
+//  * a lane's output position is a fixed byte offset in a VGPR, the tap (c, kh, kw) of each k
+//    is a byte offset read from a table with scalar loads and handed to the buffer load as its
+//    scalar offset; every tap of every position is inside the padded image - no bounds test
+//  * weight rows are addressed as fixed VGPR offset + scalar k offset
+//  * the loop is unrolled over the two LDS buffers, so every LDS address is base + immediate
+// Rows past M and columns past the batch are clamped to valid ones and dropped in the epilogue.
+__global__ void __launch_bounds__(dev::kBlock, 3)
+convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
+  __shared__ float4 As[2][BK / 4][FPITCH];
+  __shared__ float4 Bs[2][BK / 4][FPITCH];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tileIdx = p.tile0 + blockIdx.x;
+  const int mTile = tileIdx % p.mTiles, nTile = tileIdx / p.mTiles;
+  const int m0 = mTile * BM, j0 = nTile * BN;
+
+  float16v acc[2][2];
 #pragma unroll
-    for (int tj = 0; tj < 2; ++tj)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int ti = 0; ti < 2; ++ti)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-          dst[(wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3)) * BN + wn * 64 + tj * 32 + idx] = acc[ti][tj][v];
-    return;
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)p.w, 0, p.wBytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.xBytes, 0x00020000);
+  const int rowA = t >> 1, colB = t & 127;
+  const int aOff = (min(m0 + rowA, p.M - 1) * g.K + (t & 1) * 8) * 4;
+  const int kB = __builtin_amdgcn_readfirstlane((t >> 7) * 8);
+  int posOff;
+  {
+    const long lg = min((long)j0 + colB, (long)p.Ncols - 1);
+    const int n = (int)(lg / g.L);
+    const int l = (int)(lg - (long)n * g.L);
+    const int oh = l / g.oW, ow = l - oh * g.oW;
+    posOff = ((n * g.Cin * g.H + oh * g.dH) * g.W + ow * g.dW) * 4;
   }
+  const int ktBegin = blockIdx.y * p.ktPerSplit;
+  const int nkt = min(g.K / BK, ktBegin + p.ktPerSplit);  // this workgroup reduces k-tiles [ktBegin, nkt)
+
+  u32x4 ra0, ra1;
+  unsigned rb[8];
+  // The 8 tap offsets of a wave and k-tile are fetched with scalar loads one tile ahead of their use,
+  // so that no wave waits on the scalar cache inside the loop (the table has BK spare entries at its end).
+  const int4 *tapBase = reinterpret_cast<const int4 *>(p.taps + kB);
+  int4 e0 = tapBase[ktBegin * (BK / 4)], e1 = tapBase[ktBegin * (BK / 4) + 1];
+  auto loadTiles = [&](int kt) {
+    const int k0 = __builtin_amdgcn_readfirstlane(kt * BK);
+    ra0 = __builtin_amdgcn_raw_buffer_load_b128(wr, aOff, k0 * 4, 0);
+    ra1 = __builtin_amdgcn_raw_buffer_load_b128(wr, aOff + 16, k0 * 4, 0);
+    rb[0] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e0.x, 0);
+    rb[1] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e0.y, 0);
+    rb[2] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e0.z, 0);
+    rb[3] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e0.w, 0);
+    rb[4] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e1.x, 0);
+    rb[5] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e1.y, 0);
+    rb[6] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e1.z, 0);
+    rb[7] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e1.w, 0);
+  };
+  auto loadTaps = [&](int kt) { e0 = tapBase[kt * (BK / 4)], e1 = tapBase[kt * (BK / 4) + 1]; };
+  u32x4 *aDst = reinterpret_cast<u32x4 *>(&As[0][(t & 1) * 2][rowA]);
+  u32x4 *bDst = reinterpret_cast<u32x4 *>(&Bs[0][(t >> 7) * 2][colB]);
+  auto storeTiles = [&](auto bufc) {
+    constexpr int o = decltype(bufc)::value * (BK / 4) * FPITCH;
+    aDst[o] = ra0;
+    aDst[o + FPITCH] = ra1;
+    bDst[o] = u32x4{rb[0], rb[1], rb[2], rb[3]};
+    bDst[o + FPITCH] = u32x4{rb[4], rb[5], rb[6], rb[7]};
+  };
+  const int grp = lane >> 5, idx = lane & 31;
+  const float4 *aSrc = &As[0][grp][wm * 64 + idx];
+  const float4 *bSrc = &Bs[0][grp][wn * 64 + idx];
+  auto compute = [&](auto bufc) {
+    constexpr int o = decltype(bufc)::value * (BK / 4) * FPITCH;
+    float4 a[2][2], b[2][2];
 #pragma unroll
-  for (int tj = 0; tj < 2; ++tj) {
-    const long col = (long)j0 + wn * 64 + tj * 32 + idx;
-    if (col >= p.Ncols) continue;
-    const int n = (int)(col / g.L);
-    const int l = (int)(col - (long)n * g.L);
-    float *dst = p.out + (long)n * p.M * g.L + l;
+    for (int s = 0; s < 2; ++s) {
+      a[s][0] = aSrc[o + 2 * s * FPITCH], a[s][1] = aSrc[o + 2 * s * FPITCH + 32];
+      b[s][0] = bSrc[o + 2 * s * FPITCH], b[s][1] = bSrc[o + 2 * s * FPITCH + 32];
+    }
 #pragma unroll
-    for (int ti = 0; ti < 2; ++ti)
+    for (int s = 0; s < 2; ++s) {
+      const float av0[4] = {a[s][0].x, a[s][0].y, a[s][0].z, a[s][0].w}, av1[4] = {a[s][1].x, a[s][1].y, a[s][1].z, a[s][1].w};
+      const float bv0[4] = {b[s][0].x, b[s][0].y, b[s][0].z, b[s][0].w}, bv1[4] = {b[s][1].x, b[s][1].y, b[s][1].z, b[s][1].w};
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
-        if (row < p.M) {
-          float val = acc[ti][tj][v];
-          if (p.bias) val += p.bias[row];
-          dst[(long)row * g.L] = val;
-        }
+      for (int j = 0; j < 4; ++j) {
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv0[j], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv1[j], acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv0[j], acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv1[j], acc[1][1], 0, 0, 0);
       }
+    }
+  };
+  using Buf0 = std::integral_constant<int, 0>;
+  using Buf1 = std::integral_constant<int, 1>;
+
+  loadTiles(ktBegin);
+  loadTaps(ktBegin + 1);
+  storeTiles(Buf0{});
+  __syncthreads();
+  // One k-tile: issue the global loads of the next tile first, then the MFMAs of this one, then
+  // park the loaded tile in the other LDS buffer. The scheduling fences keep the compiler from
+  // sinking the loads below the MFMAs (which would expose their latency at the stores).
+#define FWD_STEP(CUR, NXT, KT_NEXT)            \
+  loadTiles(KT_NEXT);                          \
+  __builtin_amdgcn_sched_barrier(0);           \
+  compute(CUR{});                              \
+  __builtin_amdgcn_sched_barrier(0);           \
+  loadTaps(KT_NEXT + 1);                       \
+  storeTiles(NXT{});                           \
+  __syncthreads();
+  int kt = ktBegin;
+  for (; kt + 2 < nkt; kt += 2) {  // tile kt sits in buffer 0
+    FWD_STEP(Buf0, Buf1, kt + 1)
+    FWD_STEP(Buf1, Buf0, kt + 2)
   }
+  if (kt + 2 == nkt) {  // two tiles left
+    FWD_STEP(Buf0, Buf1, kt + 1)
+    compute(Buf1{});
+  } else {
+    compute(Buf0{});
+  }
+#undef FWD_STEP
+  fwdEpilogue(p, g, acc, blockIdx.x, blockIdx.y, m0, j0, wm, wn, grp, idx);
 }
 
 // out tile = bias + sum over the nSplit partial tiles (ascending split order).
@@ -575,18 +713,21 @@ fwdTailFixupKernel(FwdArgs p, ConvGeom g) {
 
 // ---- weight gradient, second generation ------------------------------------------
 // partial[split][o][k] = sum over the split's positions r = (n, l) of gy[n][o][l] * col[k][n,l].
-// Same MFMA core and float4 operand layout as the forward kernel, with the reduction
+// Same MFMA core and float4 operand layout as the forward kernels, with the reduction
 // running over positions: 4 consecutive l of one gradOutput row are already a float4
 // in memory (L % 4 == 0), so the A tile goes from 16-byte buffer loads to
 // ds_write_b128 without a transpose. For the B tile a lane owns one position of the
-// k-tile and 8 columns k; the columns never change, so their taps (c, kh, kw) are
-// resolved once into registers and each k-tile costs one position decomposition per
-// lane. 16 consecutive lanes gather 16 consecutive positions (64-byte runs of x).
+// k-tile and 8 columns k; the columns never change, so their tap offsets are resolved
+// once into registers, the images carry their zero border in memory (no bounds test)
+// and a gather costs one add per element on top of one position update per k-tile.
+// 16 consecutive lanes gather 16 consecutive positions (64-byte runs of x).
+// L16: L % 16 == 0 - a k-tile never crosses an image, so the gradOutput offsets are a
+// fixed VGPR part plus a scalar part.
 constexpr int GPITCH = BN + 4;  // float4 per position-group row of Bs: the 4 groups of a wave's scalar stores hit disjoint banks
 
 struct GradWeightArgs {
   const float *gy;  // (N, M, L)
-  const float *x;   // (N, Cin, H, W)
+  const float *x;   // (N, Cin, H, W) of g: images with their zero border
   float *partial;   // (splits, M, Ncols)
   int M, Ncols;     // Cout, K
   int mTiles, nTiles;
@@ -595,7 +736,8 @@ struct GradWeightArgs {
   unsigned magicOW;
 };
 
-__global__ void __launch_bounds__(dev::kBlock)
+template <bool L16>
+__global__ void __launch_bounds__(dev::kBlock, 3)
 convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   __shared__ float4 As[2][BK / 4][FPITCH];
   __shared__ float4 Bs[2][BK / 4][GPITCH];
@@ -624,87 +766,92 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   const int rowA = t >> 1;
   const int rowOffA = min(m0 + rowA, p.M - 1) * g.L * 4;  // rows past M are clamped and dropped in the epilogue
   const int imgStrideA = p.M * g.L * 4;
-  int nA, lA;
+  int nA, lA;  // L16: scalar image and position of the k-tile; else: of this lane's first group
   {
-    const long r = (long)ktBegin * BK + (t & 1) * 8;
+    const long r = (long)ktBegin * BK + (L16 ? 0 : (t & 1) * 8);
     nA = (int)(r / g.L);
     lA = (int)(r - (long)nA * g.L);
   }
   // ---- B loader: position t & 15 of the k-tile, columns (t >> 4) + 16 i
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.xBytes, 0x00020000);
   const int rB = t & 15, cB = t >> 4;
-  int tapOff[8], tapHW[8];
+  int tapOff[8];
   {
     const int KK = g.kH * g.kW;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int k = j0 + cB + 16 * i;
+      const int k = min(j0 + cB + 16 * i, p.Ncols - 1);  // columns past K are dropped in the epilogue
       const int c = k / KK, rem = k - c * KK;
       const int kh = rem / g.kW, kw = rem - kh * g.kW;
       tapOff[i] = ((c * g.H + kh) * g.W + kw) * 4;
-      tapHW[i] = k < p.Ncols ? (kh << 16) | kw : 0x4000 << 16;  // columns past K fail the row test
     }
   }
-  int nB, lB;
+  const int imgStrideB = g.Cin * g.H * g.W * 4;
+  const int rowStepB = g.dH * g.W * 4, colStepB = g.dW * 4;
+  int lB, nOffB;  // position inside the image, byte offset of the image (>= xBytes past the batch: loads return 0)
   {
     const long r = (long)ktBegin * BK + rB;
-    nB = (int)(r / g.L);
-    lB = (int)(r - (long)nB * g.L);
+    const int n = (int)(r / g.L);
+    lB = (int)(r - (long)n * g.L);
+    nOffB = n * imgStrideB;
   }
-  const int imgStrideB = g.Cin * g.H * g.W * 4;
 
-  float4 ra0, ra1;
-  float rb[8];
+  u32x4 ra0, ra1;
+  unsigned rb[8];
   // loads the k-tile the position counters stand on, then advances them by BK (L >= BK: one wrap at most)
   auto loadTiles = [&]() {
-    {
+    if constexpr (L16) {
+      // N*L is a multiple of BK here, so every k-tile lies inside the batch (the scalar offset is not range-checked)
+      const int so = __builtin_amdgcn_readfirstlane(nA * imgStrideA + lA * 4);
+      ra0 = __builtin_amdgcn_raw_buffer_load_b128(gr, rowOffA + (t & 1) * 32, so, 0);
+      ra1 = __builtin_amdgcn_raw_buffer_load_b128(gr, rowOffA + (t & 1) * 32 + 16, so, 0);
+      lA += BK;
+      if (lA >= g.L) lA -= g.L, ++nA;
+    } else {
       int n1 = nA, l1 = lA + 4;
       if (l1 >= g.L) l1 -= g.L, ++n1;
       const int o0 = nA < g.N ? nA * imgStrideA + rowOffA + lA * 4 : kOob;
       const int o1 = n1 < g.N ? n1 * imgStrideA + rowOffA + l1 * 4 : kOob;
-      ra0 = dev::bufLoad4(gr, o0);
-      ra1 = dev::bufLoad4(gr, o1);
+      ra0 = __builtin_amdgcn_raw_buffer_load_b128(gr, o0, 0, 0);
+      ra1 = __builtin_amdgcn_raw_buffer_load_b128(gr, o1, 0, 0);
       lA += BK;
       if (lA >= g.L) lA -= g.L, ++nA;
     }
     {
       const int oh = dev::fastDiv(lB, p.magicOW), ow = lB - oh * g.oW;
-      const int ih0 = nB < g.N ? oh * g.dH - g.padH : -(1 << 28);
-      const int iw0 = ow * g.dW - g.padW;
-      const int posOff = nB * imgStrideB + (ih0 * g.W + iw0) * 4;  // only used when the tap is inside the image
+      const int posOff = nOffB + oh * rowStepB + ow * colStepB;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int ih = ih0 + (tapHW[i] >> 16), iw = iw0 + (tapHW[i] & 0xffff);
-        const bool ok = ((unsigned)ih < (unsigned)g.H) & ((unsigned)iw < (unsigned)g.W);
-        rb[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, ok ? posOff + tapOff[i] : kOob, 0, 0));
-      }
+      for (int i = 0; i < 8; ++i)
+        rb[i] = __builtin_amdgcn_raw_buffer_load_b32(xr, (int)((unsigned)posOff + (unsigned)tapOff[i]), 0, 0);
       lB += BK;
-      if (lB >= g.L) lB -= g.L, ++nB;
+      if (lB >= g.L) lB -= g.L, nOffB += imgStrideB;
     }
   };
-  auto storeTiles = [&](int buf) {
-    As[buf][(t & 1) * 2][rowA] = ra0;
-    As[buf][(t & 1) * 2 + 1][rowA] = ra1;
-    float *b = reinterpret_cast<float *>(&Bs[buf][rB >> 2][cB]) + (rB & 3);
+  u32x4 *aDst = reinterpret_cast<u32x4 *>(&As[0][(t & 1) * 2][rowA]);
+  unsigned *bDst = reinterpret_cast<unsigned *>(&Bs[0][rB >> 2][cB]) + (rB & 3);
+  auto storeTiles = [&](auto bufc) {
+    constexpr int buf = decltype(bufc)::value;
+    aDst[buf * (BK / 4) * FPITCH] = ra0;
+    aDst[buf * (BK / 4) * FPITCH + FPITCH] = ra1;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) b[64 * i] = rb[i];  // column + 16 = 16 float4 further
+    for (int i = 0; i < 8; ++i) bDst[buf * (BK / 4) * GPITCH * 4 + 64 * i] = rb[i];  // column + 16 = 16 float4 further
   };
-
-  if (ktBegin < ktEnd) {
-    loadTiles();
-    storeTiles(0);
-  }
-  __syncthreads();
   const int grp = lane >> 5, idx = lane & 31;
-  for (int kt = ktBegin; kt < ktEnd; ++kt) {
-    const int buf = (kt - ktBegin) & 1;
-    if (kt + 1 < ktEnd) loadTiles();
+  const float4 *aSrc = &As[0][grp][wm * 64 + idx];
+  const float4 *bSrc = &Bs[0][grp][wn * 64 + idx];
+  auto compute = [&](auto bufc) {
+    constexpr int buf = decltype(bufc)::value;
+    constexpr int oa = buf * (BK / 4) * FPITCH, ob = buf * (BK / 4) * GPITCH;
+    float4 a[2][2], b[2][2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const float4 a0 = As[buf][2 * s + grp][wm * 64 + idx], a1 = As[buf][2 * s + grp][wm * 64 + 32 + idx];
-      const float4 b0 = Bs[buf][2 * s + grp][wn * 64 + idx], b1 = Bs[buf][2 * s + grp][wn * 64 + 32 + idx];
-      const float av0[4] = {a0.x, a0.y, a0.z, a0.w}, av1[4] = {a1.x, a1.y, a1.z, a1.w};
-      const float bv0[4] = {b0.x, b0.y, b0.z, b0.w}, bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+      a[s][0] = aSrc[oa + 2 * s * FPITCH], a[s][1] = aSrc[oa + 2 * s * FPITCH + 32];
+      b[s][0] = bSrc[ob + 2 * s * GPITCH], b[s][1] = bSrc[ob + 2 * s * GPITCH + 32];
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const float av0[4] = {a[s][0].x, a[s][0].y, a[s][0].z, a[s][0].w}, av1[4] = {a[s][1].x, a[s][1].y, a[s][1].z, a[s][1].w};
+      const float bv0[4] = {b[s][0].x, b[s][0].y, b[s][0].z, b[s][0].w}, bv1[4] = {b[s][1].x, b[s][1].y, b[s][1].z, b[s][1].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv0[j], acc[0][0], 0, 0, 0);
@@ -713,9 +860,34 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
         acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv1[j], acc[1][1], 0, 0, 0);
       }
     }
-    if (kt + 1 < ktEnd) storeTiles(buf ^ 1);
+  };
+  using Buf0 = std::integral_constant<int, 0>;
+  using Buf1 = std::integral_constant<int, 1>;
+
+#define GW_STEP(CUR, NXT)            \
+  loadTiles();                       \
+  __builtin_amdgcn_sched_barrier(0); \
+  compute(CUR{});                    \
+  __builtin_amdgcn_sched_barrier(0); \
+  storeTiles(NXT{});                 \
+  __syncthreads();
+  if (ktBegin < ktEnd) {
+    loadTiles();
+    storeTiles(Buf0{});
     __syncthreads();
+    int kt = ktBegin;
+    for (; kt + 2 < ktEnd; kt += 2) {  // tile kt sits in buffer 0
+      GW_STEP(Buf0, Buf1)
+      GW_STEP(Buf1, Buf0)
+    }
+    if (kt + 2 == ktEnd) {  // two tiles left
+      GW_STEP(Buf0, Buf1)
+      compute(Buf1{});
+    } else {
+      compute(Buf0{});
+    }
   }
+#undef GW_STEP
 
   // lane holds column (lane & 31), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
   float *dst = p.partial + (long)split * p.M * p.Ncols;
@@ -941,8 +1113,9 @@ bool forceGeneric() {
 // over all CUs (partials in scratch, folded by fwdTailFixupKernel in a fixed order).
 struct FwdPlan {
   int mTiles, total, full, tail, nSplit, ktPerSplit;
-  int tapEntries;      // > 0: the FAST kernel applies; entries of the tap table at the start of the scratch
-  long scratchFloats;  // tap table (2 ints per entry) followed by the tail partials
+  int tapEntries;      // > 0: the padded kernel applies; entries of the tap table at the start of the scratch
+  long paddedFloats;   // floats of the zero-bordered copy of the images (0: no border needed, or generic kernel)
+  long scratchFloats;  // tap table, tail partials, padded images
 };
 FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
   FwdPlan pl{};
@@ -959,8 +1132,11 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
   pl.full = pl.total - pl.tail;
   pl.ktPerSplit = launch::ceilDiv(nkt, nSplit);
   pl.nSplit = launch::ceilDiv(nkt, pl.ktPerSplit);
-  pl.tapEntries = (g.K % BK == 0 && g.K % 4 == 0 && g.kH < 0x4000 && g.kW < 0x4000) ? nkt * BK : 0;
-  pl.scratchFloats = 2L * pl.tapEntries + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0);
+  const long padded = (long)nImages * g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW);
+  const bool fast = !forceGeneric() && g.K % BK == 0 && padded * 4 < 0x7fffffffL && (long)M * g.K * 4 < 0x7fffffffL;
+  pl.tapEntries = fast ? g.K + BK : 0;  // BK spare entries: the kernel reads one k-tile ahead
+  pl.paddedFloats = fast && (g.padH > 0 || g.padW > 0) ? padded : 0;
+  pl.scratchFloats = pl.tapEntries + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0) + pl.paddedFloats;
   return pl;
 }
 
@@ -968,30 +1144,38 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
 void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const float *w, const float *x, float *out,
                        const float *bias, int M, int nImages, const ConvGeom &g) {
   const bool fast = pl.tapEntries > 0 && launch::aligned16(w) && launch::aligned16(scratch);
-  float *partial = scratch + 2L * pl.tapEntries;
+  float *partial = scratch + pl.tapEntries;
+  ConvGeom gk = g;  // geometry the kernel sees
+  FwdArgs p{};
+  p.x = x;
   if (fast) {
+    gk.H = g.H + 2 * g.padH, gk.W = g.W + 2 * g.padW, gk.padH = gk.padW = 0;
+    if (pl.paddedFloats > 0) {
+      float *xp = partial + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0);
+      launchPadPlanes(s, x, xp, (long)nImages * g.Cin, g.H, g.W, g.padH, g.padW);
+      p.x = xp;
+    }
     buildTapTableKernel<<<launch::directGrid(pl.tapEntries, dev::kBlock), dev::kBlock, 0, s>>>(
-        reinterpret_cast<int2 *>(scratch), pl.tapEntries, g);
+        reinterpret_cast<int *>(scratch), pl.tapEntries, gk);
     THC_HIP_CHECK(hipGetLastError());
   }
-  FwdArgs p{};
-  p.taps = reinterpret_cast<const int2 *>(scratch);
+  p.taps = reinterpret_cast<const int *>(scratch);
   p.w = w;
-  p.x = x;
   p.out = out;
   p.bias = bias;
   p.M = M;
   p.Ncols = nImages * g.L;
   p.mTiles = pl.mTiles;
-  p.xBytes = (int)((long)nImages * g.Cin * g.H * g.W * sizeof(float));
+  p.xBytes = (int)((long)nImages * gk.Cin * gk.H * gk.W * sizeof(float));
+  p.wBytes = (int)((long)M * g.K * sizeof(float));
   p.vecA = (g.K % 4 == 0) && launch::aligned16(w);
   p.nSplit = 1;
   p.ktPerSplit = launch::ceilDiv(g.K, BK);
   if (pl.full > 0) {
     if (fast)
-      convFwdImplicitKernel<true><<<dim3(pl.full), dev::kBlock, 0, s>>>(p, g);
+      convFwdPaddedKernel<<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
     else
-      convFwdImplicitKernel<false><<<dim3(pl.full), dev::kBlock, 0, s>>>(p, g);
+      convFwdImplicitKernel<<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
     THC_HIP_CHECK(hipGetLastError());
   }
   if (pl.tail > 0) {
@@ -1000,11 +1184,11 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
     p.nSplit = pl.nSplit;
     p.partial = partial;
     if (fast)
-      convFwdImplicitKernel<true><<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, g);
+      convFwdPaddedKernel<<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, gk);
     else
-      convFwdImplicitKernel<false><<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, g);
+      convFwdImplicitKernel<<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, gk);
     THC_HIP_CHECK(hipGetLastError());
-    fwdTailFixupKernel<<<dim3(pl.tail, BM * BN / (4 * dev::kBlock)), dev::kBlock, 0, s>>>(p, g);
+    fwdTailFixupKernel<<<dim3(pl.tail, BM * BN / (4 * dev::kBlock)), dev::kBlock, 0, s>>>(p, gk);
     THC_HIP_CHECK(hipGetLastError());
   }
 }
@@ -1044,7 +1228,7 @@ void THNN_CudaSpatialConvolutionMM_updateOutput(THCState *state, THCudaTensor *i
   hipStream_t s = state->stream;
   // images per launch so that the flat column index n*L + l fits an int
   int group = (int)std::min<long>(g.N, std::max<long>(1, 0x7fffffffL / 2 / g.L));
-  const long imgBytes = (long)g.Cin * g.H * g.W * sizeof(float);
+  const long imgBytes = (long)g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW) * sizeof(float);  // with its zero border
   const bool implicit2 = !forceGeneric() && imgBytes < (1L << 30);
   if (implicit2) group = (int)std::min<long>(group, std::max<long>(1, ((1L << 31) - 1 - 4096) / imgBytes));
   if (implicit2) {
@@ -1100,7 +1284,8 @@ void THNN_CudaSpatialConvolutionMM_updateGradInput(THCState *state, THCudaTensor
   // Stride 1: gradInput is a forward convolution of gradOutput with the flipped,
   // transposed weights and padding k-1-pad, so it runs on the implicit-GEMM
   // forward kernel and no gradient columns ever reach memory.
-  const long goImgBytes = (long)g.Cout * g.L * sizeof(float);
+  const long goImgBytes =
+      (long)g.Cout * (g.oH + 2 * (g.kH - 1 - g.padH)) * (g.oW + 2 * (g.kW - 1 - g.padW)) * sizeof(float);  // with its zero border
   if (g.dH == 1 && g.dW == 1 && g.padH <= g.kH - 1 && g.padW <= g.kW - 1 && !forceGeneric() &&
       goImgBytes < (1L << 30)) {
     ConvGeom t = g;  // the transposed problem
@@ -1187,29 +1372,36 @@ void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTens
   const int mT = (int)tiles(g.Cout, BM), nT = (int)tiles(g.K, BN);
   const int totalKt = launch::ceilDiv(g.N * g.L, BK);
   // second-generation kernel: gradOutput rows loadable as float4 groups, 32-bit byte offsets into both operands
-  const long gyBytes = (long)g.N * g.Cout * g.L * 4, xBytes = (long)g.N * g.Cin * g.H * g.W * 4;
+  const bool bordered = g.padH > 0 || g.padW > 0;
+  const long gyBytes = (long)g.N * g.Cout * g.L * 4;
+  const long xpFloats = (long)g.N * g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW);
   const bool fast = !forceGeneric() && g.L % 4 == 0 && g.L >= BK && launch::aligned16(go.ptr()) &&
-                    gyBytes < 0x7fffffffL && xBytes < 0x7fffffffL && g.kH < 0x4000 && g.kW < 0x4000 &&
-                    (long)g.L * g.oW < 0x7fffffffL;
-  const int slots = residentSlots(fast ? (const void *)convGradWeightKernel : (const void *)convGemmKernel<kGradWeight>);
+                    gyBytes < 0x7fffffffL && xpFloats * 4 < 0x7fffffffL - 65536 && (long)g.L * g.oW < 0x7fffffffL;
+  const bool l16 = g.L % BK == 0;
+  const void *kern = !fast ? (const void *)convGemmKernel<kGradWeight>
+                     : l16 ? (const void *)convGradWeightKernel<true>
+                           : (const void *)convGradWeightKernel<false>;
+  const int slots = residentSlots(kern);
   int splits = std::max(1, std::min(totalKt, slots / (mT * nT)));
   const int perSplit = launch::ceilDiv(totalKt, splits);
   splits = launch::ceilDiv(totalKt, perSplit);
   const long count = (long)g.Cout * g.K;
+  // scratch: the splits' partial products, then (second-generation kernel) the images with their zero border
+  const long partialFloats = (splits * count + 3) / 4 * 4;
   Temp tmp;
-  float *partial;
-  if (columns) {
-    resize(state, columns, {(long)splits * g.Cout, g.K});
-    if (!isContiguous(erase(columns))) error("columns tensor has to be contiguous");
-    partial = data(columns);
-  } else {
-    tmp = Temp(s, (size_t)splits * count * sizeof(float));
-    partial = (float *)tmp.get();
-  }
+  float *partial = scratchFloats(state, columns, partialFloats + (fast && bordered ? xpFloats : 0), tmp, "columns");
   if (fast) {
+    ConvGeom gk = g;
+    const float *xk = in.ptr();
+    if (bordered) {
+      float *xp = partial + partialFloats;
+      launchPadPlanes(s, in.ptr(), xp, (long)g.N * g.Cin, g.H, g.W, g.padH, g.padW);
+      gk.H = g.H + 2 * g.padH, gk.W = g.W + 2 * g.padW, gk.padH = gk.padW = 0;
+      xk = xp;
+    }
     GradWeightArgs q{};
     q.gy = go.ptr();
-    q.x = in.ptr();
+    q.x = xk;
     q.partial = partial;
     q.M = g.Cout;
     q.Ncols = g.K;
@@ -1218,9 +1410,12 @@ void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTens
     q.totalKt = totalKt;
     q.ktPerSplit = perSplit;
     q.gyBytes = (int)gyBytes;
-    q.xBytes = (int)xBytes;
+    q.xBytes = (int)(xpFloats * 4);
     q.magicOW = dev::magicOf(g.oW);
-    convGradWeightKernel<<<dim3(mT * nT * splits), dev::kBlock, 0, s>>>(q, g);
+    if (l16)
+      convGradWeightKernel<true><<<dim3(mT * nT * splits), dev::kBlock, 0, s>>>(q, gk);
+    else
+      convGradWeightKernel<false><<<dim3(mT * nT * splits), dev::kBlock, 0, s>>>(q, gk);
   } else {
     GemmArgs p{};
     p.a = go.ptr();

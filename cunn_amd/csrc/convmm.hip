@@ -554,6 +554,24 @@ convFwdImplicitKernel(FwdArgs p, ConvGeom g) {
   fwdEpilogue(p, g, acc, blockIdx.x, blockIdx.y, m0, j0, wm, wn, grp, idx);
 }
 
+// One half of a k-tile for one wave: 4 ds_read_b128 (two k-groups... one per lane group) and 16 MFMAs.
+// aSrc / bSrc point at the lane's operands of k-group (lane / 32) in buffer 0; OA / OB are the float4
+// offsets of the buffer and super-step, compile-time so that they fold into the LDS instruction.
+template <int OA, int OB>
+__device__ __forceinline__ void mfmaHalf(const float4 *aSrc, const float4 *bSrc, float16v (&acc)[2][2]) {
+  const float4 a0 = aSrc[OA], a1 = aSrc[OA + 32];
+  const float4 b0 = bSrc[OB], b1 = bSrc[OB + 32];
+  const float av0[4] = {a0.x, a0.y, a0.z, a0.w}, av1[4] = {a1.x, a1.y, a1.z, a1.w};
+  const float bv0[4] = {b0.x, b0.y, b0.z, b0.w}, bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv0[j], acc[0][0], 0, 0, 0);
+    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv1[j], acc[0][1], 0, 0, 0);
+    acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv0[j], acc[1][0], 0, 0, 0);
+    acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv1[j], acc[1][1], 0, 0, 0);
+  }
+}
+
 // Forward kernel for images that carry their zero border in memory (padH = padW = 0 in g,
 // K % BK == 0, 16-byte loadable weight rows). On this part every ordinary vector-ALU
 // instruction takes issue time away from the MFMA pipe, so the main loop has none:
@@ -629,57 +647,49 @@ convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
   const int grp = lane >> 5, idx = lane & 31;
   const float4 *aSrc = &As[0][grp][wm * 64 + idx];
   const float4 *bSrc = &Bs[0][grp][wn * 64 + idx];
-  auto compute = [&](auto bufc) {
-    constexpr int o = decltype(bufc)::value * (BK / 4) * FPITCH;
-    float4 a[2][2], b[2][2];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      a[s][0] = aSrc[o + 2 * s * FPITCH], a[s][1] = aSrc[o + 2 * s * FPITCH + 32];
-      b[s][0] = bSrc[o + 2 * s * FPITCH], b[s][1] = bSrc[o + 2 * s * FPITCH + 32];
-    }
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const float av0[4] = {a[s][0].x, a[s][0].y, a[s][0].z, a[s][0].w}, av1[4] = {a[s][1].x, a[s][1].y, a[s][1].z, a[s][1].w};
-      const float bv0[4] = {b[s][0].x, b[s][0].y, b[s][0].z, b[s][0].w}, bv1[4] = {b[s][1].x, b[s][1].y, b[s][1].z, b[s][1].w};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv0[j], acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv1[j], acc[0][1], 0, 0, 0);
-        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv0[j], acc[1][0], 0, 0, 0);
-        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv1[j], acc[1][1], 0, 0, 0);
-      }
-    }
-  };
   using Buf0 = std::integral_constant<int, 0>;
   using Buf1 = std::integral_constant<int, 1>;
+  constexpr int BUFA = (BK / 4) * FPITCH;  // float4 per LDS buffer
+
+  // Software pipeline. While tile kt is multiplied out of one LDS buffer, tile kt + 1 waits in
+  // registers and tile kt + 2 is requested from memory:
+  //   first 16 MFMAs of kt | registers (kt + 1) -> other LDS buffer, global loads of kt + 2 |
+  //   last 16 MFMAs of kt | barrier
+  // The LDS stores and the load issue sit between the two MFMA halves, so the matrix pipe has
+  // queued work while they run and the only stall left at the barrier is the LDS read latency.
+  // The scheduling fences pin that order.
+  auto step = [&](auto cur, auto nxt, int kt, bool store, bool load) {
+    constexpr int C = decltype(cur)::value, N = decltype(nxt)::value;
+    mfmaHalf<C * BUFA, C * BUFA>(aSrc, bSrc, acc);
+    __builtin_amdgcn_sched_barrier(0);
+    if (store) storeTiles(nxt);
+    if (load) {
+      loadTiles(kt + 2);
+      loadTaps(kt + 3);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    mfmaHalf<C * BUFA + 2 * FPITCH, C * BUFA + 2 * FPITCH>(aSrc, bSrc, acc);
+    (void)N;
+    __syncthreads();
+  };
 
   loadTiles(ktBegin);
   loadTaps(ktBegin + 1);
   storeTiles(Buf0{});
-  __syncthreads();
-  // One k-tile: issue the global loads of the next tile first, then the MFMAs of this one, then
-  // park the loaded tile in the other LDS buffer. The scheduling fences keep the compiler from
-  // sinking the loads below the MFMAs (which would expose their latency at the stores).
-#define FWD_STEP(CUR, NXT, KT_NEXT)            \
-  loadTiles(KT_NEXT);                          \
-  __builtin_amdgcn_sched_barrier(0);           \
-  compute(CUR{});                              \
-  __builtin_amdgcn_sched_barrier(0);           \
-  loadTaps(KT_NEXT + 1);                       \
-  storeTiles(NXT{});                           \
+  if (ktBegin + 1 < nkt) {
+    loadTiles(ktBegin + 1);
+    loadTaps(ktBegin + 2);
+  }
   __syncthreads();
   int kt = ktBegin;
-  for (; kt + 2 < nkt; kt += 2) {  // tile kt sits in buffer 0
-    FWD_STEP(Buf0, Buf1, kt + 1)
-    FWD_STEP(Buf1, Buf0, kt + 2)
+  for (; kt + 3 < nkt; kt += 2) {  // tile kt sits in buffer 0, tile kt + 1 in registers
+    step(Buf0{}, Buf1{}, kt, true, true);
+    step(Buf1{}, Buf0{}, kt + 1, true, true);
   }
-  if (kt + 2 == nkt) {  // two tiles left
-    FWD_STEP(Buf0, Buf1, kt + 1)
-    compute(Buf1{});
-  } else {
-    compute(Buf0{});
-  }
-#undef FWD_STEP
+  // one to three tiles left
+  step(Buf0{}, Buf1{}, kt, kt + 1 < nkt, kt + 2 < nkt);
+  if (kt + 1 < nkt) step(Buf1{}, Buf0{}, kt + 1, kt + 2 < nkt, false);
+  if (kt + 2 < nkt) step(Buf0{}, Buf1{}, kt + 2, false, false);
   fwdEpilogue(p, g, acc, blockIdx.x, blockIdx.y, m0, j0, wm, wn, grp, idx);
 }
 
@@ -839,55 +849,36 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   const int grp = lane >> 5, idx = lane & 31;
   const float4 *aSrc = &As[0][grp][wm * 64 + idx];
   const float4 *bSrc = &Bs[0][grp][wn * 64 + idx];
-  auto compute = [&](auto bufc) {
-    constexpr int buf = decltype(bufc)::value;
-    constexpr int oa = buf * (BK / 4) * FPITCH, ob = buf * (BK / 4) * GPITCH;
-    float4 a[2][2], b[2][2];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      a[s][0] = aSrc[oa + 2 * s * FPITCH], a[s][1] = aSrc[oa + 2 * s * FPITCH + 32];
-      b[s][0] = bSrc[ob + 2 * s * GPITCH], b[s][1] = bSrc[ob + 2 * s * GPITCH + 32];
-    }
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const float av0[4] = {a[s][0].x, a[s][0].y, a[s][0].z, a[s][0].w}, av1[4] = {a[s][1].x, a[s][1].y, a[s][1].z, a[s][1].w};
-      const float bv0[4] = {b[s][0].x, b[s][0].y, b[s][0].z, b[s][0].w}, bv1[4] = {b[s][1].x, b[s][1].y, b[s][1].z, b[s][1].w};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv0[j], acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv1[j], acc[0][1], 0, 0, 0);
-        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv0[j], acc[1][0], 0, 0, 0);
-        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv1[j], acc[1][1], 0, 0, 0);
-      }
-    }
-  };
   using Buf0 = std::integral_constant<int, 0>;
   using Buf1 = std::integral_constant<int, 1>;
+  constexpr int BUFA = (BK / 4) * FPITCH, BUFB = (BK / 4) * GPITCH;  // float4 per LDS buffer
 
-#define GW_STEP(CUR, NXT)            \
-  loadTiles();                       \
-  __builtin_amdgcn_sched_barrier(0); \
-  compute(CUR{});                    \
-  __builtin_amdgcn_sched_barrier(0); \
-  storeTiles(NXT{});                 \
-  __syncthreads();
+  // same software pipeline as the forward kernel: tile kt in LDS, kt + 1 in registers, kt + 2 requested
+  auto step = [&](auto cur, auto nxt, bool store, bool load) {
+    constexpr int C = decltype(cur)::value;
+    mfmaHalf<C * BUFA, C * BUFB>(aSrc, bSrc, acc);
+    __builtin_amdgcn_sched_barrier(0);
+    if (store) storeTiles(nxt);
+    if (load) loadTiles();
+    __builtin_amdgcn_sched_barrier(0);
+    mfmaHalf<C * BUFA + 2 * FPITCH, C * BUFB + 2 * GPITCH>(aSrc, bSrc, acc);
+    __syncthreads();
+  };
   if (ktBegin < ktEnd) {
     loadTiles();
     storeTiles(Buf0{});
+    if (ktBegin + 1 < ktEnd) loadTiles();
     __syncthreads();
     int kt = ktBegin;
-    for (; kt + 2 < ktEnd; kt += 2) {  // tile kt sits in buffer 0
-      GW_STEP(Buf0, Buf1)
-      GW_STEP(Buf1, Buf0)
+    for (; kt + 3 < ktEnd; kt += 2) {  // tile kt sits in buffer 0, tile kt + 1 in registers
+      step(Buf0{}, Buf1{}, true, true);
+      step(Buf1{}, Buf0{}, true, true);
     }
-    if (kt + 2 == ktEnd) {  // two tiles left
-      GW_STEP(Buf0, Buf1)
-      compute(Buf1{});
-    } else {
-      compute(Buf0{});
-    }
+    // one to three tiles left
+    step(Buf0{}, Buf1{}, kt + 1 < ktEnd, kt + 2 < ktEnd);
+    if (kt + 1 < ktEnd) step(Buf1{}, Buf0{}, kt + 2 < ktEnd, false);
+    if (kt + 2 < ktEnd) step(Buf0{}, Buf1{}, false, false);
   }
-#undef GW_STEP
 
   // lane holds column (lane & 31), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
   float *dst = p.partial + (long)split * p.M * p.Ncols;
@@ -1134,7 +1125,7 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
   pl.nSplit = launch::ceilDiv(nkt, pl.ktPerSplit);
   const long padded = (long)nImages * g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW);
   const bool fast = !forceGeneric() && g.K % BK == 0 && padded * 4 < 0x7fffffffL && (long)M * g.K * 4 < 0x7fffffffL;
-  pl.tapEntries = fast ? g.K + BK : 0;  // BK spare entries: the kernel reads one k-tile ahead
+  pl.tapEntries = fast ? g.K + 2 * BK : 0;  // spare entries: the kernel reads tap offsets up to two k-tiles ahead
   pl.paddedFloats = fast && (g.padH > 0 || g.padW > 0) ? padded : 0;
   pl.scratchFloats = pl.tapEntries + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0) + pl.paddedFloats;
   return pl;

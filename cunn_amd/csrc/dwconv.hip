@@ -36,6 +36,7 @@ struct DwGeom {
   int nblk;           // grid size
   int nslots;         // N * tilesPerPlane (accGradParameters partials per (c,j) and tap)
   unsigned magicTiles, magicC;  // dev::magicOf(tilesPerPlane), dev::magicOf(C): used by the strip kernels
+  unsigned magicOW4, magicW4;   // dev::magicOf(oW / 4), dev::magicOf(W / 4)
 };
 
 // (plane, tile, channel) of a workgroup of the strip kernels
@@ -43,7 +44,7 @@ struct BlockPos {
   int plane, tile, c;
 };
 __device__ __forceinline__ BlockPos blockPos(const DwGeom &g) {
-  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int bid = blockIdx.x;  // consecutive workgroups work on neighbouring planes: one compact window of memory in flight
   BlockPos b;
   b.plane = g.tilesPerPlane == 1 ? bid : dev::fastDiv(bid, g.magicTiles);
   b.tile = bid - b.plane * g.tilesPerPlane;
@@ -378,7 +379,10 @@ dwAccGradDirect(const float *__restrict__ in, const float *__restrict__ gradOut,
 // index inside the window is a compile-time constant, so the inner loops are
 // straight-line FMAs on registers.
 
-template <int KS, int ST>
+// ONE: depth multiplier 1 and the band is a single load batch (at most kLoadBatch 16-byte loads
+// per lane) - its loads are issued before anything else and the taps and bias are fetched while
+// they are in flight.
+template <int KS, int ST, bool ONE>
 __global__ void __launch_bounds__(dev::kBlock)
 dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strides4 ws,
            const float *__restrict__ bias, Strides2 bs, float *__restrict__ out, DwGeom g) {
@@ -391,18 +395,27 @@ dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strid
   const int nOut = min(g.tileRows, g.oH - oh0);
   const int nIn = (nOut - 1) * ST + KS;
   const int pitch = S::pitch(g.W);
-  S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
+  typename S::InFlight fl;
+  if (ONE) S::issue(fl, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
+  float w[KS * KS];
+  loadTaps<KS>(weight, ws, 0, c, w);
+  float b = bias ? bias[c * bs.s1] : 0.f;
+  if (ONE)
+    S::commit(smem, fl, g.W, nIn);
+  else
+    S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
   __syncthreads();
   const int oW4 = g.oW >> 2;
-  const unsigned magicOw4 = dev::magicOf(oW4);
   const int total = nOut * oW4;
-  for (int j = 0; j < g.M; ++j) {
-    float w[KS * KS];
-    loadTaps<KS>(weight, ws, j, c, w);
-    const float b = bias ? bias[j * bs.s0 + c * bs.s1] : 0.f;
-    float *o = out + (((long)plane * g.M + j) * g.oH + oh0) * g.oW;
+  const int nMul = ONE ? 1 : g.M;
+  for (int j = 0; j < nMul; ++j) {
+    if (!ONE && j > 0) {
+      loadTaps<KS>(weight, ws, j, c, w);
+      b = bias ? bias[j * bs.s0 + c * bs.s1] : 0.f;
+    }
+    float *o = out + (((long)plane * nMul + j) * g.oH + oh0) * g.oW;
     for (int i = threadIdx.x; i < total; i += blockDim.x) {
-      const int r = dev::fastDiv(i, magicOw4), b4 = i - r * oW4;
+      const int r = dev::fastDiv(i, g.magicOW4), b4 = i - r * oW4;
       const float *p = smem + r * ST * pitch;
       float acc[4] = {b, b, b, b};
 #pragma unroll
@@ -423,7 +436,8 @@ dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strid
 // 4b .. 4b+3). The gradOutput rows are staged zero-padded, so no tap needs a
 // bounds test, and which (kh, kw) reaches which patch element is resolved at
 // compile time: only the K*K/(ST*ST) taps that really contribute are executed.
-template <int KS, int ST>
+// M1: depth multiplier 1 - the taps are fetched once, before the band, and stay in scalar registers.
+template <int KS, int ST, bool M1>
 __global__ void __launch_bounds__(dev::kBlock)
 dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ weight, Strides4 ws,
                  float *__restrict__ gradIn, DwGeom g, int stageRows) {
@@ -441,16 +455,21 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
   const int nRows = min(g.tileRows, g.H - h0);
   const int pitch = g.oW + dev::kStripPadL;
   const long L = (long)g.oH * g.oW;
-  for (int j = 0; j < g.M; ++j)
+  // the taps of the first multiplier are requested before the band, so that they arrive in its shadow
+  float w[KS * KS];
+  loadTaps<KS>(weight, ws, 0, c, w);
+  const int nMul = M1 ? 1 : g.M;
+  for (int j = 0; j < nMul; ++j)
     dev::loadRowsPadded<true>(smem + (size_t)j * (stageRows * pitch + dev::kStripPadL),
-                              gradOut + ((long)plane * g.M + j) * L, g.oH, g.oW, h0 / ST + QH0, stageRows, pitch,
+                              gradOut + ((long)plane * nMul + j) * L, g.oH, g.oW, h0 / ST + QH0, stageRows, pitch,
                               dev::kStripPadL);
   __syncthreads();
   const int W4 = g.W >> 2;
-  const unsigned magicW4 = dev::magicOf(W4);
+  const unsigned magicW4 = g.magicW4;
   const int nA = (nRows + ST - 1) / ST;
   const int total = nA * W4;
   float *o = gradIn + ((long)plane * g.H + h0) * g.W;
+#pragma unroll 2
   for (int i = threadIdx.x; i < total; i += blockDim.x) {
     const int a = dev::fastDiv(i, magicW4), b = i - a * W4;
     float acc[ST][4];
@@ -458,9 +477,8 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
     for (int dy = 0; dy < ST; ++dy)
 #pragma unroll
       for (int dx = 0; dx < 4; ++dx) acc[dy][dx] = 0.f;
-    for (int j = 0; j < g.M; ++j) {
-      float w[KS * KS];
-      loadTaps<KS>(weight, ws, j, c, w);
+    for (int j = 0; j < nMul; ++j) {
+      if (!M1) loadTaps<KS>(weight, ws, j, c, w);
       const float *gj = smem + (size_t)j * (stageRows * pitch + dev::kStripPadL) + dev::kStripPadL + QW0 + b * CPB;
 #pragma unroll
       for (int qh = QH0; qh <= QH1; ++qh) {
@@ -490,7 +508,9 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
 }
 
 // accGradParameters stage 1 with the same 4-wide windows as the forward pass.
-template <int KS, int ST>
+// ONE: depth multiplier 1 and both bands (input, gradOutput) are a single load batch: all their
+// loads are issued back to back before the first wait, one memory round trip per workgroup.
+template <int KS, int ST, bool ONE>
 __global__ void __launch_bounds__(dev::kBlock)
 dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, float *__restrict__ partial,
                DwGeom g) {
@@ -508,21 +528,39 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
   const int nIn = (nOut - 1) * ST + KS;
   const int pitch = S::pitch(g.W);
   float *gs = smem + S::floats((g.tileRows - 1) * ST + KS, g.W);  // multiple of 4 floats
-  S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
+  const int nMul = ONE ? 1 : g.M;
+  if (ONE) {
+    typename S::InFlight fl;
+    S::issue(fl, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
+    const int n4 = (nOut * g.oW) >> 2;
+    const __amdgpu_buffer_rsrc_t rs = dev::makeRsrc(gradOut + ((long)plane * g.oH + oh0) * g.oW, (long)n4 * 16);
+    float4 gv[dev::kLoadBatch];
+#pragma unroll
+    for (int u = 0; u < dev::kLoadBatch; ++u) gv[u] = dev::bufLoad4(rs, (u * dev::kBlock + threadIdx.x) * 16);  // past the end reads 0
+    S::commit(smem, fl, g.W, nIn);
+#pragma unroll
+    for (int u = 0; u < dev::kLoadBatch; ++u) {
+      const int i = u * dev::kBlock + threadIdx.x;
+      if (i < n4) reinterpret_cast<float4 *>(gs)[i] = gv[u];
+    }
+  } else {
+    S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
+  }
   const int oW4 = g.oW >> 2;
-  const unsigned magicOw4 = dev::magicOf(oW4);
   const int total = nOut * oW4;
   const int slot = n * g.tilesPerPlane + tile;
   const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
-  for (int j = 0; j < g.M; ++j) {
-    if (j > 0) __syncthreads();
-    dev::loadFlat<true>(gs, gradOut + (((long)plane * g.M + j) * g.oH + oh0) * g.oW, nOut * g.oW);
+  for (int j = 0; j < nMul; ++j) {
+    if (!ONE) {
+      if (j > 0) __syncthreads();
+      dev::loadFlat<true>(gs, gradOut + (((long)plane * g.M + j) * g.oH + oh0) * g.oW, nOut * g.oW);
+    }
     __syncthreads();
     float acc[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) acc[t] = 0.f;
     for (int i = threadIdx.x; i < total; i += blockDim.x) {
-      const int r = dev::fastDiv(i, magicOw4), b4 = i - r * oW4;
+      const int r = dev::fastDiv(i, g.magicOW4), b4 = i - r * oW4;
       const float *p = smem + r * ST * pitch;
       const float4 gy4 = *reinterpret_cast<const float4 *>(gs + r * g.oW + b4 * 4);
       const float gy[4] = {gy4.x, gy4.y, gy4.z, gy4.w};
@@ -547,7 +585,7 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
       float v = 0.f;
 #pragma unroll
       for (int w = 0; w < nWaves; ++w) v += red[w][threadIdx.x];
-      partial[(((long)c * g.M + j) * T + threadIdx.x) * g.nslots + slot] = v;
+      partial[(((long)c * nMul + j) * T + threadIdx.x) * g.nslots + slot] = v;
     }
   }
 }
@@ -701,6 +739,14 @@ bool stripGeometry(const DwGeom &g) {
          g.W % 4 == 0 && g.oW % 4 == 0;
 }
 
+#define DW_STRIP_DISPATCH1(KERNEL, FLAG, ...)                                            \
+  do {                                                                                   \
+    if (g.kH == 3 && g.dH == 1) KERNEL<3, 1, FLAG><<<grid, block, lds, s>>>(__VA_ARGS__); \
+    if (g.kH == 3 && g.dH == 2) KERNEL<3, 2, FLAG><<<grid, block, lds, s>>>(__VA_ARGS__); \
+    if (g.kH == 5 && g.dH == 1) KERNEL<5, 1, FLAG><<<grid, block, lds, s>>>(__VA_ARGS__); \
+    if (g.kH == 5 && g.dH == 2) KERNEL<5, 2, FLAG><<<grid, block, lds, s>>>(__VA_ARGS__); \
+  } while (0)
+
 #define DW_STRIP_DISPATCH(KERNEL, ...)                                           \
   do {                                                                           \
     if (g.kH == 3 && g.dH == 1) KERNEL<3, 1><<<grid, block, lds, s>>>(__VA_ARGS__); \
@@ -762,7 +808,11 @@ void THNN_CudaSpatialDepthWiseConvolution_updateOutput(THCState *state, THCudaTe
       size_t lds = sbytes(g.tileRows);
       dim3 grid(g.nblk), block(dev::kBlock);
       g.magicTiles = dev::magicOf(g.tilesPerPlane), g.magicC = dev::magicOf(g.C);
-      DW_STRIP_DISPATCH(dwFwdStrip, in.ptr(), data(weight), strides4(weight), bptr, strides2(bias), data(output), g);
+      g.magicOW4 = dev::magicOf(g.oW / 4), g.magicW4 = dev::magicOf(g.W / 4);
+      if (g.M == 1 && staged(g.tileRows) <= (size_t)launch::kBatchFloats)
+        DW_STRIP_DISPATCH1(dwFwdStrip, true, in.ptr(), data(weight), strides4(weight), bptr, strides2(bias), data(output), g);
+      else
+        DW_STRIP_DISPATCH1(dwFwdStrip, false, in.ptr(), data(weight), strides4(weight), bptr, strides2(bias), data(output), g);
       THC_HIP_CHECK(hipGetLastError());
       return;
     }
@@ -822,7 +872,11 @@ void THNN_CudaSpatialDepthWiseConvolution_updateGradInput(THCState *state, THCud
       size_t lds = sbytes(units);
       dim3 grid(g.nblk), block(dev::kBlock);
       g.magicTiles = dev::magicOf(g.tilesPerPlane), g.magicC = dev::magicOf(g.C);
-      DW_STRIP_DISPATCH(dwGradInputStrip, go.ptr(), data(weight), strides4(weight), data(gradInput), g, units + extra);
+      g.magicOW4 = dev::magicOf(g.oW / 4), g.magicW4 = dev::magicOf(g.W / 4);
+      if (g.M == 1)
+        DW_STRIP_DISPATCH1(dwGradInputStrip, true, go.ptr(), data(weight), strides4(weight), data(gradInput), g, units + extra);
+      else
+        DW_STRIP_DISPATCH1(dwGradInputStrip, false, go.ptr(), data(weight), strides4(weight), data(gradInput), g, units + extra);
       THC_HIP_CHECK(hipGetLastError());
       return;
     }
@@ -900,7 +954,11 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
     if (useStrip) {
       dim3 grid(g.nblk), block(dev::kBlock);
       g.magicTiles = dev::magicOf(g.tilesPerPlane), g.magicC = dev::magicOf(g.C);
-      DW_STRIP_DISPATCH(dwAccGradStrip, in.ptr(), go.ptr(), partial, g);
+      g.magicOW4 = dev::magicOf(g.oW / 4), g.magicW4 = dev::magicOf(g.W / 4);
+      if (g.M == 1 && staged(g.tileRows) <= (size_t)launch::kBatchFloats && aligned16(go.ptr()))
+        DW_STRIP_DISPATCH1(dwAccGradStrip, true, in.ptr(), go.ptr(), partial, g);
+      else
+        DW_STRIP_DISPATCH1(dwAccGradStrip, false, in.ptr(), go.ptr(), partial, g);
     } else {
       if (ks == 3 && st == 1) launchAcc1<3, 1>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
       if (ks == 3 && st == 2) launchAcc1<3, 2>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);

@@ -57,6 +57,53 @@ struct Strip {
     else
       loadRowsSplit(dst, plane, H, W, r0, nRows, pitch(W), fill);
   }
+  // The same staging in two halves: issue() starts the (at most kLoadBatch per lane) 16-byte
+  // loads of a band into registers, commit() parks them in LDS in the layout stage() produces
+  // (zero fill). Whatever else a workgroup needs before it can compute (taps, bias, derived
+  // indices) is fetched between the two, while the band is in flight.
+  // One batch only: nRows * W / 4 <= kLoadBatch * blockDim.x.
+  struct InFlight {
+    float4 v[kLoadBatch];
+    int off[kLoadBatch];
+  };
+  __device__ static void issue(InFlight &f, const float *plane, int H, int W, int r0, int nRows) {
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const int W4 = W >> 2, total = nRows * W4;
+    const unsigned magic = magicOf(W4);
+    const int p = pitch(W);
+    const __amdgpu_buffer_rsrc_t rs = makeRsrc(plane, (long)H * W * 4);
+#pragma unroll
+    for (int u = 0; u < kLoadBatch; ++u) {
+      const int i = u * nt + tid;
+      const int r = fastDiv(i, magic), c4 = i - r * W4;
+      const int gr = r0 + r;
+      const bool ok = i < total && (unsigned)gr < (unsigned)H;
+      f.off[u] = (i < total) ? r * p + kStripPadL + (ST == 1 ? (c4 << 2) : (c4 << 1)) : -1;
+      f.v[u] = bufLoad4(rs, ok ? (gr * W + (c4 << 2)) * 4 : kBufOob);
+    }
+  }
+  __device__ static void commit(float *dst, const InFlight &f, int W, int nRows) {
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const int p = pitch(W);
+    if (ST == 1) {
+      for (int i = tid; i < (nRows + 1) * kStripPadL; i += nt) dst[(i >> 2) * p + (i & 3)] = 0.f;
+#pragma unroll
+      for (int u = 0; u < kLoadBatch; ++u)
+        if (f.off[u] >= 0) *reinterpret_cast<float4 *>(dst + f.off[u]) = f.v[u];
+    } else {
+      const int oddOff = (W >> 1) + 8;
+      for (int i = tid; i < nRows * 8 + 4; i += nt) {
+        const int r = i >> 3, k = i & 7;
+        dst[r * p + (k < 4 ? k : (W >> 1) + k)] = 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < kLoadBatch; ++u)
+        if (f.off[u] >= 0) {
+          *reinterpret_cast<float2 *>(dst + f.off[u]) = make_float2(f.v[u].x, f.v[u].z);
+          *reinterpret_cast<float2 *>(dst + f.off[u] + oddOff - 4) = make_float2(f.v[u].y, f.v[u].w);
+        }
+    }
+  }
   // window element j is input column 4*ST*b4 - PAD + j
   static constexpr int half(int j) { return (j - PAD) % 2 == 0 ? (j - PAD) / 2 : (j - PAD - 1) / 2; }
   static constexpr bool even(int j) { return (j - PAD) % 2 == 0; }

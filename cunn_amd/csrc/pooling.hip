@@ -31,7 +31,7 @@ struct PoolGeom {
 
 // (plane, tile) of a workgroup of the strip kernels
 __device__ __forceinline__ void blockPos(const PoolGeom &g, int &plane, int &tile) {
-  const int bid = dev::xcdRemap(blockIdx.x, g.nblk);
+  const int bid = blockIdx.x;  // consecutive workgroups work on neighbouring planes
   plane = g.tilesPerPlane == 1 ? bid : dev::fastDiv(bid, g.magicTiles);
   tile = bid - plane * g.tilesPerPlane;
 }
@@ -403,6 +403,60 @@ avgPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, PoolGeom 
   }
 }
 
+// Non-overlapping average pooling (window = stride = KS, no padding, H = KS*oH, W = KS*oW): no
+// input element is shared between windows, so nothing is staged. With these extents the planes
+// of the batch form one tall image of planes*oH output rows; a lane owns 4 consecutive outputs
+// of one of those rows and streams its KS x 4*KS input patch through registers with 16-byte
+// loads (forward), or expands 4 gradOutput values into that patch (backward).
+template <int KS>
+__global__ void __launch_bounds__(dev::kBlock)
+avgPoolFwdFlat(const float *__restrict__ in, float *__restrict__ out, int oW4, unsigned magicOw4, int W, unsigned total) {
+  const unsigned i = blockIdx.x * dev::kBlock + threadIdx.x;
+  if (i >= total) return;
+  const unsigned R = dev::fastDiv((int)i, magicOw4), b = i - R * oW4;
+  const float4 *p = reinterpret_cast<const float4 *>(in + (size_t)R * KS * W) + b * KS;
+  const int W4 = W >> 2;
+  float4 v[KS][KS];
+#pragma unroll
+  for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+    for (int k = 0; k < KS; ++k) v[kh][k] = p[kh * W4 + k];
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int kh = 0; kh < KS; ++kh) {
+    float row[4 * KS];
+#pragma unroll
+    for (int k = 0; k < KS; ++k) row[4 * k] = v[kh][k].x, row[4 * k + 1] = v[kh][k].y, row[4 * k + 2] = v[kh][k].z, row[4 * k + 3] = v[kh][k].w;
+#pragma unroll
+    for (int kw = 0; kw < KS; ++kw)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc[q] += row[q * KS + kw];
+  }
+  reinterpret_cast<float4 *>(out)[i] = make_float4(acc[0] / (float)(KS * KS), acc[1] / (float)(KS * KS),
+                                                  acc[2] / (float)(KS * KS), acc[3] / (float)(KS * KS));
+}
+
+template <int KS>
+__global__ void __launch_bounds__(dev::kBlock)
+avgPoolBwdFlat(const float *__restrict__ gradOut, float *__restrict__ gradIn, int oW4, unsigned magicOw4, int W, unsigned total) {
+  const unsigned i = blockIdx.x * dev::kBlock + threadIdx.x;
+  if (i >= total) return;
+  const unsigned R = dev::fastDiv((int)i, magicOw4), b = i - R * oW4;
+  const float4 g4 = reinterpret_cast<const float4 *>(gradOut)[i];
+  const float gq[4] = {g4.x / (float)(KS * KS), g4.y / (float)(KS * KS), g4.z / (float)(KS * KS), g4.w / (float)(KS * KS)};
+  float row[4 * KS];
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+#pragma unroll
+    for (int kw = 0; kw < KS; ++kw) row[q * KS + kw] = gq[q];
+  float4 *p = reinterpret_cast<float4 *>(gradIn + (size_t)R * KS * W) + b * KS;
+  const int W4 = W >> 2;
+#pragma unroll
+  for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+    for (int k = 0; k < KS; ++k) p[kh * W4 + k] = make_float4(row[4 * k], row[4 * k + 1], row[4 * k + 2], row[4 * k + 3]);
+}
+
 // Backward gathers. MAX: gradOutput and the argmax (narrowed to int32, base
 // removed, -2 outside) are staged with a 4-cell fill in front of every row; a
 // patch element adds the gradOutput of each covering window whose argmax is that
@@ -534,6 +588,16 @@ bool stripCombo(const PoolGeom &g) {
 
 // Forward strips read 4 fill cells beyond a row at most (and, in the split
 // stride-2 layout, only even columns may overhang).
+// Geometry of the flat average-pooling kernels: window = stride in {2, 3, 4}, no padding, extents
+// that the windows tile exactly, rows of 4-output groups, and item indices that keep the reciprocal
+// division exact.
+bool avgFlatOk(const PoolGeom &g, long planes) {
+  const bool sq = g.kH == g.kW && g.dH == g.kH && g.dW == g.kW && g.padH == 0 && g.padW == 0;
+  const long total = planes * g.oH * (g.oW / 4);
+  return forcedPath() == 0 && sq && g.kH >= 2 && g.kH <= 4 && g.H == g.oH * g.kH && g.W == g.oW * g.kW && g.oW % 4 == 0 &&
+         total > 0 && total * (g.oW / 4) < 0xffffffffL && total < 0x7fffffffL;
+}
+
 bool stripFwdOk(const PoolGeom &g) {
   if (forcedPath() != 0 || !stripCombo(g) || g.oW % 4 != 0) return false;
   if (g.W % (4 * g.dW) != 0) return false;
@@ -810,7 +874,14 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
     auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.W * sizeof(float); };
     auto sbytes = [&](int rows) { return fwdStripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
     auto staged = [&](int rows) { return (size_t)((rows - 1) * g.dH + g.kH) * g.W; };
-    if (stripFwdOk(g) && vec && aligned16(data(output)) &&
+    if (avgFlatOk(g, planes) && vec && aligned16(data(output))) {
+      const unsigned total = (unsigned)(planes * g.oH * (g.oW / 4));
+      const unsigned grid = (total + dev::kBlock - 1) / dev::kBlock;
+      const unsigned magic = dev::magicOf(g.oW / 4);
+      if (g.kH == 2) avgPoolFwdFlat<2><<<grid, dev::kBlock, 0, s>>>(in.ptr(), data(output), g.oW / 4, magic, g.W, total);
+      if (g.kH == 3) avgPoolFwdFlat<3><<<grid, dev::kBlock, 0, s>>>(in.ptr(), data(output), g.oW / 4, magic, g.W, total);
+      if (g.kH == 4) avgPoolFwdFlat<4><<<grid, dev::kBlock, 0, s>>>(in.ptr(), data(output), g.oW / 4, magic, g.W, total);
+    } else if (stripFwdOk(g) && vec && aligned16(data(output)) &&
         launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane, staged)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
       g.magicTiles = dev::magicOf(g.tilesPerPlane);
@@ -880,7 +951,14 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
   const int spitch = g.oW + dev::kStripPadL;
   auto sbytes = [&](int units) { return ((size_t)(units + extra) * spitch + dev::kStripPadL) * sizeof(float); };
   int units = 0;
-  if (stripBwdOk(g) && vec && aligned16(data(gradInput)) &&
+  if (avgFlatOk(g, planes) && vec && aligned16(data(gradInput))) {
+    const unsigned total = (unsigned)(planes * g.oH * (g.oW / 4));
+    const unsigned grid = (total + dev::kBlock - 1) / dev::kBlock;
+    const unsigned magic = dev::magicOf(g.oW / 4);
+    if (g.kH == 2) avgPoolBwdFlat<2><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.oW / 4, magic, g.W, total);
+    if (g.kH == 3) avgPoolBwdFlat<3><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.oW / 4, magic, g.W, total);
+    if (g.kH == 4) avgPoolBwdFlat<4><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.oW / 4, magic, g.W, total);
+  } else if (stripBwdOk(g) && vec && aligned16(data(gradInput)) &&
       launch::pickBand(launch::ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
     g.tileRows = units * g.dH;
     g.nblk = (int)(planes * g.tilesPerPlane);

@@ -204,6 +204,9 @@ POOL_CASES = [
     (2, 3, 48, 48, 3, 3, 2, 2, 0, 0, True),      # unpadded 3x3 s2, ceil mode: last window overhangs
     (1, 2, 300, 264, 3, 3, 2, 2, 1, 1, False),   # strip kernels, several bands
     (2, 2, 31, 40, 3, 3, 1, 1, 1, 1, False),     # 3x3 s1 strip with odd height
+    (3, 2, 27, 48, 3, 3, 3, 3, 0, 0, False),     # window = stride 3, exact tiling (flat average kernels)
+    (2, 3, 40, 64, 4, 4, 4, 4, 0, 0, True),      # window = stride 4, exact tiling, ceil mode without effect
+    (2, 2, 22, 24, 2, 2, 2, 2, 0, 0, False),     # window = stride 2, oW = 12
 ]
 
 

@@ -75,6 +75,15 @@ __device__ __forceinline__ int ceilDivPos(int a, int b) {  // ceil(a / b) for b 
   return (a >= 0) ? (a + b - 1) / b : -((-a) / b);
 }
 
+// 16-byte store of data that is not read again soon (an output tensor written once): the
+// non-temporal hint keeps it from displacing tensors that the next kernels re-read from the
+// last-level cache.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void storeStream4(float *p, float4 v) {
+  f32x4 q = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(q, reinterpret_cast<f32x4 *>(p));
+}
+
 // Number of independent 16-byte (or 4-byte) global loads a lane keeps in flight
 // before it starts storing to LDS: the loads of one batch are issued back to
 // back, so a band costs ceil(per-lane loads / kLoadBatch) memory round trips

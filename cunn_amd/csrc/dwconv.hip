@@ -304,30 +304,31 @@ dwAccGradStage1(const float *__restrict__ in, const float *__restrict__ gradOut,
   }
 }
 
-// Stage 2: one workgroup per (c,j); wave w folds taps w, w+4, ... over all
-// slots in a fixed order and accumulates scale * sum into the caller's tensors.
+// Stage 2: one wave per ((c,j), tap) folds the partials of all slots in a fixed order and
+// accumulates scale * sum into the caller's tensors; the old value is requested before the
+// partials so that the read-modify-write costs no second round trip.
 __global__ void __launch_bounds__(dev::kBlock)
 dwAccGradStage2(const float *__restrict__ partial, float *__restrict__ gradWeight, Strides4 gs,
-                float *__restrict__ gradBias, Strides2 bs, int M, int kW, int T, int nslots, float scale) {
-  const int cj = blockIdx.x;
+                float *__restrict__ gradBias, Strides2 bs, int M, int kW, int T, int nslots, float scale, int pairs) {
+  const int lane = threadIdx.x % dev::kWave;
+  const int pair = blockIdx.x * (dev::kBlock / dev::kWave) + threadIdx.x / dev::kWave;  // (c*M + j) * T + t
+  if (pair >= pairs) return;
+  const int cj = pair / T, t = pair - cj * T;
   const int c = cj / M, j = cj - c * M;
-  const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
-  for (int t = wave; t < T; t += blockDim.x / dev::kWave) {
-    const float *p = partial + ((long)cj * T + t) * nslots;
-    float v = 0.f;
-    for (int s = lane; s < nslots; s += dev::kWave) v += p[s];
-    v = dev::waveSum(v);
-    if (lane == 0) {
-      if (t < T - 1) {
-        int kh = t / kW, kw = t - kh * kW;
-        float *dst = gradWeight + j * gs.s0 + c * gs.s1 + kh * gs.s2 + kw * gs.s3;
-        *dst += scale * v;
-      } else if (gradBias) {
-        float *dst = gradBias + j * bs.s0 + c * bs.s1;
-        *dst += scale * v;
-      }
-    }
+  float *dst;
+  if (t < T - 1) {
+    const int kh = t / kW, kw = t - kh * kW;
+    dst = gradWeight + j * gs.s0 + c * gs.s1 + kh * gs.s2 + kw * gs.s3;
+  } else {
+    if (!gradBias) return;
+    dst = gradBias + j * bs.s0 + c * bs.s1;
   }
+  const float old = *dst;
+  const float *p = partial + (long)pair * nslots;
+  float v = 0.f;
+  for (int s = lane; s < nslots; s += dev::kWave) v += p[s];
+  v = dev::waveSum(v);
+  if (lane == 0) *dst = old + scale * v;
 }
 
 // Any geometry: one workgroup per (c, j, tap) - tap == kH*kW is the bias - that
@@ -427,7 +428,7 @@ dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strid
 #pragma unroll
           for (int q = 0; q < 4; ++q) acc[q] = fmaf(win[q * ST + kw], w[kh * KS + kw], acc[q]);
       }
-      *reinterpret_cast<float4 *>(o + (long)r * g.oW + b4 * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      dev::storeStream4(o + (long)r * g.oW + b4 * 4, make_float4(acc[0], acc[1], acc[2], acc[3]));
     }
   }
 }
@@ -502,8 +503,7 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
 #pragma unroll
     for (int dy = 0; dy < ST; ++dy)
       if (a * ST + dy < nRows)
-        *reinterpret_cast<float4 *>(o + (long)(a * ST + dy) * g.W + b * 4) =
-            make_float4(acc[dy][0], acc[dy][1], acc[dy][2], acc[dy][3]);
+        dev::storeStream4(o + (long)(a * ST + dy) * g.W + b * 4, make_float4(acc[dy][0], acc[dy][1], acc[dy][2], acc[dy][3]));
   }
 }
 
@@ -966,8 +966,9 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
       if (ks == 5 && st == 2) launchAcc1<5, 2>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
     }
     THC_HIP_CHECK(hipGetLastError());
-    dwAccGradStage2<<<g.C * g.M, dev::kBlock, 0, s>>>(partial, data(gradWeight), strides4(gradWeight), gbPtr,
-                                                      strides2(gradBias), g.M, g.kW, T, g.nslots, scale);
+    const int pairs = g.C * g.M * T;
+    dwAccGradStage2<<<ceilDiv(pairs, dev::kBlock / dev::kWave), dev::kBlock, 0, s>>>(
+        partial, data(gradWeight), strides4(gradWeight), gbPtr, strides2(gradBias), g.M, g.kW, T, g.nslots, scale, pairs);
   } else {
     int T = g.kH * g.kW + 1;
     dwAccGradDirect<<<g.C * g.M * T, dev::kBlock, 0, s>>>(in.ptr(), go.ptr(), data(gradWeight),

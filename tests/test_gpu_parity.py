@@ -118,6 +118,32 @@ def test_dwconv_fallback_kernels(T, case, mode):
         _dw_run(T, case, x, w, b)
 
 
+def test_dwconv_accgrad_deterministic(T):
+    """accGradParameters folds per-workgroup partials in a fixed order (no atomics): repeated
+    calls on the same inputs are bit-identical."""
+    THNN, CT = T.THNN, T.CudaTensor
+    case = (6, 40, 1, 56, 56, 3, 3, 2, 2, 1, 1)
+    N, C, M, H, W, kW, kH, dW, dH, pW, pH = case
+    rng, x, w, b = _dw_inputs(case, 9)
+    oH = (H + 2 * pH - kH) // dH + 1
+    gy = rng.standard_normal((N, C, oH, oH)).astype(np.float32)
+    gw0 = rng.standard_normal(w.shape).astype(np.float32)
+    gb0 = rng.standard_normal(b.shape).astype(np.float32)
+    rgw, rgb = O.dwconv_accGradParameters(x, gy, gw0.copy(), gb0.copy(), kW, kH, dW, dH, pW, pH, 0.5)
+
+    def run():
+        tgw, tgb = CT.from_numpy(gw0), CT.from_numpy(gb0)
+        THNN.SpatialDepthWiseConvolution_accGradParameters(CT.from_numpy(x), CT.from_numpy(gy), tgw, tgb, CT(), CT(),
+                                                           kW, kH, dW, dH, pW, pH, 0.5)
+        return tgw.numpy(), tgb.numpy()
+
+    results = [run() for _ in range(3)]
+    for gw, gb in results:
+        close(gw, rgw, WG_RTOL, WG_ATOL)
+        close(gb, rgb, WG_RTOL, WG_ATOL)
+        assert np.array_equal(gw, results[0][0]) and np.array_equal(gb, results[0][1])
+
+
 def test_dwconv_no_bias_scale_and_accumulate(T):
     case = (3, 6, 2, 20, 24, 3, 3, 2, 2, 1, 1)
     rng, x, w, _ = _dw_inputs(case, 3, bias=False)

@@ -19,6 +19,12 @@ ENTRY_POINTS = [
     "SpatialDepthWiseConvolution_accGradParameters",
     "SpatialDilatedMaxPooling_updateOutput", "SpatialDilatedMaxPooling_updateGradInput",
     "SpatialMaxPooling_updateOutput", "SpatialMaxPooling_updateGradInput",
+    "SpatialDilatedConvolution_updateOutput", "SpatialDilatedConvolution_updateGradInput",
+    "SpatialDilatedConvolution_accGradParameters",
+    "SpatialFullDilatedConvolution_updateOutput", "SpatialFullDilatedConvolution_updateGradInput",
+    "SpatialFullDilatedConvolution_accGradParameters",
+    "SpatialFullConvolution_updateOutput", "SpatialFullConvolution_updateGradInput",
+    "SpatialFullConvolution_accGradParameters",
 ]
 
 _T = C.c_void_p  # THCudaTensor* / THCudaLongTensor* / THCState*
@@ -39,6 +45,15 @@ SIGNATURES = {
     "SpatialDilatedMaxPooling_updateGradInput": [_T] * 5 + [_i] * 8 + [_b],
     "SpatialMaxPooling_updateOutput": [_T] * 4 + [_i] * 6 + [_b],
     "SpatialMaxPooling_updateGradInput": [_T] * 5 + [_i] * 6 + [_b],
+    "SpatialDilatedConvolution_updateOutput": [_T] * 7 + [_i] * 8,
+    "SpatialDilatedConvolution_updateGradInput": [_T] * 6 + [_i] * 8,
+    "SpatialDilatedConvolution_accGradParameters": [_T] * 7 + [_i] * 8 + [_f],
+    "SpatialFullDilatedConvolution_updateOutput": [_T] * 7 + [_i] * 10,
+    "SpatialFullDilatedConvolution_updateGradInput": [_T] * 6 + [_i] * 10,
+    "SpatialFullDilatedConvolution_accGradParameters": [_T] * 7 + [_i] * 10 + [_f],
+    "SpatialFullConvolution_updateOutput": [_T] * 7 + [_i] * 8,
+    "SpatialFullConvolution_updateGradInput": [_T] * 6 + [_i] * 8,
+    "SpatialFullConvolution_accGradParameters": [_T] * 7 + [_i] * 8 + [_f],
 }
 
 _LP = C.POINTER(C.c_long)

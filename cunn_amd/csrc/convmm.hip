@@ -37,6 +37,7 @@ constexpr int PITCH = 132;  // 8 * PITCH % 64 == 32: the two k-halves of a trans
 struct ConvGeom {
   int N, Cin, Cout, H, W, oH, oW;
   int kH, kW, dH, dW, padH, padW;
+  int dilH, dilW;  // tap spacing (1 = ordinary convolution)
   int K;  // Cin * kH * kW
   int L;  // oH * oW
 };
@@ -79,7 +80,7 @@ __device__ __forceinline__ void mfmaTile(const float (*As)[PITCH], const float (
 // x[c][oh*dH - padH + kh][ow*dW - padW + kw] or 0 (lib/THCUNN/im2col.h:24-36).
 __device__ __forceinline__ float gatherCol(const float *__restrict__ xb, const ConvGeom &g, int c, int kh, int kw,
                                            int ih0, int iw0) {
-  int ih = ih0 + kh, iw = iw0 + kw;
+  int ih = ih0 + kh * g.dilH, iw = iw0 + kw * g.dilW;
   return (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W) ? xb[((long)c * g.H + ih) * g.W + iw] : 0.f;
 }
 
@@ -390,14 +391,14 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
   }
 }
 
-// taps[k] = ((c*H + kh)*W + kw) * 4 for k = (c*kH + kh)*kW + kw; g is the geometry of the padded images.
+// taps[k] = ((c*H + kh*dilH)*W + kw*dilW) * 4 for k = (c*kH + kh)*kW + kw; g is the geometry of the padded images.
 __global__ void __launch_bounds__(dev::kBlock)
 buildTapTableKernel(int *taps, int entries, ConvGeom g) {
   const int KK = g.kH * g.kW;
   for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < entries; k += gridDim.x * blockDim.x) {
     const int c = k / KK, rem = k - c * KK;
     const int kh = rem / g.kW, kw = rem - kh * g.kW;
-    taps[k] = ((c * g.H + kh) * g.W + kw) * 4;
+    taps[k] = ((c * g.H + kh * g.dilH) * g.W + kw * g.dilW) * 4;
   }
 }
 
@@ -504,9 +505,9 @@ convFwdImplicitKernel(FwdArgs p, ConvGeom g) {
     float tmp[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int ih = ih0 + kh, iw = iw0 + kw;
+      const int ih = ih0 + kh * g.dilH, iw = iw0 + kw * g.dilW;
       const bool ok = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W && (k + i) < g.K;
-      const int soff = ((c * g.H + kh) * g.W + kw) * 4;  // scalar
+      const int soff = ((c * g.H + kh * g.dilH) * g.W + kw * g.dilW) * 4;  // scalar
       const int off = ok ? posOff + soff : kOob;
       tmp[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
       if (++kw == g.kW) {
@@ -793,7 +794,7 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
       const int k = min(j0 + cB + 16 * i, p.Ncols - 1);  // columns past K are dropped in the epilogue
       const int c = k / KK, rem = k - c * KK;
       const int kh = rem / g.kW, kw = rem - kh * g.kW;
-      tapOff[i] = ((c * g.H + kh) * g.W + kw) * 4;
+      tapOff[i] = ((c * g.H + kh * g.dilH) * g.W + kw * g.dilW) * 4;
     }
   }
   const int imgStrideB = g.Cin * g.H * g.W * 4;
@@ -943,6 +944,13 @@ gradBiasKernel(const float *__restrict__ gy, float *__restrict__ gradBias, int N
   }
 }
 
+// t[n][c][:] += bias[c] over a (N, C, plane) tensor
+__global__ void __launch_bounds__(dev::kBlock)
+addPlaneBiasKernel(float *__restrict__ t, const float *__restrict__ bias, long total, int plane, int C) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x)
+    t[i] += bias[(int)((i / plane) % C)];
+}
+
 // Wf[c][(o, kh', kw')] = W[o][(c, kH-1-kh', kW-1-kw')]: with these weights the
 // stride-1 gradInput is a plain forward convolution of gradOutput (padding k-1-pad).
 __global__ void __launch_bounds__(dev::kBlock)
@@ -1017,17 +1025,43 @@ struct ConvCall {
   bool batch;
 };
 
-// lib/THCUNN/generic/SpatialConvolutionMM.cu:5-56. `weight` may be 2-D (Cout, Cin*kH*kW)
-// or 4-D contiguous; only its extents are read here.
+ConvGeom makeGeom(int N, int Cin, int Cout, int H, int W, int oH, int oW, int kH, int kW, int dH, int dW, int padH,
+                  int padW, int dilH, int dilW) {
+  ConvGeom g{};
+  g.N = N, g.Cin = Cin, g.Cout = Cout, g.H = H, g.W = W, g.oH = oH, g.oW = oW;
+  g.kH = kH, g.kW = kW, g.dH = dH, g.dW = dW, g.padH = padH, g.padW = padW, g.dilH = dilH, g.dilW = dilW;
+  g.K = g.Cin * kH * kW;
+  g.L = g.oH * g.oW;
+  if ((long)g.Cin * g.H * g.W >= 0x7fffffffL || (long)g.Cout * g.L >= 0x7fffffffL || (long)g.K * g.L >= 0x7fffffffL * 8L)
+    error("spatial convolution: image too large");
+  return g;
+}
+
+// Shape rules of lib/THCUNN/generic/SpatialConvolutionMM.cu:5-56 (kConvMM: `weight` 2-D
+// (Cout, Cin*kH*kW) or 4-D) and of generic/SpatialDilatedConvolution.cu:5-67 (kDilated: 4-D weight,
+// dilation > 0); only the extents of `weight` are read here.
+enum ConvFlavor { kConvMM, kDilated };
 ConvCall convSetup(THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *weight, THCudaTensor *bias,
-                   const char *weightName, int kH, int kW, int dH, int dW, int padH, int padW) {
+                   const char *weightName, int kH, int kW, int dH, int dW, int padH, int padW, int dilH = 1,
+                   int dilW = 1, ConvFlavor flavor = kConvMM) {
   THC_ARG_CHECK(input && weight, 2, "input and weight tensors expected");
-  THC_ARG_CHECK(isContiguous(erase(weight)), 4, "%s tensor has to be contiguous", weightName);
+  if (flavor == kDilated)
+    THC_ARG_CHECK(weight->nDimension == 4, 4,
+                  "4D weight tensor (nOutputPlane,nInputPlane,kH,kW) expected, but got: %s",
+                  sizeDesc(erase(weight)).c_str());
+  else
+    THC_ARG_CHECK(isContiguous(erase(weight)), 4, "%s tensor has to be contiguous", weightName);
   THC_ARG_CHECK(kW > 0 && kH > 0, 9, "kernel size should be greater than zero, but got kH: %d kW: %d", kH, kW);
   THC_ARG_CHECK(dW > 0 && dH > 0, 11, "stride should be greater than zero, but got dH: %d dW: %d", dH, dW);
+  if (flavor == kDilated)
+    THC_ARG_CHECK(isContiguous(erase(weight)), 4, "%s tensor has to be contiguous", weightName);
   THC_ARG_CHECK(!bias || isContiguous(erase(bias)), 5, "bias tensor has to be contiguous");
-  THC_ARG_CHECK(weight->nDimension == 2 || weight->nDimension == 4, 5,
-                "2D or 4D weight tensor expected, but got: %s", sizeDesc(erase(weight)).c_str());
+  if (flavor == kDilated)
+    THC_ARG_CHECK(dilW > 0 && dilH > 0, 14, "dilation should be greater than 0, but got dilationH: %d dilationW: %d",
+                  dilH, dilW);
+  else
+    THC_ARG_CHECK(weight->nDimension == 2 || weight->nDimension == 4, 5,
+                  "2D or 4D weight tensor expected, but got: %s", sizeDesc(erase(weight)).c_str());
   long nOutputPlane = weight->size[0];
   long wcols = weight->nDimension == 2 ? weight->size[1] : weight->size[1] * weight->size[2] * weight->size[3];
   if (bias) checkDimSize(erase(bias), "bias", 1, 0, nOutputPlane);
@@ -1040,10 +1074,10 @@ ConvCall convSetup(THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *
   }
   THC_ARG_CHECK(ndim == 3 || ndim == 4, 2, "3D or 4D input tensor expected but got: %s",
                 sizeDesc(erase(input)).c_str());
-  long nInputPlane = wcols / (kH * kW);
+  long nInputPlane = flavor == kDilated ? weight->size[1] : wcols / (kH * kW);
   long inputHeight = input->size[dimh], inputWidth = input->size[dimw];
-  long outputHeight = (inputHeight + 2 * padH - kH) / dH + 1;
-  long outputWidth = (inputWidth + 2 * padW - kW) / dW + 1;
+  long outputHeight = (inputHeight + 2 * padH - (dilH * (kH - 1) + 1)) / dH + 1;
+  long outputWidth = (inputWidth + 2 * padW - (dilW * (kW - 1) + 1)) / dW + 1;
   if (outputWidth < 1 || outputHeight < 1)
     error("Given input size: (%ld x %ld x %ld). Calculated output size: (%ld x %ld x %ld). Output size is too small",
           nInputPlane, inputHeight, inputWidth, nOutputPlane, outputHeight, outputWidth);
@@ -1060,15 +1094,8 @@ ConvCall convSetup(THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *
     error("%s of shape %s does not match a %d x %d kernel", weightName, sizeDesc(erase(weight)).c_str(), kH, kW);
   ConvCall call;
   call.batch = ndim == 4;
-  ConvGeom &g = call.g;
-  g.N = call.batch ? (int)input->size[0] : 1;
-  g.Cin = (int)nInputPlane, g.Cout = (int)nOutputPlane;
-  g.H = (int)inputHeight, g.W = (int)inputWidth, g.oH = (int)outputHeight, g.oW = (int)outputWidth;
-  g.kH = kH, g.kW = kW, g.dH = dH, g.dW = dW, g.padH = padH, g.padW = padW;
-  g.K = g.Cin * kH * kW;
-  g.L = g.oH * g.oW;
-  if ((long)g.Cin * g.H * g.W >= 0x7fffffffL || (long)g.K * g.L >= 0x7fffffffL * 8L)
-    error("SpatialConvolutionMM: image too large");
+  call.g = makeGeom(call.batch ? (int)input->size[0] : 1, (int)nInputPlane, (int)nOutputPlane, (int)inputHeight,
+                    (int)inputWidth, (int)outputHeight, (int)outputWidth, kH, kW, dH, dW, padH, padW, dilH, dilW);
   return call;
 }
 
@@ -1196,25 +1223,13 @@ float *scratchFloats(THCState *state, THCudaTensor *buffer, long floats, Temp &t
   return (float *)tmp.get();
 }
 
-}  // namespace
+// ---- the three passes on raw device pointers -------------------------------------------------
+// `scratchBuf` is the caller's buffer tensor (columns / gradColumns) or null; its contents are
+// unspecified afterwards.
 
-extern "C" {
-
-void THNN_CudaSpatialConvolutionMM_updateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output,
-                                                THCudaTensor *weight, THCudaTensor *bias, THCudaTensor *columns,
-                                                THCudaTensor *ones, int kW, int kH, int dW, int dH, int padW,
-                                                int padH) {
-  THNN_ENTER
-  (void)ones;  // never read; `columns` is used (and resized) only as scratch for K-split tail tiles
-  THC_ARG_CHECK(output != nullptr, 3, "output tensor expected");
-  ConvCall call = convSetup(input, nullptr, weight, bias, "weight", kH, kW, dH, dW, padH, padW);
-  ConvGeom &g = call.g;
-  Contiguous in(state, input);
-  if (call.batch)
-    resize(state, output, {g.N, g.Cout, g.oH, g.oW});
-  else
-    resize(state, output, {g.Cout, g.oH, g.oW});
-  if (!isContiguous(erase(output))) error("output tensor has to be contiguous");
+// out(N, Cout, oH, oW) = bias + conv(x(N, Cin, H, W), w(Cout, K))
+void convForward(THCState *state, const ConvGeom &g, const float *x, const float *w, const float *bias, float *out,
+                 THCudaTensor *scratchBuf, const char *bufName) {
   if ((long)g.N * g.Cout == 0) return;
   hipStream_t s = state->stream;
   // images per launch so that the flat column index n*L + l fits an int
@@ -1225,21 +1240,22 @@ void THNN_CudaSpatialConvolutionMM_updateOutput(THCState *state, THCudaTensor *i
   if (implicit2) {
     FwdPlan pl = planFwdImplicit(g.Cout, std::min(group, g.N), g);
     Temp tmp;
-    float *scratch = scratchFloats(state, columns, pl.scratchFloats, tmp, "columns");
+    float *scratch = scratchFloats(state, scratchBuf, pl.scratchFloats, tmp, bufName);
     for (int n0 = 0; n0 < g.N; n0 += group) {
       int cnt = std::min(group, g.N - n0);
       if (cnt != std::min(group, g.N)) pl = planFwdImplicit(g.Cout, cnt, g);  // last, smaller group: needs no more scratch
-      launchFwdImplicit(s, pl, scratch, data(weight), in.ptr() + (long)n0 * g.Cin * g.H * g.W,
-                        data(output) + (long)n0 * g.Cout * g.L, bias ? data(bias) : nullptr, g.Cout, cnt, g);
+      launchFwdImplicit(s, pl, scratch, w, x + (long)n0 * g.Cin * g.H * g.W, out + (long)n0 * g.Cout * g.L, bias, g.Cout,
+                        cnt, g);
     }
+    return;
   }
-  for (int n0 = 0; !implicit2 && n0 < g.N; n0 += group) {
+  for (int n0 = 0; n0 < g.N; n0 += group) {
     int cnt = std::min(group, g.N - n0);
     GemmArgs p{};
-    p.a = data(weight);
-    p.b = in.ptr();
-    p.c = data(output);
-    p.bias = bias ? data(bias) : nullptr;
+    p.a = w;
+    p.b = x;
+    p.c = out;
+    p.bias = bias;
     p.M = g.Cout;
     p.Ncols = cnt * g.L;
     p.R = g.K;
@@ -1251,38 +1267,27 @@ void THNN_CudaSpatialConvolutionMM_updateOutput(THCState *state, THCudaTensor *i
     convGemmKernel<kForward><<<grid, dev::kBlock, 0, s>>>(p, g);
     THC_HIP_CHECK(hipGetLastError());
   }
-  THNN_LEAVE
 }
 
-void THNN_CudaSpatialConvolutionMM_updateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput,
-                                                   THCudaTensor *gradInput, THCudaTensor *weight,
-                                                   THCudaTensor *gradColumns, THCudaTensor *ones, int kW, int kH,
-                                                   int dW, int dH, int padW, int padH) {
-  THNN_ENTER
-  (void)ones;
-  THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
-  THC_ARG_CHECK(gradInput != nullptr, 4, "gradInput tensor expected");
-  ConvCall call = convSetup(input, gradOutput, weight, nullptr, "weight", kH, kW, dH, dW, padH, padW);
-  ConvGeom &g = call.g;
-  Contiguous go(state, gradOutput);
-  if (call.batch)
-    resize(state, gradInput, {g.N, g.Cin, g.H, g.W});
-  else
-    resize(state, gradInput, {g.Cin, g.H, g.W});
-  if (!isContiguous(erase(gradInput))) error("gradInput tensor has to be contiguous");
+// gi(N, Cin, H, W) = conv^T(gy(N, Cout, oH, oW), w(Cout, K))
+// + bias[c] per plane of gi when bias != null (the transposed convolution's forward pass)
+void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const float *w, float *gi,
+                   THCudaTensor *scratchBuf, const char *bufName, const float *bias = nullptr) {
   if ((long)g.N * g.Cin == 0) return;
   hipStream_t s = state->stream;
   // Stride 1: gradInput is a forward convolution of gradOutput with the flipped,
-  // transposed weights and padding k-1-pad, so it runs on the implicit-GEMM
+  // transposed weights and padding dil*(k-1)-pad, so it runs on the implicit-GEMM
   // forward kernel and no gradient columns ever reach memory.
-  const long goImgBytes =
-      (long)g.Cout * (g.oH + 2 * (g.kH - 1 - g.padH)) * (g.oW + 2 * (g.kW - 1 - g.padW)) * sizeof(float);  // with its zero border
-  if (g.dH == 1 && g.dW == 1 && g.padH <= g.kH - 1 && g.padW <= g.kW - 1 && !forceGeneric() &&
-      goImgBytes < (1L << 30)) {
+  const int tpH = g.dilH * (g.kH - 1) - g.padH, tpW = g.dilW * (g.kW - 1) - g.padW;
+  const long goImgBytes = (long)g.Cout * (g.oH + 2 * std::max(tpH, 0)) * (g.oW + 2 * std::max(tpW, 0)) * sizeof(float);  // with its zero border
+  // (with stride 1 the extents correspond exactly unless a transposed convolution asks for output padding)
+  const bool exact = g.H == g.oH + 2 * tpH - g.dilH * (g.kH - 1) && g.W == g.oW + 2 * tpW - g.dilW * (g.kW - 1);
+  if (g.dH == 1 && g.dW == 1 && tpH >= 0 && tpW >= 0 && exact && !forceGeneric() && goImgBytes < (1L << 30) &&
+      (long)g.Cout * g.K < 0x7fffffffL / 4) {
     ConvGeom t = g;  // the transposed problem
     t.Cin = g.Cout, t.Cout = g.Cin;
     t.H = g.oH, t.W = g.oW, t.oH = g.H, t.oW = g.W;
-    t.padH = g.kH - 1 - g.padH, t.padW = g.kW - 1 - g.padW;
+    t.padH = tpH, t.padW = tpW;
     t.K = g.Cout * g.kH * g.kW;
     t.L = g.H * g.W;
     int group = (int)std::min<long>(g.N, std::max<long>(1, 0x7fffffffL / 2 / t.L));
@@ -1290,15 +1295,15 @@ void THNN_CudaSpatialConvolutionMM_updateGradInput(THCState *state, THCudaTensor
     FwdPlan pl = planFwdImplicit(t.Cout, std::min(group, g.N), t);
     const long wfFloats = ((long)g.Cout * g.K + 3) / 4 * 4;
     Temp tmp;
-    float *buf = scratchFloats(state, gradColumns, wfFloats + pl.scratchFloats, tmp, "gradColumns");
-    flipWeightKernel<<<launch::directGrid((long)g.Cout * g.K, dev::kBlock), dev::kBlock, 0, s>>>(data(weight), buf, g.Cout,
-                                                                                                g.Cin, g.kH, g.kW);
+    float *buf = scratchFloats(state, scratchBuf, wfFloats + pl.scratchFloats, tmp, bufName);
+    flipWeightKernel<<<launch::directGrid((long)g.Cout * g.K, dev::kBlock), dev::kBlock, 0, s>>>(w, buf, g.Cout, g.Cin,
+                                                                                                g.kH, g.kW);
     THC_HIP_CHECK(hipGetLastError());
     for (int n0 = 0; n0 < g.N; n0 += group) {
       int cnt = std::min(group, g.N - n0);
       if (cnt != std::min(group, g.N)) pl = planFwdImplicit(t.Cout, cnt, t);
-      launchFwdImplicit(s, pl, buf + wfFloats, buf, go.ptr() + (long)n0 * g.Cout * g.L,
-                        data(gradInput) + (long)n0 * g.Cin * g.H * g.W, nullptr, t.Cout, cnt, t);
+      launchFwdImplicit(s, pl, buf + wfFloats, buf, gy + (long)n0 * g.Cout * g.L, gi + (long)n0 * g.Cin * g.H * g.W,
+                        bias, t.Cout, cnt, t);
     }
     return;
   }
@@ -1307,20 +1312,12 @@ void THNN_CudaSpatialConvolutionMM_updateGradInput(THCState *state, THCudaTensor
   int group = (int)std::max<long>(1, std::min<long>(g.N, (64L << 20) / 4 / perImg));
   group = (int)std::min<long>(group, std::max<long>(1, 0x7fffffffL / 2 / g.L));
   Temp tmp;
-  float *gcol;
-  if (gradColumns) {
-    resize(state, gradColumns, {(long)group * g.K, g.L});
-    if (!isContiguous(erase(gradColumns))) error("gradColumns tensor has to be contiguous");
-    gcol = data(gradColumns);
-  } else {
-    tmp = Temp(s, (size_t)group * perImg * sizeof(float));
-    gcol = (float *)tmp.get();
-  }
+  float *gcol = scratchFloats(state, scratchBuf, (long)group * perImg, tmp, bufName);
   for (int n0 = 0; n0 < g.N; n0 += group) {
     int cnt = std::min(group, g.N - n0);
     GemmArgs p{};
-    p.a = data(weight);
-    p.b = go.ptr();
+    p.a = w;
+    p.b = gy;
     p.c = gcol;
     p.M = g.K;
     p.Ncols = cnt * g.L;
@@ -1333,25 +1330,30 @@ void THNN_CudaSpatialConvolutionMM_updateGradInput(THCState *state, THCudaTensor
     THC_HIP_CHECK(hipGetLastError());
     long total = (long)cnt * g.Cin * g.H * g.W;
     col2imKernel<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(
-        gcol, data(gradInput) + (long)n0 * g.Cin * g.H * g.W, cnt, g.Cin, g.H, g.W, g.kH, g.kW, g.padH, g.padW, g.dH,
-        g.dW, 1, 1, g.oH, g.oW);
+        gcol, gi + (long)n0 * g.Cin * g.H * g.W, cnt, g.Cin, g.H, g.W, g.kH, g.kW, g.padH, g.padW, g.dH, g.dW, g.dilH,
+        g.dilW, g.oH, g.oW);
     THC_HIP_CHECK(hipGetLastError());
   }
-  THNN_LEAVE
+  if (bias) {
+    const long total = (long)g.N * g.Cin * g.H * g.W;
+    addPlaneBiasKernel<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(gi, bias, total, g.H * g.W, g.Cin);
+    THC_HIP_CHECK(hipGetLastError());
+  }
 }
 
-void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput,
-                                                     THCudaTensor *gradWeight, THCudaTensor *gradBias,
-                                                     THCudaTensor *columns, THCudaTensor *ones, int kW, int kH,
-                                                     int dW, int dH, int padW, int padH, float scale) {
-  THNN_ENTER
-  (void)ones;
-  THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
-  THC_ARG_CHECK(gradWeight != nullptr, 4, "gradWeight tensor expected");
-  ConvCall call = convSetup(input, gradOutput, gradWeight, gradBias, "weight", kH, kW, dH, dW, padH, padW);
-  ConvGeom &g = call.g;
-  Contiguous in(state, input);
-  Contiguous go(state, gradOutput);
+// gB[o] += scale * sum_{n,l} gy[n][o][l] over a (N, C, L) tensor
+void convGradBias(hipStream_t s, const float *gy, float *gB, int N, int C, int L, float scale) {
+  if ((long)N * C * L == 0) return;
+  if (L % 4 == 0 && launch::aligned16(gy) && (long)N * (L / 4) < 0x7fffffffL)
+    gradBiasKernel<true><<<C, kBiasBlock, 0, s>>>(gy, gB, N, C, L, scale);
+  else
+    gradBiasKernel<false><<<C, kBiasBlock, 0, s>>>(gy, gB, N, C, L, scale);
+  THC_HIP_CHECK(hipGetLastError());
+}
+
+// gW(Cout, K) += scale * sum_n gy_n(Cout x L) * im2col(x_n)^T
+void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const float *gy, float *gW,
+                    THCudaTensor *scratchBuf, float scale) {
   if ((long)g.N * g.Cout * g.K == 0) return;
   hipStream_t s = state->stream;
 
@@ -1359,14 +1361,14 @@ void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTens
   // resident workgroup slots of the chip exactly once: with fewer, fatter
   // splits some CUs would carry one workgroup more than others for the whole
   // kernel.
-  if ((long)g.N * g.L >= 0x7fffffffL) error("SpatialConvolutionMM: batch too large");
+  if ((long)g.N * g.L >= 0x7fffffffL) error("spatial convolution: batch too large");
   const int mT = (int)tiles(g.Cout, BM), nT = (int)tiles(g.K, BN);
   const int totalKt = launch::ceilDiv(g.N * g.L, BK);
   // second-generation kernel: gradOutput rows loadable as float4 groups, 32-bit byte offsets into both operands
   const bool bordered = g.padH > 0 || g.padW > 0;
   const long gyBytes = (long)g.N * g.Cout * g.L * 4;
   const long xpFloats = (long)g.N * g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW);
-  const bool fast = !forceGeneric() && g.L % 4 == 0 && g.L >= BK && launch::aligned16(go.ptr()) &&
+  const bool fast = !forceGeneric() && g.L % 4 == 0 && g.L >= BK && launch::aligned16(gy) &&
                     gyBytes < 0x7fffffffL && xpFloats * 4 < 0x7fffffffL - 65536 && (long)g.L * g.oW < 0x7fffffffL;
   const bool l16 = g.L % BK == 0;
   const void *kern = !fast ? (const void *)convGemmKernel<kGradWeight>
@@ -1380,18 +1382,18 @@ void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTens
   // scratch: the splits' partial products, then (second-generation kernel) the images with their zero border
   const long partialFloats = (splits * count + 3) / 4 * 4;
   Temp tmp;
-  float *partial = scratchFloats(state, columns, partialFloats + (fast && bordered ? xpFloats : 0), tmp, "columns");
+  float *partial = scratchFloats(state, scratchBuf, partialFloats + (fast && bordered ? xpFloats : 0), tmp, "columns");
   if (fast) {
     ConvGeom gk = g;
-    const float *xk = in.ptr();
+    const float *xk = x;
     if (bordered) {
       float *xp = partial + partialFloats;
-      launchPadPlanes(s, in.ptr(), xp, (long)g.N * g.Cin, g.H, g.W, g.padH, g.padW);
+      launchPadPlanes(s, x, xp, (long)g.N * g.Cin, g.H, g.W, g.padH, g.padW);
       gk.H = g.H + 2 * g.padH, gk.W = g.W + 2 * g.padW, gk.padH = gk.padW = 0;
       xk = xp;
     }
     GradWeightArgs q{};
-    q.gy = go.ptr();
+    q.gy = gy;
     q.x = xk;
     q.partial = partial;
     q.M = g.Cout;
@@ -1409,8 +1411,8 @@ void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTens
       convGradWeightKernel<false><<<dim3(mT * nT * splits), dev::kBlock, 0, s>>>(q, gk);
   } else {
     GemmArgs p{};
-    p.a = go.ptr();
-    p.b = in.ptr();
+    p.a = gy;
+    p.b = x;
     p.c = partial;
     p.M = g.Cout;
     p.Ncols = g.K;
@@ -1423,16 +1425,299 @@ void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTens
     convGemmKernel<kGradWeight><<<grid, dev::kBlock, 0, s>>>(p, g);
   }
   THC_HIP_CHECK(hipGetLastError());
-  foldPartialsKernel<<<launch::directGrid(count, dev::kBlock), dev::kBlock, 0, s>>>(partial, data(gradWeight), count,
-                                                                                   splits, scale);
+  foldPartialsKernel<<<launch::directGrid(count, dev::kBlock), dev::kBlock, 0, s>>>(partial, gW, count, splits, scale);
   THC_HIP_CHECK(hipGetLastError());
-  if (gradBias) {
-    if (g.L % 4 == 0 && launch::aligned16(go.ptr()) && (long)g.N * (g.L / 4) < 0x7fffffffL)
-      gradBiasKernel<true><<<g.Cout, kBiasBlock, 0, s>>>(go.ptr(), data(gradBias), g.N, g.Cout, g.L, scale);
-    else
-      gradBiasKernel<false><<<g.Cout, kBiasBlock, 0, s>>>(go.ptr(), data(gradBias), g.N, g.Cout, g.L, scale);
-    THC_HIP_CHECK(hipGetLastError());
+}
+
+// ---- entry-point bodies shared by SpatialConvolutionMM and SpatialDilatedConvolution --------
+void convUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output, THCudaTensor *weight,
+                      THCudaTensor *bias, THCudaTensor *columns, int kW, int kH, int dW, int dH, int padW, int padH,
+                      int dilW, int dilH, ConvFlavor flavor) {
+  THC_ARG_CHECK(output != nullptr, 3, "output tensor expected");
+  ConvCall call = convSetup(input, nullptr, weight, bias, "weight", kH, kW, dH, dW, padH, padW, dilH, dilW, flavor);
+  ConvGeom &g = call.g;
+  Contiguous in(state, input);
+  if (call.batch)
+    resize(state, output, {g.N, g.Cout, g.oH, g.oW});
+  else
+    resize(state, output, {g.Cout, g.oH, g.oW});
+  if (!isContiguous(erase(output))) error("output tensor has to be contiguous");
+  convForward(state, g, in.ptr(), data(weight), bias ? data(bias) : nullptr, data(output), columns, "columns");
+}
+
+void convUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradInput,
+                         THCudaTensor *weight, THCudaTensor *gradColumns, int kW, int kH, int dW, int dH, int padW,
+                         int padH, int dilW, int dilH, ConvFlavor flavor) {
+  THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
+  THC_ARG_CHECK(gradInput != nullptr, 4, "gradInput tensor expected");
+  ConvCall call = convSetup(input, gradOutput, weight, nullptr, "weight", kH, kW, dH, dW, padH, padW, dilH, dilW, flavor);
+  ConvGeom &g = call.g;
+  Contiguous go(state, gradOutput);
+  if (call.batch)
+    resize(state, gradInput, {g.N, g.Cin, g.H, g.W});
+  else
+    resize(state, gradInput, {g.Cin, g.H, g.W});
+  if (!isContiguous(erase(gradInput))) error("gradInput tensor has to be contiguous");
+  convGradInput(state, g, go.ptr(), data(weight), data(gradInput), gradColumns, "gradColumns");
+}
+
+void convAccGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradWeight,
+                           THCudaTensor *gradBias, THCudaTensor *columns, int kW, int kH, int dW, int dH, int padW,
+                           int padH, int dilW, int dilH, float scale, ConvFlavor flavor) {
+  THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
+  THC_ARG_CHECK(gradWeight != nullptr, 4, "gradWeight tensor expected");
+  ConvCall call = convSetup(input, gradOutput, gradWeight, gradBias, "weight", kH, kW,
+                            dH, dW, padH, padW, dilH, dilW, flavor);
+  ConvGeom &g = call.g;
+  Contiguous in(state, input);
+  Contiguous go(state, gradOutput);
+  convGradWeight(state, g, in.ptr(), go.ptr(), data(gradWeight), columns, scale);
+  if (gradBias) convGradBias(state->stream, go.ptr(), data(gradBias), g.N, g.Cout, g.L, scale);
+}
+
+// ---- transposed ("full") convolution -----------------------------------------------------------
+// SpatialFull(Dilated)Convolution maps the (N, Cin, H, W) input to (N, Cout, oH, oW) with
+// oH = (H-1)*dH - 2*padH + dilH*(kH-1) + 1 + adjH; its weight is (Cin, Cout, kH, kW). It is the
+// ordinary convolution C with input (N, Cout, oH, oW), output (N, Cin, H, W) and weight
+// (Cin, Cout*kH*kW) run backwards: updateOutput = C's gradInput pass (+ bias), updateGradInput =
+// C's forward pass, accGradParameters = C's weight-gradient pass with the roles of input and
+// gradOutput swapped (lib/THCUNN/generic/SpatialFullDilatedConvolution.cu:141-165, 268-298, 385-414).
+// The geometry returned here is C's.
+ConvCall fullSetup(THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *weight, THCudaTensor *bias, int kH,
+                   int kW, int dH, int dW, int padH, int padW, int dilH, int dilW, int adjH, int adjW) {
+  // lib/THCUNN/generic/SpatialFullDilatedConvolution.cu:5-66
+  THC_ARG_CHECK(input && weight, 2, "input and weight tensors expected");
+  THC_ARG_CHECK(kW > 0 && kH > 0, 9, "kernel size should be greater than zero, but got kH: %d kW: %d", kH, kW);
+  THC_ARG_CHECK(dW > 0 && dH > 0, 11, "stride should be greater than zero, but got dH: %d dW: %d", dH, dW);
+  THC_ARG_CHECK(dilW > 0 && dilH > 0, 15, "dilation should be greater than zero, but got dilationH: %d, dilationW: %d",
+                dilH, dilW);
+  THC_ARG_CHECK((adjW < dW || adjW < dilW) && (adjH < dH || adjH < dilH), 15,
+                "output padding must be smaller than either stride or dilation, but got adjH: %d adjW: %d dH: %d dW: %d "
+                "dilationH: %d dilationW: %d",
+                adjH, adjW, dH, dW, dilH, dilW);
+  THC_ARG_CHECK(isContiguous(erase(weight)), 4, "weight tensor has to be contiguous");
+  THC_ARG_CHECK(!bias || isContiguous(erase(bias)), 5, "bias tensor has to be contiguous");
+  THC_ARG_CHECK(weight->nDimension == 2 || weight->nDimension == 4, 5, "2D or 4D weight tensor expected, but got: %s",
+                sizeDesc(erase(weight)).c_str());
+  if (bias) checkDimSize(erase(bias), "bias", 1, 0, weight->size[1]);
+  int ndim = input->nDimension;
+  int dimf = 0, dimh = 1, dimw = 2;
+  if (ndim == 4) {
+    dimf++;
+    dimh++;
+    dimw++;
   }
+  THC_ARG_CHECK(ndim == 3 || ndim == 4, 2, "3D or 4D input tensor expected but got: %s",
+                sizeDesc(erase(input)).c_str());
+  if (weight->nDimension != 4) error("transposed convolution: 4D weight tensor (nInputPlane,nOutputPlane,kH,kW) expected");
+  long nInputPlane = weight->size[0], nOutputPlane = weight->size[1];
+  long inputHeight = input->size[dimh], inputWidth = input->size[dimw];
+  long outputHeight = (inputHeight - 1) * dH - 2 * padH + (dilH * (kH - 1) + 1) + adjH;
+  long outputWidth = (inputWidth - 1) * dW - 2 * padW + (dilW * (kW - 1) + 1) + adjW;
+  if (outputWidth < 1 || outputHeight < 1)
+    error("Given input size: (%ld x %ld x %ld). Calculated output size: (%ld x %ld x %ld). Output size is too small",
+          nInputPlane, inputHeight, inputWidth, nOutputPlane, outputHeight, outputWidth);
+  checkDimSize(erase(input), "input", ndim, dimf, nInputPlane);
+  if (gradOutput) {
+    checkDimSize(erase(gradOutput), "gradOutput", ndim, dimf, nOutputPlane);
+    checkDimSize(erase(gradOutput), "gradOutput", ndim, dimh, outputHeight);
+    checkDimSize(erase(gradOutput), "gradOutput", ndim, dimw, outputWidth);
+    if (ndim == 4 && gradOutput->size[0] != input->size[0])
+      error("input and gradOutput batch sizes do not match: input %s, gradOutput %s", sizeDesc(erase(input)).c_str(),
+            sizeDesc(erase(gradOutput)).c_str());
+  }
+  if (weight->size[2] != kH || weight->size[3] != kW)
+    error("weight of shape %s does not match a %d x %d kernel", sizeDesc(erase(weight)).c_str(), kH, kW);
+  ConvCall call;
+  call.batch = ndim == 4;
+  call.g = makeGeom(call.batch ? (int)input->size[0] : 1, (int)nOutputPlane, (int)nInputPlane, (int)outputHeight,
+                    (int)outputWidth, (int)inputHeight, (int)inputWidth, kH, kW, dH, dW, padH, padW, dilH, dilW);
+  return call;
+}
+
+void fullUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output, THCudaTensor *weight,
+                      THCudaTensor *bias, THCudaTensor *columns, int kW, int kH, int dW, int dH, int padW, int padH,
+                      int dilW, int dilH, int adjW, int adjH) {
+  THC_ARG_CHECK(output != nullptr, 3, "output tensor expected");
+  ConvCall call = fullSetup(input, nullptr, weight, bias, kH, kW, dH, dW, padH, padW, dilH, dilW, adjH, adjW);
+  ConvGeom &g = call.g;
+  Contiguous in(state, input);
+  if (call.batch)
+    resize(state, output, {g.N, g.Cin, g.H, g.W});
+  else
+    resize(state, output, {g.Cin, g.H, g.W});
+  if (!isContiguous(erase(output))) error("output tensor has to be contiguous");
+  convGradInput(state, g, in.ptr(), data(weight), data(output), columns, "columns", bias ? data(bias) : nullptr);
+}
+
+void fullUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradInput,
+                         THCudaTensor *weight, THCudaTensor *gradColumns, int kW, int kH, int dW, int dH, int padW,
+                         int padH, int dilW, int dilH, int adjW, int adjH) {
+  THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
+  THC_ARG_CHECK(gradInput != nullptr, 4, "gradInput tensor expected");
+  ConvCall call = fullSetup(input, gradOutput, weight, nullptr, kH, kW, dH, dW, padH, padW, dilH, dilW, adjH, adjW);
+  ConvGeom &g = call.g;
+  Contiguous go(state, gradOutput);
+  if (call.batch)
+    resize(state, gradInput, {g.N, g.Cout, g.oH, g.oW});
+  else
+    resize(state, gradInput, {g.Cout, g.oH, g.oW});
+  if (!isContiguous(erase(gradInput))) error("gradInput tensor has to be contiguous");
+  convForward(state, g, go.ptr(), data(weight), nullptr, data(gradInput), gradColumns, "gradColumns");
+}
+
+void fullAccGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradWeight,
+                           THCudaTensor *gradBias, THCudaTensor *columns, int kW, int kH, int dW, int dH, int padW,
+                           int padH, int dilW, int dilH, int adjW, int adjH, float scale) {
+  THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
+  THC_ARG_CHECK(gradWeight != nullptr, 4, "gradWeight tensor expected");
+  ConvCall call = fullSetup(input, gradOutput, gradWeight, gradBias, kH, kW, dH, dW, padH, padW, dilH, dilW, adjH, adjW);
+  ConvGeom &g = call.g;
+  Contiguous in(state, input);
+  Contiguous go(state, gradOutput);
+  convGradWeight(state, g, go.ptr(), in.ptr(), data(gradWeight), columns, scale);
+  if (gradBias) convGradBias(state->stream, go.ptr(), data(gradBias), g.N, g.Cin, g.H * g.W, scale);
+}
+
+}  // namespace
+
+extern "C" {
+
+void THNN_CudaSpatialConvolutionMM_updateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output,
+                                                THCudaTensor *weight, THCudaTensor *bias, THCudaTensor *columns,
+                                                THCudaTensor *ones, int kW, int kH, int dW, int dH, int padW,
+                                                int padH) {
+  THNN_ENTER
+  (void)ones;  // never read; `columns` is used (and resized) only as scratch
+  convUpdateOutput(state, input, output, weight, bias, columns, kW, kH, dW, dH, padW, padH, 1, 1, kConvMM);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialConvolutionMM_updateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput,
+                                                   THCudaTensor *gradInput, THCudaTensor *weight,
+                                                   THCudaTensor *gradColumns, THCudaTensor *ones, int kW, int kH,
+                                                   int dW, int dH, int padW, int padH) {
+  THNN_ENTER
+  (void)ones;
+  convUpdateGradInput(state, input, gradOutput, gradInput, weight, gradColumns, kW, kH, dW, dH, padW, padH, 1, 1, kConvMM);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialConvolutionMM_accGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput,
+                                                     THCudaTensor *gradWeight, THCudaTensor *gradBias,
+                                                     THCudaTensor *columns, THCudaTensor *ones, int kW, int kH,
+                                                     int dW, int dH, int padW, int padH, float scale) {
+  THNN_ENTER
+  (void)ones;
+  convAccGradParameters(state, input, gradOutput, gradWeight, gradBias, columns, kW, kH, dW, dH, padW, padH, 1, 1, scale,
+                        kConvMM);
+  THNN_LEAVE
+}
+
+// SpatialDilatedConvolution (lib/THCUNN/generic/SpatialDilatedConvolution.cu:69-190, 192-293, 295-432):
+// the same three GEMMs with taps dilationH/W apart.
+void THNN_CudaSpatialDilatedConvolution_updateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output,
+                                                     THCudaTensor *weight, THCudaTensor *bias, THCudaTensor *columns,
+                                                     THCudaTensor *ones, int kW, int kH, int dW, int dH, int padW,
+                                                     int padH, int dilationW, int dilationH) {
+  THNN_ENTER
+  (void)ones;
+  convUpdateOutput(state, input, output, weight, bias, columns, kW, kH, dW, dH, padW, padH, dilationW, dilationH,
+                   kDilated);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialDilatedConvolution_updateGradInput(THCState *state, THCudaTensor *input,
+                                                        THCudaTensor *gradOutput, THCudaTensor *gradInput,
+                                                        THCudaTensor *weight, THCudaTensor *gradColumns, int kW,
+                                                        int kH, int dW, int dH, int padW, int padH, int dilationW,
+                                                        int dilationH) {
+  THNN_ENTER
+  convUpdateGradInput(state, input, gradOutput, gradInput, weight, gradColumns, kW, kH, dW, dH, padW, padH, dilationW,
+                      dilationH, kDilated);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialDilatedConvolution_accGradParameters(THCState *state, THCudaTensor *input,
+                                                          THCudaTensor *gradOutput, THCudaTensor *gradWeight,
+                                                          THCudaTensor *gradBias, THCudaTensor *columns,
+                                                          THCudaTensor *ones, int kW, int kH, int dW, int dH,
+                                                          int padW, int padH, int dilationW, int dilationH,
+                                                          float scale) {
+  THNN_ENTER
+  (void)ones;
+  convAccGradParameters(state, input, gradOutput, gradWeight, gradBias, columns, kW, kH, dW, dH, padW, padH, dilationW,
+                        dilationH, scale, kDilated);
+  THNN_LEAVE
+}
+
+// SpatialFullDilatedConvolution / SpatialFullConvolution
+// (lib/THCUNN/generic/SpatialFullDilatedConvolution.cu:68-204, 206-312, 314-465; generic/SpatialFullConvolution.cu:5-59)
+void THNN_CudaSpatialFullDilatedConvolution_updateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output,
+                                                         THCudaTensor *weight, THCudaTensor *bias,
+                                                         THCudaTensor *columns, THCudaTensor *ones, int kW, int kH,
+                                                         int dW, int dH, int padW, int padH, int dilationW,
+                                                         int dilationH, int adjW, int adjH) {
+  THNN_ENTER
+  (void)ones;
+  fullUpdateOutput(state, input, output, weight, bias, columns, kW, kH, dW, dH, padW, padH, dilationW, dilationH, adjW,
+                   adjH);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialFullDilatedConvolution_updateGradInput(THCState *state, THCudaTensor *input,
+                                                            THCudaTensor *gradOutput, THCudaTensor *gradInput,
+                                                            THCudaTensor *weight, THCudaTensor *gradColumns, int kW,
+                                                            int kH, int dW, int dH, int padW, int padH,
+                                                            int dilationW, int dilationH, int adjW, int adjH) {
+  THNN_ENTER
+  fullUpdateGradInput(state, input, gradOutput, gradInput, weight, gradColumns, kW, kH, dW, dH, padW, padH, dilationW,
+                      dilationH, adjW, adjH);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialFullDilatedConvolution_accGradParameters(THCState *state, THCudaTensor *input,
+                                                              THCudaTensor *gradOutput, THCudaTensor *gradWeight,
+                                                              THCudaTensor *gradBias, THCudaTensor *columns,
+                                                              THCudaTensor *ones, int kW, int kH, int dW, int dH,
+                                                              int padW, int padH, int dilationW, int dilationH,
+                                                              int adjW, int adjH, float scale) {
+  THNN_ENTER
+  (void)ones;
+  fullAccGradParameters(state, input, gradOutput, gradWeight, gradBias, columns, kW, kH, dW, dH, padW, padH, dilationW,
+                        dilationH, adjW, adjH, scale);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialFullConvolution_updateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output,
+                                                  THCudaTensor *weight, THCudaTensor *bias, THCudaTensor *columns,
+                                                  THCudaTensor *ones, int kW, int kH, int dW, int dH, int padW,
+                                                  int padH, int adjW, int adjH) {
+  THNN_ENTER
+  (void)ones;
+  fullUpdateOutput(state, input, output, weight, bias, columns, kW, kH, dW, dH, padW, padH, 1, 1, adjW, adjH);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialFullConvolution_updateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput,
+                                                     THCudaTensor *gradInput, THCudaTensor *weight,
+                                                     THCudaTensor *gradColumns, int kW, int kH, int dW, int dH,
+                                                     int padW, int padH, int adjW, int adjH) {
+  THNN_ENTER
+  fullUpdateGradInput(state, input, gradOutput, gradInput, weight, gradColumns, kW, kH, dW, dH, padW, padH, 1, 1, adjW,
+                      adjH);
+  THNN_LEAVE
+}
+
+void THNN_CudaSpatialFullConvolution_accGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput,
+                                                       THCudaTensor *gradWeight, THCudaTensor *gradBias,
+                                                       THCudaTensor *columns, THCudaTensor *ones, int kW, int kH,
+                                                       int dW, int dH, int padW, int padH, int adjW, int adjH,
+                                                       float scale) {
+  THNN_ENTER
+  (void)ones;
+  fullAccGradParameters(state, input, gradOutput, gradWeight, gradBias, columns, kW, kH, dW, dH, padW, padH, 1, 1, adjW,
+                        adjH, scale);
   THNN_LEAVE
 }
 

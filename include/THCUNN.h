@@ -126,6 +126,70 @@ void THNN_CudaSpatialMaxPooling_updateGradInput(
     THCudaLongTensor *indices,
     int kW, int kH, int dW, int dH, int padW, int padH, bool ceil_mode);
 
+/* ---- next after the hot path: dilated and transposed convolution -------------
+ * Same im2col/col2im + fp32 MFMA GEMM passes as SpatialConvolutionMM. */
+
+/* replaces lib/THCUNN/generic/THCUNN.h:727-738, lib/THCUNN/generic/SpatialDilatedConvolution.cu:69-190 */
+void THNN_CudaSpatialDilatedConvolution_updateOutput(
+    THCState *state, THCudaTensor *input, THCudaTensor *output, THCudaTensor *weight,
+    THCudaTensor *bias,         /* [OPTIONAL] */
+    THCudaTensor *columns, THCudaTensor *ones,
+    int kW, int kH, int dW, int dH, int padW, int padH, int dilationW, int dilationH);
+
+/* replaces lib/THCUNN/generic/THCUNN.h:740-750, lib/THCUNN/generic/SpatialDilatedConvolution.cu:192-293 */
+void THNN_CudaSpatialDilatedConvolution_updateGradInput(
+    THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradInput,
+    THCudaTensor *weight, THCudaTensor *gradColumns,
+    int kW, int kH, int dW, int dH, int padW, int padH, int dilationW, int dilationH);
+
+/* replaces lib/THCUNN/generic/THCUNN.h:752-764, lib/THCUNN/generic/SpatialDilatedConvolution.cu:295-432 */
+void THNN_CudaSpatialDilatedConvolution_accGradParameters(
+    THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradWeight,
+    THCudaTensor *gradBias,     /* [OPTIONAL] */
+    THCudaTensor *columns, THCudaTensor *ones,
+    int kW, int kH, int dW, int dH, int padW, int padH, int dilationW, int dilationH, float scale);
+
+/* replaces lib/THCUNN/generic/THCUNN.h:766-778, lib/THCUNN/generic/SpatialFullDilatedConvolution.cu:68-204 */
+void THNN_CudaSpatialFullDilatedConvolution_updateOutput(
+    THCState *state, THCudaTensor *input, THCudaTensor *output, THCudaTensor *weight,
+    THCudaTensor *bias,         /* [OPTIONAL] */
+    THCudaTensor *columns, THCudaTensor *ones,
+    int kW, int kH, int dW, int dH, int padW, int padH, int dilationW, int dilationH, int adjW, int adjH);
+
+/* replaces lib/THCUNN/generic/THCUNN.h:780-791, lib/THCUNN/generic/SpatialFullDilatedConvolution.cu:206-312 */
+void THNN_CudaSpatialFullDilatedConvolution_updateGradInput(
+    THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradInput,
+    THCudaTensor *weight, THCudaTensor *gradColumns,
+    int kW, int kH, int dW, int dH, int padW, int padH, int dilationW, int dilationH, int adjW, int adjH);
+
+/* replaces lib/THCUNN/generic/THCUNN.h:793-806, lib/THCUNN/generic/SpatialFullDilatedConvolution.cu:314-465 */
+void THNN_CudaSpatialFullDilatedConvolution_accGradParameters(
+    THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradWeight,
+    THCudaTensor *gradBias,     /* [OPTIONAL] */
+    THCudaTensor *columns, THCudaTensor *ones,
+    int kW, int kH, int dW, int dH, int padW, int padH, int dilationW, int dilationH, int adjW, int adjH,
+    float scale);
+
+/* replaces lib/THCUNN/generic/THCUNN.h:849-860, lib/THCUNN/generic/SpatialFullConvolution.cu:5-22 */
+void THNN_CudaSpatialFullConvolution_updateOutput(
+    THCState *state, THCudaTensor *input, THCudaTensor *output, THCudaTensor *weight,
+    THCudaTensor *bias,         /* [OPTIONAL] */
+    THCudaTensor *columns, THCudaTensor *ones,
+    int kW, int kH, int dW, int dH, int padW, int padH, int adjW, int adjH);
+
+/* replaces lib/THCUNN/generic/THCUNN.h:862-872, lib/THCUNN/generic/SpatialFullConvolution.cu:24-39 */
+void THNN_CudaSpatialFullConvolution_updateGradInput(
+    THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradInput,
+    THCudaTensor *weight, THCudaTensor *gradColumns,
+    int kW, int kH, int dW, int dH, int padW, int padH, int adjW, int adjH);
+
+/* replaces lib/THCUNN/generic/THCUNN.h:874-886, lib/THCUNN/generic/SpatialFullConvolution.cu:41-59 */
+void THNN_CudaSpatialFullConvolution_accGradParameters(
+    THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradWeight,
+    THCudaTensor *gradBias,     /* [OPTIONAL] */
+    THCudaTensor *columns, THCudaTensor *ones,
+    int kW, int kH, int dW, int dH, int padW, int padH, int adjW, int adjH, float scale);
+
 #ifdef __cplusplus
 }
 #endif

@@ -155,6 +155,93 @@ def convmm_accGradParameters(x, gradOut, gradWeight, gradBias, kW, kH, dW, dH, p
     return gradWeight, gradBias
 
 
+# ------------------------------------------------- dilated convolution ----
+def dilconv_updateOutput(x, weight, bias, kW, kH, dW, dH, padW, padH, dilW, dilH):
+    x = _f(x)
+    N, Cin, H, W = x.shape
+    weight = _f(weight).reshape(weight.shape[0], -1)
+    Cout = weight.shape[0]
+    assert weight.shape[1] == Cin * kH * kW
+    bias = None if bias is None else _f(bias)
+    oH, oW = conv_out_size(H, kH, dH, padH, dilH), conv_out_size(W, kW, dW, padW, dilW)
+    out = np.empty((N, Cout, oH, oW), np.float32)
+    lib().oracle_dilconv_updateOutput(_p(x), _p(weight), _p(bias), _p(out), N, Cin, Cout, H, W,
+                                      kW, kH, dW, dH, padW, padH, dilW, dilH)
+    return out
+
+
+def dilconv_updateGradInput(x_shape, gradOut, weight, kW, kH, dW, dH, padW, padH, dilW, dilH):
+    gradOut = _f(gradOut)
+    N, Cin, H, W = x_shape
+    weight = _f(weight).reshape(weight.shape[0], -1)
+    gi = np.empty((N, Cin, H, W), np.float32)
+    lib().oracle_dilconv_updateGradInput(_p(gradOut), _p(weight), _p(gi), N, Cin, weight.shape[0], H, W,
+                                         kW, kH, dW, dH, padW, padH, dilW, dilH)
+    return gi
+
+
+def dilconv_accGradParameters(x, gradOut, gradWeight, gradBias, kW, kH, dW, dH, padW, padH, dilW, dilH, scale=1.0):
+    x, gradOut = _f(x), _f(gradOut)
+    N, Cin, H, W = x.shape
+    assert gradWeight.dtype == np.float32 and gradWeight.flags.c_contiguous
+    lib().oracle_dilconv_accGradParameters(_p(x), _p(gradOut), _p(gradWeight), _p(gradBias), N, Cin,
+                                           gradWeight.shape[0], H, W, kW, kH, dW, dH, padW, padH, dilW, dilH,
+                                           C.c_float(scale))
+    return gradWeight, gradBias
+
+
+# ---------------------------------------------- transposed convolution ----
+def full_out_size(n, k, d, pad, dil, adj):
+    return (n - 1) * d - 2 * pad + (dil * (k - 1) + 1) + adj
+
+
+def fullconv_updateOutput(x, weight, bias, kW, kH, dW, dH, padW, padH, dilW=1, dilH=1, adjW=0, adjH=0):
+    """weight (Cin, Cout, kH, kW)"""
+    x, weight = _f(x), _f(weight)
+    N, Cin, H, W = x.shape
+    Cout = weight.shape[1]
+    assert weight.shape == (Cin, Cout, kH, kW)
+    bias = None if bias is None else _f(bias)
+    oH, oW = full_out_size(H, kH, dH, padH, dilH, adjH), full_out_size(W, kW, dW, padW, dilW, adjW)
+    out = np.empty((N, Cout, oH, oW), np.float32)
+    lib().oracle_fullconv_updateOutput(_p(x), _p(weight), _p(bias), _p(out), N, Cin, Cout, H, W, oH, oW,
+                                       kW, kH, dW, dH, padW, padH, dilW, dilH)
+    return out
+
+
+def _full_check(H, W, oH, oW, kW, kH, dW, dH, padW, padH, dilW, dilH):
+    # The reference's im2col over the output-sized image produces conv_out(oH) x conv_out(oW) columns and
+    # assumes that this is H x W (generic/SpatialFullDilatedConvolution.cu:255, 268-273); with an output
+    # padding >= stride (allowed when it is < dilation) that does not hold and the reference overruns its buffer.
+    if conv_out_size(oH, kH, dH, padH, dilH) != H or conv_out_size(oW, kW, dW, padW, dilW) != W:
+        raise ValueError("output padding >= stride: not defined by the reference's backward passes")
+
+
+def fullconv_updateGradInput(x_shape, gradOut, weight, kW, kH, dW, dH, padW, padH, dilW=1, dilH=1, adjW=0, adjH=0):
+    gradOut, weight = _f(gradOut), _f(weight)
+    N, Cin, H, W = x_shape
+    Cout = weight.shape[1]
+    oH, oW = gradOut.shape[2:]
+    _full_check(H, W, oH, oW, kW, kH, dW, dH, padW, padH, dilW, dilH)
+    gi = np.empty((N, Cin, H, W), np.float32)
+    lib().oracle_fullconv_updateGradInput(_p(gradOut), _p(weight), _p(gi), N, Cin, Cout, H, W, oH, oW,
+                                          kW, kH, dW, dH, padW, padH, dilW, dilH)
+    return gi
+
+
+def fullconv_accGradParameters(x, gradOut, gradWeight, gradBias, kW, kH, dW, dH, padW, padH, dilW=1, dilH=1,
+                               adjW=0, adjH=0, scale=1.0):
+    x, gradOut = _f(x), _f(gradOut)
+    N, Cin, H, W = x.shape
+    Cout = gradWeight.shape[1]
+    oH, oW = gradOut.shape[2:]
+    _full_check(H, W, oH, oW, kW, kH, dW, dH, padW, padH, dilW, dilH)
+    assert gradWeight.dtype == np.float32 and gradWeight.flags.c_contiguous
+    lib().oracle_fullconv_accGradParameters(_p(x), _p(gradOut), _p(gradWeight), _p(gradBias), N, Cin, Cout,
+                                            H, W, oH, oW, kW, kH, dW, dH, padW, padH, dilW, dilH, C.c_float(scale))
+    return gradWeight, gradBias
+
+
 # -------------------------------------------------------------------- BN ----
 def _ncl(x):
     x = _f(x)

@@ -252,10 +252,10 @@ void oracle_dwconv_accGradParameters(const float *in, const float *gradOut, floa
 
 /* generic/SpatialConvolutionMM.cu:129-194: per sample: out = bias broadcast
  * (or zero); im2col; out(Cout x L) += W(Cout x K) * col(K x L) */
-void oracle_convmm_updateOutput(const float *in, const float *weight, const float *bias, float *out,
-                                int N, int Cin, int Cout, int H, int W, int kW, int kH, int dW,
-                                int dH, int padW, int padH) {
-  int oH = conv_out(H, padH, kH, dH, 1), oW = conv_out(W, padW, kW, dW, 1);
+static void conv_forward(const float *in, const float *weight, const float *bias, float *out,
+                         int N, int Cin, int Cout, int H, int W, int kW, int kH, int dW,
+                         int dH, int padW, int padH, int dilW, int dilH) {
+  int oH = conv_out(H, padH, kH, dH, dilH), oW = conv_out(W, padW, kW, dW, dilW);
   int K = Cin * kH * kW, L = oH * oW;
   float *col = (float *)malloc(sizeof(float) * (size_t)K * L);
   for (int n = 0; n < N; ++n) {
@@ -264,46 +264,140 @@ void oracle_convmm_updateOutput(const float *in, const float *weight, const floa
       float b = bias ? bias[oc] : 0.f;
       for (int l = 0; l < L; ++l) o[(size_t)oc * L + l] = b;
     }
-    oracle_im2col(in + (size_t)n * Cin * H * W, Cin, H, W, kH, kW, padH, padW, dH, dW, 1, 1, col);
+    oracle_im2col(in + (size_t)n * Cin * H * W, Cin, H, W, kH, kW, padH, padW, dH, dW, dilH, dilW, col);
     gemm_nn(Cout, L, K, 1.f, weight, col, 1.f, o);
   }
   free(col);
 }
+void oracle_convmm_updateOutput(const float *in, const float *weight, const float *bias, float *out,
+                                int N, int Cin, int Cout, int H, int W, int kW, int kH, int dW,
+                                int dH, int padW, int padH) {
+  conv_forward(in, weight, bias, out, N, Cin, Cout, H, W, kW, kH, dW, dH, padW, padH, 1, 1);
+}
+/* generic/SpatialDilatedConvolution.cu:69-190: the same per-sample bias fill, im2col (with
+ * dilation, im2col.h:24-36) and GEMM */
+void oracle_dilconv_updateOutput(const float *in, const float *weight, const float *bias, float *out,
+                                 int N, int Cin, int Cout, int H, int W, int kW, int kH, int dW,
+                                 int dH, int padW, int padH, int dilW, int dilH) {
+  conv_forward(in, weight, bias, out, N, Cin, Cout, H, W, kW, kH, dW, dH, padW, padH, dilW, dilH);
+}
 
 /* generic/SpatialConvolutionMM.cu:272-308: per sample: gradCol(K x L) =
  * W^T * gradOut_n ; gradIn_n = col2im(gradCol) */
-void oracle_convmm_updateGradInput(const float *gradOut, const float *weight, float *gradIn, int N,
-                                   int Cin, int Cout, int H, int W, int kW, int kH, int dW, int dH,
-                                   int padW, int padH) {
-  int oH = conv_out(H, padH, kH, dH, 1), oW = conv_out(W, padW, kW, dW, 1);
+static void conv_grad_input(const float *gradOut, const float *weight, float *gradIn, int N,
+                            int Cin, int Cout, int H, int W, int kW, int kH, int dW, int dH,
+                            int padW, int padH, int dilW, int dilH) {
+  int oH = conv_out(H, padH, kH, dH, dilH), oW = conv_out(W, padW, kW, dW, dilW);
   int K = Cin * kH * kW, L = oH * oW;
   float *col = (float *)malloc(sizeof(float) * (size_t)K * L);
   for (int n = 0; n < N; ++n) {
     gemm_tn(Cout, L, K, weight, gradOut + (size_t)n * Cout * L, col);
-    oracle_col2im(col, Cin, H, W, oH, oW, kH, kW, padH, padW, dH, dW, 1, 1,
+    oracle_col2im(col, Cin, H, W, oH, oW, kH, kW, padH, padW, dH, dW, dilH, dilW,
                   gradIn + (size_t)n * Cin * H * W);
   }
   free(col);
+}
+void oracle_convmm_updateGradInput(const float *gradOut, const float *weight, float *gradIn, int N,
+                                   int Cin, int Cout, int H, int W, int kW, int kH, int dW, int dH,
+                                   int padW, int padH) {
+  conv_grad_input(gradOut, weight, gradIn, N, Cin, Cout, H, W, kW, kH, dW, dH, padW, padH, 1, 1);
+}
+/* generic/SpatialDilatedConvolution.cu:192-293 */
+void oracle_dilconv_updateGradInput(const float *gradOut, const float *weight, float *gradIn, int N,
+                                    int Cin, int Cout, int H, int W, int kW, int kH, int dW, int dH,
+                                    int padW, int padH, int dilW, int dilH) {
+  conv_grad_input(gradOut, weight, gradIn, N, Cin, Cout, H, W, kW, kH, dW, dH, padW, padH, dilW, dilH);
 }
 
 /* generic/SpatialConvolutionMM.cu:396-470: per sample: im2col;
  * gradW(Cout x K) += scale * gradOut_n(Cout x L) * col^T (beta = 1);
  * gradBias += scale * gradOut_n * ones */
-void oracle_convmm_accGradParameters(const float *in, const float *gradOut, float *gradWeight,
-                                     float *gradBias, int N, int Cin, int Cout, int H, int W, int kW,
-                                     int kH, int dW, int dH, int padW, int padH, float scale) {
-  int oH = conv_out(H, padH, kH, dH, 1), oW = conv_out(W, padW, kW, dW, 1);
+static void conv_acc_grad(const float *in, const float *gradOut, float *gradWeight,
+                          float *gradBias, int N, int Cin, int Cout, int H, int W, int kW,
+                          int kH, int dW, int dH, int padW, int padH, int dilW, int dilH, float scale) {
+  int oH = conv_out(H, padH, kH, dH, dilH), oW = conv_out(W, padW, kW, dW, dilW);
   int K = Cin * kH * kW, L = oH * oW;
   float *col = (float *)malloc(sizeof(float) * (size_t)K * L);
   for (int n = 0; n < N; ++n) {
     const float *g = gradOut + (size_t)n * Cout * L;
-    oracle_im2col(in + (size_t)n * Cin * H * W, Cin, H, W, kH, kW, padH, padW, dH, dW, 1, 1, col);
+    oracle_im2col(in + (size_t)n * Cin * H * W, Cin, H, W, kH, kW, padH, padW, dH, dW, dilH, dilW, col);
     gemm_nt_acc(Cout, K, L, scale, g, col, gradWeight);
     if (gradBias)
       for (int oc = 0; oc < Cout; ++oc) {
         double s = 0.0;
         for (int l = 0; l < L; ++l) s += (double)g[(size_t)oc * L + l];
         gradBias[oc] += scale * (float)s;
+      }
+  }
+  free(col);
+}
+void oracle_convmm_accGradParameters(const float *in, const float *gradOut, float *gradWeight,
+                                     float *gradBias, int N, int Cin, int Cout, int H, int W, int kW,
+                                     int kH, int dW, int dH, int padW, int padH, float scale) {
+  conv_acc_grad(in, gradOut, gradWeight, gradBias, N, Cin, Cout, H, W, kW, kH, dW, dH, padW, padH, 1, 1, scale);
+}
+/* generic/SpatialDilatedConvolution.cu:295-432 */
+void oracle_dilconv_accGradParameters(const float *in, const float *gradOut, float *gradWeight,
+                                      float *gradBias, int N, int Cin, int Cout, int H, int W, int kW,
+                                      int kH, int dW, int dH, int padW, int padH, int dilW, int dilH,
+                                      float scale) {
+  conv_acc_grad(in, gradOut, gradWeight, gradBias, N, Cin, Cout, H, W, kW, kH, dW, dH, padW, padH, dilW, dilH, scale);
+}
+
+/* ------------------------------------------ SpatialFull(Dilated)Convolution --
+ * weight (Cin, Cout, kH, kW) = (Cin, Cout*kH*kW), bias (Cout) or NULL, input (N, Cin, H, W),
+ * output (N, Cout, oH, oW) with oH = (H-1)*dH - 2*padH + dilH*(kH-1) + 1 + adjH
+ * (lib/THCUNN/generic/SpatialFullDilatedConvolution.cu:104-105). */
+
+/* generic/SpatialFullDilatedConvolution.cu:129-193: per sample:
+ * columns(Cout*kH*kW x H*W) = W^T * input_n ; output_n = col2im(columns) ; output_n += bias */
+void oracle_fullconv_updateOutput(const float *in, const float *weight, const float *bias, float *out,
+                                  int N, int Cin, int Cout, int H, int W, int oH, int oW, int kW, int kH,
+                                  int dW, int dH, int padW, int padH, int dilW, int dilH) {
+  int Kf = Cout * kH * kW, HW = H * W;
+  float *col = (float *)malloc(sizeof(float) * (size_t)Kf * HW);
+  for (int n = 0; n < N; ++n) {
+    float *o = out + (size_t)n * Cout * oH * oW;
+    gemm_tn(Cin, HW, Kf, weight, in + (size_t)n * Cin * HW, col);
+    oracle_col2im(col, Cout, oH, oW, H, W, kH, kW, padH, padW, dH, dW, dilH, dilW, o);
+    if (bias)
+      for (int oc = 0; oc < Cout; ++oc)
+        for (int l = 0; l < oH * oW; ++l) o[(size_t)oc * oH * oW + l] += bias[oc];
+  }
+  free(col);
+}
+
+/* generic/SpatialFullDilatedConvolution.cu:262-298: per sample:
+ * gradColumns = im2col(gradOutput_n) ; gradInput_n(Cin x H*W) = W * gradColumns */
+void oracle_fullconv_updateGradInput(const float *gradOut, const float *weight, float *gradIn, int N,
+                                     int Cin, int Cout, int H, int W, int oH, int oW, int kW, int kH,
+                                     int dW, int dH, int padW, int padH, int dilW, int dilH) {
+  int Kf = Cout * kH * kW, HW = H * W;
+  float *col = (float *)malloc(sizeof(float) * (size_t)Kf * HW);
+  for (int n = 0; n < N; ++n) {
+    oracle_im2col(gradOut + (size_t)n * Cout * oH * oW, Cout, oH, oW, kH, kW, padH, padW, dH, dW, dilH, dilW, col);
+    gemm_nn(Cin, HW, Kf, 1.f, weight, col, 0.f, gradIn + (size_t)n * Cin * HW);
+  }
+  free(col);
+}
+
+/* generic/SpatialFullDilatedConvolution.cu:379-453: per sample: columns = im2col(gradOutput_n);
+ * gradWeight(Cin x Cout*kH*kW) += scale * input_n * columns^T ; gradBias += scale * gradOutput_n * ones */
+void oracle_fullconv_accGradParameters(const float *in, const float *gradOut, float *gradWeight,
+                                       float *gradBias, int N, int Cin, int Cout, int H, int W, int oH,
+                                       int oW, int kW, int kH, int dW, int dH, int padW, int padH, int dilW,
+                                       int dilH, float scale) {
+  int Kf = Cout * kH * kW, HW = H * W;
+  float *col = (float *)malloc(sizeof(float) * (size_t)Kf * HW);
+  for (int n = 0; n < N; ++n) {
+    const float *g = gradOut + (size_t)n * Cout * oH * oW;
+    oracle_im2col(g, Cout, oH, oW, kH, kW, padH, padW, dH, dW, dilH, dilW, col);
+    gemm_nt_acc(Cin, Kf, HW, scale, in + (size_t)n * Cin * HW, col, gradWeight);
+    if (gradBias)
+      for (int oc = 0; oc < Cout; ++oc) {
+        double sum = 0.0;
+        for (int l = 0; l < oH * oW; ++l) sum += (double)g[(size_t)oc * oH * oW + l];
+        gradBias[oc] += scale * (float)sum;
       }
   }
   free(col);

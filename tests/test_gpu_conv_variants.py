@@ -1,0 +1,188 @@
+"""GPU parity of SpatialDilatedConvolution and SpatialFull(Dilated)Convolution through the C ABI
+against the CPU oracle (same tolerances as SpatialConvolutionMM: 1e-5 rel / 1e-4 abs outputs and
+gradients, 1e-3 rel weight gradients). The cases cover every kernel path: zero-bordered fast
+kernels (K % 16 == 0), generic kernels, stride-1 gradInput through the forward kernel, gradient
+columns + col2im, output padding, 3-D inputs, non-contiguous inputs, accumulation with scale."""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from oracle import oracle as O  # noqa: E402
+from test_gpu_parity import T, close, WG_RTOL, WG_ATOL  # noqa: E402,F401
+
+DIL_CASES = [
+    # N, Cin, Cout, H, W, kW, kH, dW, dH, padW, padH, dilW, dilH
+    (4, 16, 32, 28, 28, 3, 3, 1, 1, 2, 2, 2, 2),     # "same" dilated 3x3, fast kernels, stride-1 gradInput
+    (3, 8, 24, 21, 25, 3, 3, 1, 1, 0, 0, 3, 2),      # no padding, dilated, K % 16 != 0 -> generic forward
+    (2, 16, 16, 30, 30, 3, 3, 2, 2, 1, 1, 2, 2),     # stride 2: gradient columns + col2im
+    (2, 5, 7, 19, 23, 2, 4, 1, 2, 1, 3, 4, 1),       # rectangular everything
+    (2, 32, 8, 16, 16, 1, 1, 1, 1, 0, 0, 5, 5),      # 1x1: dilation without effect
+    (2, 16, 16, 20, 20, 3, 3, 1, 1, 5, 5, 2, 2),     # pad > dil*(k-1): gradInput cannot use the forward kernel
+    (5, 16, 8, 40, 44, 5, 5, 1, 1, 4, 4, 2, 2),      # L % 16 != 0 in the weight-gradient kernel
+]
+
+
+def _dil_run(T, case, bias=True, xt=None, scale=1.0, seed=80, single=False):
+    N, Cin, Cout, H, W, kW, kH, dW, dH, pW, pH, dlW, dlH = case
+    THNN, CT = T.THNN, T.CudaTensor
+    rng = np.random.default_rng(seed)
+    K = Cin * kH * kW
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, kH, kW)) * np.sqrt(2.0 / K)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32) if bias else None
+    args = (kW, kH, dW, dH, pW, pH, dlW, dlH)
+    xin = x[0] if single else x
+    tx = xt(xin) if xt else CT.from_numpy(xin)
+    tw, tb = CT.from_numpy(w), (CT.from_numpy(b) if bias else None)
+    out, cols, ones = CT(), CT(), CT()
+    THNN.SpatialDilatedConvolution_updateOutput(tx, out, tw, tb, cols, ones, *args)
+    ry = O.dilconv_updateOutput(x, w, b, *args)
+    y = out.numpy()
+    assert y.shape == (ry[0].shape if single else ry.shape)
+    close(y, ry[0] if single else ry)
+    gy = rng.standard_normal(ry.shape).astype(np.float32)
+    tgy = CT.from_numpy(gy[0] if single else gy)
+    gi = CT()
+    THNN.SpatialDilatedConvolution_updateGradInput(tx, tgy, gi, tw, CT(), *args)
+    rgi = O.dilconv_updateGradInput(x.shape, gy, w, *args)
+    close(gi.numpy(), rgi[0] if single else rgi)
+    gw0 = rng.standard_normal(w.shape).astype(np.float32)
+    gb0 = rng.standard_normal(Cout).astype(np.float32)
+    tgw, tgb = CT.from_numpy(gw0), (CT.from_numpy(gb0) if bias else None)
+    THNN.SpatialDilatedConvolution_accGradParameters(tx, tgy, tgw, tgb, cols, ones, *args, scale)
+    rgw, rgb = O.dilconv_accGradParameters(x, gy, gw0.reshape(Cout, K).copy(), gb0.copy() if bias else None, *args,
+                                           scale=scale)
+    close(tgw.numpy().reshape(Cout, K), rgw, WG_RTOL, WG_ATOL * max(1.0, abs(scale)) * 4)
+    if bias:
+        close(tgb.numpy(), rgb, WG_RTOL, WG_ATOL * max(1.0, abs(scale)) * 4)
+
+
+@pytest.mark.parametrize("case", DIL_CASES)
+def test_dilated_convolution(T, case):
+    _dil_run(T, case)
+
+
+def test_dilated_convolution_variants(T):
+    rng = np.random.default_rng(81)
+    _dil_run(T, DIL_CASES[0], bias=False, scale=0.5)
+    _dil_run(T, DIL_CASES[3], xt=lambda a: T.CudaTensor.noncontiguous_from_numpy(a, rng), scale=2.0)
+    _dil_run(T, (1,) + DIL_CASES[1][1:], single=True)
+    os.environ["THCUNN_CONV_FORCE_GENERIC"] = "1"
+    try:
+        _dil_run(T, DIL_CASES[0])
+        _dil_run(T, DIL_CASES[2])
+    finally:
+        os.environ.pop("THCUNN_CONV_FORCE_GENERIC", None)
+
+
+def test_dilated_convolution_dilation_one_is_convmm(T):
+    """With dilation 1 the entry point gives bit-identical results to SpatialConvolutionMM."""
+    THNN, CT = T.THNN, T.CudaTensor
+    rng = np.random.default_rng(82)
+    x = rng.standard_normal((3, 16, 20, 24)).astype(np.float32)
+    w = (rng.standard_normal((8, 16, 3, 3)) * 0.1).astype(np.float32)
+    b = rng.standard_normal(8).astype(np.float32)
+    a, c = CT(), CT()
+    THNN.SpatialDilatedConvolution_updateOutput(CT.from_numpy(x), a, CT.from_numpy(w), CT.from_numpy(b), CT(), CT(),
+                                                3, 3, 1, 1, 1, 1, 1, 1)
+    THNN.SpatialConvolutionMM_updateOutput(CT.from_numpy(x), c, CT.from_numpy(w), CT.from_numpy(b), CT(), CT(),
+                                           3, 3, 1, 1, 1, 1)
+    assert np.array_equal(a.numpy(), c.numpy())
+
+
+def test_dilated_convolution_errors(T):
+    THNN, CT = T.THNN, T.CudaTensor
+    x = CT.from_numpy(np.zeros((1, 4, 8, 8), np.float32))
+    w2 = CT.from_numpy(np.zeros((4, 36), np.float32))
+    w4 = CT.from_numpy(np.zeros((4, 4, 3, 3), np.float32))
+    with pytest.raises(T.THError, match="4D weight tensor"):
+        THNN.SpatialDilatedConvolution_updateOutput(x, CT(), w2, None, CT(), CT(), 3, 3, 1, 1, 0, 0, 1, 1)
+    with pytest.raises(T.THError, match="dilation should be greater than 0"):
+        THNN.SpatialDilatedConvolution_updateOutput(x, CT(), w4, None, CT(), CT(), 3, 3, 1, 1, 0, 0, 0, 1)
+    with pytest.raises(T.THError, match="Output size is too small"):
+        THNN.SpatialDilatedConvolution_updateOutput(x, CT(), w4, None, CT(), CT(), 3, 3, 1, 1, 0, 0, 4, 4)
+
+
+FULL_CASES = [
+    # N, Cin, Cout, H, W, kW, kH, dW, dH, padW, padH, dilW, dilH, adjW, adjH
+    (4, 16, 32, 14, 14, 4, 4, 2, 2, 1, 1, 1, 1, 0, 0),    # the usual 2x upsampling deconvolution
+    (3, 32, 16, 12, 15, 3, 3, 2, 2, 1, 1, 1, 1, 1, 1),    # output padding
+    (2, 16, 16, 20, 20, 3, 3, 1, 1, 1, 1, 1, 1, 0, 0),    # stride 1: forward through the flipped-weight kernel
+    (2, 5, 7, 9, 11, 3, 2, 3, 2, 1, 0, 2, 2, 2, 1),       # rectangular, dilated, adj < stride
+    (2, 8, 4, 10, 10, 5, 5, 1, 1, 0, 0, 2, 2, 0, 0),      # stride 1, dilated, no padding
+    (2, 6, 10, 8, 8, 2, 2, 2, 2, 0, 0, 1, 1, 0, 0),       # k = stride: non-overlapping
+]
+
+
+def _full_run(T, case, bias=True, xt=None, scale=1.0, seed=90, dilated_entry=True, single=False):
+    N, Cin, Cout, H, W, kW, kH, dW, dH, pW, pH, dlW, dlH, aW, aH = case
+    THNN, CT = T.THNN, T.CudaTensor
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cin, Cout, kH, kW)) * np.sqrt(2.0 / (Cin * kH * kW))).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32) if bias else None
+    oargs = (kW, kH, dW, dH, pW, pH, dlW, dlH, aW, aH)
+    if dilated_entry:
+        fo, fg, fa = (THNN.SpatialFullDilatedConvolution_updateOutput, THNN.SpatialFullDilatedConvolution_updateGradInput,
+                      THNN.SpatialFullDilatedConvolution_accGradParameters)
+        args = oargs
+    else:
+        assert dlW == 1 and dlH == 1
+        fo, fg, fa = (THNN.SpatialFullConvolution_updateOutput, THNN.SpatialFullConvolution_updateGradInput,
+                      THNN.SpatialFullConvolution_accGradParameters)
+        args = (kW, kH, dW, dH, pW, pH, aW, aH)
+    xin = x[0] if single else x
+    tx = xt(xin) if xt else CT.from_numpy(xin)
+    tw, tb = CT.from_numpy(w), (CT.from_numpy(b) if bias else None)
+    out, cols, ones = CT(), CT(), CT()
+    fo(tx, out, tw, tb, cols, ones, *args)
+    ry = O.fullconv_updateOutput(x, w, b, *oargs)
+    y = out.numpy()
+    assert y.shape == (ry[0].shape if single else ry.shape)
+    close(y, ry[0] if single else ry)
+    gy = rng.standard_normal(ry.shape).astype(np.float32)
+    tgy = CT.from_numpy(gy[0] if single else gy)
+    gi = CT()
+    fg(tx, tgy, gi, tw, CT(), *args)
+    rgi = O.fullconv_updateGradInput(x.shape, gy, w, *oargs)
+    close(gi.numpy(), rgi[0] if single else rgi)
+    gw0 = rng.standard_normal(w.shape).astype(np.float32)
+    gb0 = rng.standard_normal(Cout).astype(np.float32)
+    tgw, tgb = CT.from_numpy(gw0), (CT.from_numpy(gb0) if bias else None)
+    fa(tx, tgy, tgw, tgb, cols, ones, *args, scale)
+    rgw, rgb = O.fullconv_accGradParameters(x, gy, gw0.copy(), gb0.copy() if bias else None, *oargs, scale=scale)
+    close(tgw.numpy(), rgw, WG_RTOL, WG_ATOL * max(1.0, abs(scale)) * 4)
+    if bias:
+        close(tgb.numpy(), rgb, WG_RTOL, WG_ATOL * max(1.0, abs(scale)) * 4)
+
+
+@pytest.mark.parametrize("case", FULL_CASES)
+def test_full_convolution(T, case):
+    _full_run(T, case)
+
+
+def test_full_convolution_variants(T):
+    rng = np.random.default_rng(91)
+    _full_run(T, FULL_CASES[0], bias=False, scale=0.5, dilated_entry=False)
+    _full_run(T, FULL_CASES[1], dilated_entry=False, xt=lambda a: T.CudaTensor.noncontiguous_from_numpy(a, rng), scale=2.0)
+    _full_run(T, (1,) + FULL_CASES[2][1:], single=True, dilated_entry=False)
+    os.environ["THCUNN_CONV_FORCE_GENERIC"] = "1"
+    try:
+        _full_run(T, FULL_CASES[0])
+        _full_run(T, FULL_CASES[2])
+    finally:
+        os.environ.pop("THCUNN_CONV_FORCE_GENERIC", None)
+
+
+def test_full_convolution_errors(T):
+    THNN, CT = T.THNN, T.CudaTensor
+    x = CT.from_numpy(np.zeros((1, 4, 8, 8), np.float32))
+    w = CT.from_numpy(np.zeros((4, 6, 3, 3), np.float32))
+    with pytest.raises(T.THError, match="output padding must be smaller than either stride or dilation"):
+        THNN.SpatialFullConvolution_updateOutput(x, CT(), w, None, CT(), CT(), 3, 3, 2, 2, 0, 0, 2, 0)
+    with pytest.raises(T.THError, match="bias"):
+        THNN.SpatialFullConvolution_updateOutput(x, CT(), w, CT.from_numpy(np.zeros(4, np.float32)), CT(), CT(),
+                                                 3, 3, 1, 1, 0, 0, 0, 0)

@@ -170,6 +170,87 @@ def test_convmm_vs_torch_autograd():
     close(gb, gb0 + 2.0 * tb.grad.numpy(), 1e-3, 1e-3)
 
 
+# ------------------------------------------------ dilated / transposed conv --
+DIL_CASES = [
+    # N, Cin, Cout, H, W, kW, kH, dW, dH, padW, padH, dilW, dilH
+    (2, 3, 4, 13, 15, 3, 3, 1, 1, 2, 2, 2, 2),
+    (2, 2, 5, 17, 14, 3, 2, 2, 1, 1, 0, 3, 2),
+    (1, 4, 3, 11, 11, 2, 3, 1, 2, 0, 3, 1, 3),
+]
+
+
+@pytest.mark.parametrize("case", DIL_CASES)
+def test_dilconv_vs_torch_autograd_and_adjoint(case):
+    """SpatialDilatedConvolution restated: float64 torch conv2d(dilation=) + autograd fixes the
+    values; dilation 1 reduces to SpatialConvolutionMM; <conv(x),gy> = <x,gradInput> = <W,gradW>."""
+    N, Cin, Cout, H, W, kW, kH, dW, dH, pW, pH, dlW, dlH = case
+    rng = np.random.default_rng(70)
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, kH, kW)) * 0.3).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    tx = torch.from_numpy(x).double().requires_grad_()
+    tw = torch.from_numpy(w).double().requires_grad_()
+    tb = torch.from_numpy(b).double().requires_grad_()
+    ty = F.conv2d(tx, tw, tb, stride=(dH, dW), padding=(pH, pW), dilation=(dlH, dlW))
+    y = O.dilconv_updateOutput(x, w, b, kW, kH, dW, dH, pW, pH, dlW, dlH)
+    close(y, ty.detach().numpy())
+    gy = rng.standard_normal(y.shape).astype(np.float32)
+    ty.backward(torch.from_numpy(gy).double())
+    gx = O.dilconv_updateGradInput(x.shape, gy, w, kW, kH, dW, dH, pW, pH, dlW, dlH)
+    close(gx, tx.grad.numpy())
+    gw0 = rng.standard_normal((Cout, Cin * kH * kW)).astype(np.float32)
+    gb0 = rng.standard_normal(Cout).astype(np.float32)
+    gw, gb = O.dilconv_accGradParameters(x, gy, gw0.copy(), gb0.copy(), kW, kH, dW, dH, pW, pH, dlW, dlH, scale=0.5)
+    close(gw, gw0 + 0.5 * tw.grad.numpy().reshape(Cout, -1), 1e-3, 1e-3)
+    close(gb, gb0 + 0.5 * tb.grad.numpy(), 1e-3, 1e-3)
+    y1 = O.dilconv_updateOutput(x, w, b, kW, kH, dW, dH, pW, pH, 1, 1)
+    assert np.array_equal(y1, O.convmm_updateOutput(x, w, b, kW, kH, dW, dH, pW, pH))
+
+
+FULL_CASES = [
+    # N, Cin, Cout, H, W, kW, kH, dW, dH, padW, padH, dilW, dilH, adjW, adjH
+    (2, 3, 4, 7, 9, 3, 3, 2, 2, 1, 1, 1, 1, 1, 1),
+    (2, 4, 2, 6, 5, 4, 3, 1, 1, 0, 1, 1, 1, 0, 0),
+    (1, 2, 3, 5, 6, 3, 2, 3, 2, 1, 0, 2, 2, 2, 1),
+    (2, 2, 2, 4, 4, 2, 2, 2, 2, 0, 0, 1, 1, 0, 0),
+]
+
+
+@pytest.mark.parametrize("case", FULL_CASES)
+def test_fullconv_vs_torch_and_transpose_identity(case):
+    """SpatialFull(Dilated)Convolution restated: float64 conv_transpose2d + autograd fixes the
+    values; the forward pass is the adjoint of the ordinary convolution with the same weight
+    read as (Cout_conv = Cin, Cin_conv = Cout): <full(x), z> = <x, conv(z)>."""
+    N, Cin, Cout, H, W, kW, kH, dW, dH, pW, pH, dlW, dlH, aW, aH = case
+    rng = np.random.default_rng(71)
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cin, Cout, kH, kW)) * 0.3).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    tx = torch.from_numpy(x).double().requires_grad_()
+    tw = torch.from_numpy(w).double().requires_grad_()
+    tb = torch.from_numpy(b).double().requires_grad_()
+    ty = F.conv_transpose2d(tx, tw, tb, stride=(dH, dW), padding=(pH, pW), output_padding=(aH, aW),
+                            dilation=(dlH, dlW))
+    y = O.fullconv_updateOutput(x, w, b, kW, kH, dW, dH, pW, pH, dlW, dlH, aW, aH)
+    assert y.shape == tuple(ty.shape)
+    close(y, ty.detach().numpy())
+    gy = rng.standard_normal(y.shape).astype(np.float32)
+    ty.backward(torch.from_numpy(gy).double())
+    gx = O.fullconv_updateGradInput(x.shape, gy, w, kW, kH, dW, dH, pW, pH, dlW, dlH, aW, aH)
+    close(gx, tx.grad.numpy())
+    gw0 = rng.standard_normal(w.shape).astype(np.float32)
+    gb0 = rng.standard_normal(Cout).astype(np.float32)
+    gw, gb = O.fullconv_accGradParameters(x, gy, gw0.copy(), gb0.copy(), kW, kH, dW, dH, pW, pH, dlW, dlH, aW, aH,
+                                          scale=1.5)
+    close(gw, gw0 + 1.5 * tw.grad.numpy(), 1e-3, 1e-3)
+    close(gb, gb0 + 1.5 * tb.grad.numpy(), 1e-3, 1e-3)
+    # adjoint of the ordinary (dilated) convolution over the output-sized image
+    z = rng.standard_normal(y.shape).astype(np.float32)
+    cz = O.dilconv_updateOutput(z, w.reshape(Cin, Cout * kH * kW), None, kW, kH, dW, dH, pW, pH, dlW, dlH)
+    y0 = O.fullconv_updateOutput(x, w, None, kW, kH, dW, dH, pW, pH, dlW, dlH, aW, aH)
+    close(np.vdot(y0.astype(np.float64), z), np.vdot(x.astype(np.float64), cz[:, :, :H, :W]), 1e-4, 1e-3)
+
+
 # ------------------------------------------------------------------------- BN --
 @pytest.mark.parametrize("affine", [True, False])
 @pytest.mark.parametrize("shape", [(4, 3, 5, 7), (2, 5, 1, 1), (8, 2, 6)])

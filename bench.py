@@ -295,6 +295,101 @@ def wl_conv(nsets):
                 desc=f"SpatialConvolutionMM fwd+gradInput+accGradParameters fp32 N={N} Cin={Ci} Cout={Co} {H}x{H} k3 s1 p1 bias")
 
 
+def wl_dilconv(nsets):
+    """Beyond the five configurations: SpatialDilatedConvolution at the cfg5 shape with dilation 2 ("same" padding 2)."""
+    from cunn_amd import CudaTensor as CT, THNN
+    from oracle import oracle as O
+    N, Ci, Co, H, k, dil = 64, 256, 256, 28, 3, 2
+    K = Ci * k * k
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((N, Ci, H, H)).astype(np.float32)
+    gy = rng.standard_normal((N, Co, H, H)).astype(np.float32)
+    w = (rng.standard_normal((Co, Ci, k, k)) * np.sqrt(2.0 / K)).astype(np.float32)
+    b = rng.uniform(-0.02, 0.02, Co).astype(np.float32)
+    sets = [dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), gx=CT(), w=CT.from_numpy(w), b=CT.from_numpy(b),
+                 gw=CT.from_numpy(np.zeros_like(w)), gb=CT.from_numpy(np.zeros_like(b)), cols=CT(), gcols=CT(), ones=CT())
+            for _ in range(nsets)]
+    g = (k, k, 1, 1, dil, dil, dil, dil)
+
+    def calls(i):
+        t = sets[i]
+        return [("dilconv_updateOutput", lambda: THNN.SpatialDilatedConvolution_updateOutput(t["x"], t["y"], t["w"], t["b"], t["cols"], t["ones"], *g)),
+                ("dilconv_updateGradInput", lambda: THNN.SpatialDilatedConvolution_updateGradInput(t["x"], t["gy"], t["gx"], t["w"], t["gcols"], *g)),
+                ("dilconv_accGradParameters", lambda: THNN.SpatialDilatedConvolution_accGradParameters(t["x"], t["gy"], t["gw"], t["gb"], t["cols"], t["ones"], *g, 1.0))]
+
+    fl = 2.0 * Co * K * H * H * N
+    work = {"dilconv_updateOutput": (fl, "flops"), "dilconv_updateGradInput": (fl, "flops"), "dilconv_accGradParameters": (fl, "flops")}
+    ns = 4
+
+    def cpu(reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            O.dilconv_updateOutput(x[:ns], w, b, *g)
+            O.dilconv_updateGradInput((ns,) + x.shape[1:], gy[:ns], w, *g)
+            O.dilconv_accGradParameters(x[:ns], gy[:ns], np.zeros((Co, K), np.float32), np.zeros_like(b), *g, 1.0)
+        return time.perf_counter() - t0, reps * ns, f"{reps} passes over the first {ns} of {N} images"
+
+    def verify():
+        t = sets[0]
+        for _, fn in calls(0):
+            fn()
+        m = 2
+        np.testing.assert_allclose(t["y"].numpy()[:m], O.dilconv_updateOutput(x[:m], w, b, *g), rtol=1e-5, atol=1e-4)
+        np.testing.assert_allclose(t["gx"].numpy()[:m], O.dilconv_updateGradInput((m,) + x.shape[1:], gy[:m], w, *g), rtol=1e-5, atol=1e-4)
+        t["gw"].fill(0.0), t["gb"].fill(0.0)
+
+    return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="mfma",
+                desc=f"SpatialDilatedConvolution fwd+gradInput+accGradParameters fp32 N={N} Cin={Ci} Cout={Co} {H}x{H} k3 s1 p2 dilation 2 bias")
+
+
+def wl_fullconv(nsets):
+    """Beyond the five configurations: SpatialFullConvolution, the 2x upsampling transposed convolution of a decoder."""
+    from cunn_amd import CudaTensor as CT, THNN
+    from oracle import oracle as O
+    N, Ci, Co, H, k = 64, 256, 128, 14, 4
+    rng = np.random.default_rng(6)
+    oH = (H - 1) * 2 - 2 + k
+    x = rng.standard_normal((N, Ci, H, H)).astype(np.float32)
+    gy = rng.standard_normal((N, Co, oH, oH)).astype(np.float32)
+    w = (rng.standard_normal((Ci, Co, k, k)) * np.sqrt(2.0 / (Ci * k * k))).astype(np.float32)
+    b = rng.uniform(-0.02, 0.02, Co).astype(np.float32)
+    sets = [dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), gx=CT(), w=CT.from_numpy(w), b=CT.from_numpy(b),
+                 gw=CT.from_numpy(np.zeros_like(w)), gb=CT.from_numpy(np.zeros_like(b)), cols=CT(), gcols=CT(), ones=CT())
+            for _ in range(nsets)]
+    g = (k, k, 2, 2, 1, 1, 0, 0)
+    og = (k, k, 2, 2, 1, 1, 1, 1, 0, 0)
+
+    def calls(i):
+        t = sets[i]
+        return [("fullconv_updateOutput", lambda: THNN.SpatialFullConvolution_updateOutput(t["x"], t["y"], t["w"], t["b"], t["cols"], t["ones"], *g)),
+                ("fullconv_updateGradInput", lambda: THNN.SpatialFullConvolution_updateGradInput(t["x"], t["gy"], t["gx"], t["w"], t["gcols"], *g)),
+                ("fullconv_accGradParameters", lambda: THNN.SpatialFullConvolution_accGradParameters(t["x"], t["gy"], t["gw"], t["gb"], t["cols"], t["ones"], *g, 1.0))]
+
+    fl = 2.0 * Ci * Co * k * k * H * H * N   # every input pixel meets every tap of every (Cin, Cout) pair once
+    work = {"fullconv_updateOutput": (fl, "flops"), "fullconv_updateGradInput": (fl, "flops"), "fullconv_accGradParameters": (fl, "flops")}
+    ns = 4
+
+    def cpu(reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            O.fullconv_updateOutput(x[:ns], w, b, *og)
+            O.fullconv_updateGradInput((ns,) + x.shape[1:], gy[:ns], w, *og)
+            O.fullconv_accGradParameters(x[:ns], gy[:ns], np.zeros_like(w), np.zeros_like(b), *og, scale=1.0)
+        return time.perf_counter() - t0, reps * ns, f"{reps} passes over the first {ns} of {N} images"
+
+    def verify():
+        t = sets[0]
+        for _, fn in calls(0):
+            fn()
+        m = 2
+        np.testing.assert_allclose(t["y"].numpy()[:m], O.fullconv_updateOutput(x[:m], w, b, *og), rtol=1e-5, atol=1e-4)
+        np.testing.assert_allclose(t["gx"].numpy()[:m], O.fullconv_updateGradInput((m,) + x.shape[1:], gy[:m], w, *og), rtol=1e-5, atol=1e-4)
+        t["gw"].fill(0.0), t["gb"].fill(0.0)
+
+    return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="mfma",
+                desc=f"SpatialFullConvolution fwd+gradInput+accGradParameters fp32 N={N} Cin={Ci} Cout={Co} {H}x{H}->{oH}x{oH} k4 s2 p1 bias")
+
+
 def wl_copy(nsets):
     """Calibration: plain device-to-device copy of 128 MB (2 x 128 MB of HBM traffic per launch)."""
     from cunn_amd import CudaTensor as CT
@@ -315,7 +410,7 @@ def wl_copy(nsets):
 
 
 WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda n: wl_dw("cfg2", n), "cfg3": wl_bn, "cfg4": wl_pool,
-             "cfg5": wl_conv}
+             "cfg5": wl_conv, "dilconv": wl_dilconv, "fullconv": wl_fullconv}
 
 
 def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds):

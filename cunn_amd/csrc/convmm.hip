@@ -944,11 +944,15 @@ gradBiasKernel(const float *__restrict__ gy, float *__restrict__ gradBias, int N
   }
 }
 
-// t[n][c][:] += bias[c] over a (N, C, plane) tensor
+// wt[k][o] = w[o][k] for w (rows x cols)
 __global__ void __launch_bounds__(dev::kBlock)
-addPlaneBiasKernel(float *__restrict__ t, const float *__restrict__ bias, long total, int plane, int C) {
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x)
-    t[i] += bias[(int)((i / plane) % C)];
+transposeKernel(const float *__restrict__ w, float *__restrict__ wt, int rows, int cols) {
+  const long total = (long)rows * cols;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const int o = (int)(i % rows);
+    const long k = i / rows;
+    wt[i] = w[(long)o * cols + k];
+  }
 }
 
 // Wf[c][(o, kh', kw')] = W[o][(c, kH-1-kh', kW-1-kw')]: with these weights the
@@ -994,7 +998,7 @@ im2colKernel(const float *__restrict__ im, float *__restrict__ col, int nImg, in
 // (lib/THCUNN/im2col.h:63-102); float accumulation in the reference's order.
 __global__ void __launch_bounds__(dev::kBlock)
 col2imKernel(const float *__restrict__ col, float *__restrict__ im, int nImg, int C, int H, int W, int kH, int kW,
-             int padH, int padW, int dH, int dW, int dilH, int dilW, int oH, int oW) {
+             int padH, int padW, int dH, int dW, int dilH, int dilW, int oH, int oW, const float *__restrict__ bias) {
   const long total = (long)nImg * C * H * W;
   const int extW = (kW - 1) * dilW + 1, extH = (kH - 1) * dilH + 1;
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
@@ -1005,7 +1009,7 @@ col2imKernel(const float *__restrict__ col, float *__restrict__ im, int nImg, in
     int we = min(w_im / dW + 1, oW);
     int hs = (h_im < extH) ? 0 : (h_im - extH) / dH + 1;
     int he = min(h_im / dH + 1, oH);
-    float val = 0.f;
+    float val = bias ? bias[(int)(nc % C)] : 0.f;  // per-plane bias of the transposed convolution, else 0
     for (int hc = hs; hc < he; ++hc)
       for (int wc = ws; wc < we; ++wc) {
         int hk = h_im - hc * dH, wk = w_im - wc * dW;
@@ -1141,8 +1145,15 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
   pl.mTiles = (int)tiles(M, BM);
   pl.total = pl.mTiles * (int)tiles((long)nImages * g.L, BN);
   const int cus = residentSlots(nullptr);
-  pl.tail = pl.total % cus;
-  int nSplit = (pl.tail > 0 && pl.total > cus) ? std::min(nkt / 4, cus / pl.tail) : 1;  // >= 4 k-tiles per split
+  int nSplit = 1;
+  if (pl.total > cus) {
+    pl.tail = pl.total % cus;
+    if (pl.tail > 0) nSplit = std::min(nkt / 4, cus / pl.tail);  // >= 4 k-tiles per split
+  } else {
+    // fewer tiles than CUs: every tile is split along K so that the grid fills the resident slots
+    pl.tail = pl.total;
+    nSplit = std::min(nkt / 4, residentSlots((const void *)convFwdPaddedKernel) / pl.total);
+  }
   if (nSplit < 2) {
     pl.tail = 0;
     nSplit = 1;
@@ -1307,36 +1318,57 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
     }
     return;
   }
-  // gradient columns of a group of images at a time (<= 64 MB so the buffer stays cache resident)
+  // Gradient columns of a group of images at a time (<= 128 MB so the buffer stays cache resident), then
+  // the col2im gather. gradCol[n][k][l] = sum_o W[o][k] * gy[n][o][l] is itself a 1x1 convolution of gy
+  // with the transposed weights, so it runs on the forward kernels as well.
   const long perImg = (long)g.K * g.L;
-  int group = (int)std::max<long>(1, std::min<long>(g.N, (64L << 20) / 4 / perImg));
+  int group = (int)std::max<long>(1, std::min<long>(g.N, (128L << 20) / 4 / perImg));
   group = (int)std::min<long>(group, std::max<long>(1, 0x7fffffffL / 2 / g.L));
+  const long gyImgBytes = (long)g.Cout * g.L * sizeof(float);
+  const bool viaForward = !forceGeneric() && gyImgBytes < (1L << 30) && (long)g.Cout * g.K < 0x7fffffffL / 4;
+  if (viaForward) group = (int)std::min<long>(group, std::max<long>(1, ((1L << 31) - 1 - 4096) / gyImgBytes));
+  ConvGeom q{};  // the 1x1 convolution: (N, Cout, oH, oW) -> (N, K, oH, oW)
+  q.N = g.N, q.Cin = g.Cout, q.Cout = g.K, q.H = q.oH = g.oH, q.W = q.oW = g.oW;
+  q.kH = q.kW = q.dH = q.dW = q.dilH = q.dilW = 1;
+  q.K = g.Cout, q.L = g.L;
+  FwdPlan pl{};
+  long wtFloats = 0;
+  if (viaForward) {
+    pl = planFwdImplicit(q.Cout, std::min(group, g.N), q);
+    wtFloats = ((long)g.Cout * g.K + 3) / 4 * 4;
+  }
+  const long fwdFloats = (pl.scratchFloats + 3) / 4 * 4;
   Temp tmp;
-  float *gcol = scratchFloats(state, scratchBuf, (long)group * perImg, tmp, bufName);
+  float *buf = scratchFloats(state, scratchBuf, wtFloats + fwdFloats + (long)group * perImg, tmp, bufName);
+  float *gcol = buf + wtFloats + fwdFloats;
+  if (viaForward) {
+    transposeKernel<<<launch::directGrid((long)g.Cout * g.K, dev::kBlock), dev::kBlock, 0, s>>>(w, buf, g.Cout, g.K);
+    THC_HIP_CHECK(hipGetLastError());
+  }
   for (int n0 = 0; n0 < g.N; n0 += group) {
     int cnt = std::min(group, g.N - n0);
-    GemmArgs p{};
-    p.a = w;
-    p.b = gy;
-    p.c = gcol;
-    p.M = g.K;
-    p.Ncols = cnt * g.L;
-    p.R = g.Cout;
-    p.n0 = n0;
-    p.nImages = cnt;
-    p.mTiles = (int)tiles(p.M, BM);
-    dim3 grid(p.mTiles * tiles(p.Ncols, BN), 1);
-    convGemmKernel<kGradCol><<<grid, dev::kBlock, 0, s>>>(p, g);
-    THC_HIP_CHECK(hipGetLastError());
+    if (viaForward) {
+      if (cnt != std::min(group, g.N)) pl = planFwdImplicit(q.Cout, cnt, q);
+      launchFwdImplicit(s, pl, buf + wtFloats, buf, gy + (long)n0 * g.Cout * g.L, gcol, nullptr, q.Cout, cnt, q);
+    } else {
+      GemmArgs p{};
+      p.a = w;
+      p.b = gy;
+      p.c = gcol;
+      p.M = g.K;
+      p.Ncols = cnt * g.L;
+      p.R = g.Cout;
+      p.n0 = n0;
+      p.nImages = cnt;
+      p.mTiles = (int)tiles(p.M, BM);
+      dim3 grid(p.mTiles * tiles(p.Ncols, BN), 1);
+      convGemmKernel<kGradCol><<<grid, dev::kBlock, 0, s>>>(p, g);
+      THC_HIP_CHECK(hipGetLastError());
+    }
     long total = (long)cnt * g.Cin * g.H * g.W;
     col2imKernel<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(
         gcol, gi + (long)n0 * g.Cin * g.H * g.W, cnt, g.Cin, g.H, g.W, g.kH, g.kW, g.padH, g.padW, g.dH, g.dW, g.dilH,
-        g.dilW, g.oH, g.oW);
-    THC_HIP_CHECK(hipGetLastError());
-  }
-  if (bias) {
-    const long total = (long)g.N * g.Cin * g.H * g.W;
-    addPlaneBiasKernel<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(gi, bias, total, g.H * g.W, g.Cin);
+        g.dilW, g.oH, g.oW, bias);
     THC_HIP_CHECK(hipGetLastError());
   }
 }
@@ -1746,7 +1778,7 @@ void THNN_Cuda_col2im(THCState *state, const float *col, int nImages, int channe
   long total = (long)nImages * channels * height * width;
   if (total <= 0) return;
   col2imKernel<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, state->stream>>>(
-      col, im, nImages, channels, height, width, kH, kW, padH, padW, dH, dW, dilH, dilW, oH, oW);
+      col, im, nImages, channels, height, width, kH, kW, padH, padW, dH, dW, dilH, dilW, oH, oW, nullptr);
   THC_HIP_CHECK(hipGetLastError());
   THNN_LEAVE
 }

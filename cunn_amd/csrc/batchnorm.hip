@@ -425,8 +425,9 @@ __global__ void __launch_bounds__(kResBlock)
 bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
               float *__restrict__ gradWeight, float *__restrict__ gradBias, const float *__restrict__ weight,
               const float *__restrict__ meanSrc, const float *__restrict__ stdSrc, int N, int C, int L, float scale,
-              float eps) {
+              float eps, int xlds) {
   __shared__ float red[kResWaves];
+  extern __shared__ float4 xpark[];  // !KEEPX: the first xlds (a multiple of 4) float4 of x per lane wait here for the apply phase
   const int ch = blockIdx.x;
   const int total4 = N * (L >> 2);
   const float mean = meanSrc[ch];
@@ -435,6 +436,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
   const long span = ((long)(N - 1) * C * L + L) * 4;
   const __amdgpu_buffer_rsrc_t xr = dev::makeRsrc(x + (long)ch * L, span), gr = dev::makeRsrc(gy + (long)ch * L, span);
   const __amdgpu_buffer_rsrc_t or_ = dev::makeRsrc(gx ? gx + (long)ch * L : x, gx ? span : 0);
+  constexpr int XB = R > 8 ? 8 : 4;  // x float4 per lane requested together when x is not kept in registers
   float4 d[R], xc[KEEPX ? R : 1];
   float s0 = 0.f, s1 = 0.f;
   {
@@ -468,24 +470,29 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
         wk.next();
       }
 #pragma unroll
-      for (int u0 = 0; u0 < R; u0 += 4) {
-        float4 q[4];
+      for (int u0 = 0; u0 < R; u0 += XB) {
+        float4 q[XB];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
+        for (int k = 0; k < XB; ++k) {
           q[k] = make_float4(mean, mean, mean, mean);
           if (u0 + k < R) {
             if ((u0 + k) * kResBlock + (int)threadIdx.x < total4) q[k] = dev::bufLoad4(xr, wx.offset());
             wx.next();
           }
         }
+        if (u0 < xlds) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
+          for (int k = 0; k < XB; ++k)
+            if (u0 + k < R) xpark[(u0 + k) * kResBlock + threadIdx.x] = q[k];
+        }
+#pragma unroll
+        for (int k = 0; k < XB; ++k)
           if (u0 + k < R) {
             const float4 &g4 = d[u0 + k];
             s0 += (g4.x + g4.y) + (g4.z + g4.w);
             s1 += (g4.x * (q[k].x - mean) + g4.y * (q[k].y - mean)) + (g4.z * (q[k].z - mean) + g4.w * (q[k].w - mean));
           }
-        __asm__ volatile("" ::: "memory");  // keep the batches apart: 4 loads in flight, not R
+        __asm__ volatile("" ::: "memory");  // keep the batches apart: XB loads in flight, not R
       }
     }
   }
@@ -517,23 +524,23 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
       }
     } else {
 #pragma unroll
-      for (int u0 = 0; u0 < R; u0 += 4) {
-        float4 q[4];
-        int off[4];
+      for (int u0 = 0; u0 < R; u0 += XB) {
+        float4 q[XB];
+        int off[XB];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
+        for (int k = 0; k < XB; ++k) {
           off[k] = -1;
           q[k] = make_float4(mean, mean, mean, mean);
           if (u0 + k < R) {
             if ((u0 + k) * kResBlock + (int)threadIdx.x < total4) {
               off[k] = wk.offset();
-              q[k] = dev::bufLoad4(xr, off[k]);
+              q[k] = u0 < xlds ? xpark[(u0 + k) * kResBlock + threadIdx.x] : dev::bufLoad4(xr, off[k]);
             }
             wk.next();
           }
         }
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
+        for (int k = 0; k < XB; ++k)
           if (u0 + k < R && off[k] >= 0) {
             const float4 &g4 = d[u0 + k];
             float4 r;
@@ -736,14 +743,20 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
     float *gxp = gradInput_ ? data(gradInput_) : nullptr;
 #define BN_BWD_RES(RR)                                                                                             \
   if (R == RR) {                                                                                                   \
-    if (train)                                                                                                     \
-      bnBwdResident<RR, true, (RR <= 8)><<<g.C, kResBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),          \
+    /* x parked in LDS between the two phases: 8 of the up to 13 float4 per lane (128 KB of the CU's 160 KB) */   \
+    const int xlds = (RR > 8 && train && gxp) ? 8 : 0;                                                             \
+    const size_t lds = (size_t)xlds * kResBlock * sizeof(float4);                                                  \
+    if (train) {                                                                                                   \
+      if (lds) THC_HIP_CHECK(hipFuncSetAttribute((const void *)bnBwdResident<RR, true, (RR <= 8)>,                 \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));           \
+      bnBwdResident<RR, true, (RR <= 8)><<<g.C, kResBlock, lds, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_), \
                                                         dataOrNull(gradBias_), dataOrNull(weight_), meanSrc,       \
-                                                        stdSrc, g.N, g.C, g.L, (float)scale, (float)eps);          \
-    else                                                                                                           \
-      bnBwdResident<RR, false, (RR <= 8)><<<g.C, kResBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),         \
+                                                        stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, xlds);    \
+    } else {                                                                                                       \
+      bnBwdResident<RR, false, (RR <= 8)><<<g.C, kResBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_), \
                                                          dataOrNull(gradBias_), dataOrNull(weight_), meanSrc,      \
-                                                         stdSrc, g.N, g.C, g.L, (float)scale, (float)eps);         \
+                                                         stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, 0);      \
+    }                                                                                                              \
   }
     BN_BWD_RES(2) BN_BWD_RES(4) BN_BWD_RES(8) BN_BWD_RES(12) BN_BWD_RES(13)
 #undef BN_BWD_RES

@@ -410,7 +410,7 @@ bnFwdResident(const float *__restrict__ x, float *__restrict__ y, const float *_
       r.y = gamma * (v[u].y - mean) * invStd + beta;
       r.z = gamma * (v[u].z - mean) * invStd + beta;
       r.w = gamma * (v[u].w - mean) * invStd + beta;
-      dev::bufStore4(yr, wk.offset(), r);
+      dev::bufStoreStream4(yr, wk.offset(), r);
     }
     wk.next();
   }
@@ -518,7 +518,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
           } else {
             r.x = d[u].x * gradScale, r.y = d[u].y * gradScale, r.z = d[u].z * gradScale, r.w = d[u].w * gradScale;
           }
-          dev::bufStore4(or_, wk.offset(), r);
+          dev::bufStoreStream4(or_, wk.offset(), r);
         }
         wk.next();
       }
@@ -548,7 +548,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
             r.y = (g4.y - (q[k].y - mean) * projScale - gradMean) * gradScale;
             r.z = (g4.z - (q[k].z - mean) * projScale - gradMean) * gradScale;
             r.w = (g4.w - (q[k].w - mean) * projScale - gradMean) * gradScale;
-            dev::bufStore4(or_, off[k], r);
+            dev::bufStoreStream4(or_, off[k], r);
           }
         __asm__ volatile("" ::: "memory");
       }

@@ -71,6 +71,12 @@ __device__ __forceinline__ void bufStore4(__amdgpu_buffer_rsrc_t r, int byteOff,
   __builtin_amdgcn_raw_buffer_store_b128(v, r, byteOff, 0, 0);
 }
 
+// the same with the non-temporal hint (see storeStream4)
+__device__ __forceinline__ void bufStoreStream4(__amdgpu_buffer_rsrc_t r, int byteOff, float4 f) {
+  u32x4 v = {__float_as_uint(f.x), __float_as_uint(f.y), __float_as_uint(f.z), __float_as_uint(f.w)};
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, byteOff, 0, 2);
+}
+
 __device__ __forceinline__ int ceilDivPos(int a, int b) {  // ceil(a / b) for b > 0, any sign of a
   return (a >= 0) ? (a + b - 1) / b : -((-a) / b);
 }
@@ -82,6 +88,12 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void storeStream4(float *p, float4 v) {
   f32x4 q = {v.x, v.y, v.z, v.w};
   __builtin_nontemporal_store(q, reinterpret_cast<f32x4 *>(p));
+}
+
+typedef long i64x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void storeStream2(long *p, long a, long b) {
+  i64x2 q = {a, b};
+  __builtin_nontemporal_store(q, reinterpret_cast<i64x2 *>(p));
 }
 
 // Number of independent 16-byte (or 4-byte) global loads a lane keeps in flight

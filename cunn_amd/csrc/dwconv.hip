@@ -467,43 +467,45 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
   __syncthreads();
   const int W4 = g.W >> 2;
   const unsigned magicW4 = g.magicW4;
-  const int nA = (nRows + ST - 1) / ST;
-  const int total = nA * W4;
+  // A lane produces the 4 outputs i*4 .. i*4+3 of the band in memory order, so that a wave's store is one
+  // contiguous 1 KB run (full cache lines: what the streaming stores need to run at full rate). Its row
+  // h0 + hl = ST*a + dy picks, per staged gradOutput row qh, the kernel row kh = dy + PAD - qh*ST; dy is
+  // a run-time value, so those taps are selected into per-lane weights instead of being resolved at compile time.
+  const int total = nRows * W4;
   float *o = gradIn + ((long)plane * g.H + h0) * g.W;
 #pragma unroll 2
   for (int i = threadIdx.x; i < total; i += blockDim.x) {
-    const int a = dev::fastDiv(i, magicW4), b = i - a * W4;
-    float acc[ST][4];
-#pragma unroll
-    for (int dy = 0; dy < ST; ++dy)
-#pragma unroll
-      for (int dx = 0; dx < 4; ++dx) acc[dy][dx] = 0.f;
+    const int hl = dev::fastDiv(i, magicW4), b = i - hl * W4;
+    const int a = ST == 1 ? hl : hl >> (ST == 2 ? 1 : 0), dy = hl - a * ST;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int j = 0; j < nMul; ++j) {
       if (!M1) loadTaps<KS>(weight, ws, j, c, w);
       const float *gj = smem + (size_t)j * (stageRows * pitch + dev::kStripPadL) + dev::kStripPadL + QW0 + b * CPB;
 #pragma unroll
       for (int qh = QH0; qh <= QH1; ++qh) {
+        float wq[KS];
+#pragma unroll
+        for (int kw = 0; kw < KS; ++kw) {
+          wq[kw] = 0.f;
+#pragma unroll
+          for (int dyc = 0; dyc < ST; ++dyc) {
+            const int kh = dyc + PAD - qh * ST;
+            if (kh >= 0 && kh < KS) wq[kw] = (dy == dyc) ? w[kh * KS + kw] : wq[kw];
+          }
+        }
         float win[NW];
         dev::readWindow<0, NW, OFF, ALIGN>(gj + (a + qh - QH0) * pitch, win);
 #pragma unroll
-        for (int dy = 0; dy < ST; ++dy) {
-          const int kh = dy + PAD - qh * ST;
-          if (kh < 0 || kh >= KS) continue;
+        for (int dx = 0; dx < 4; ++dx)
 #pragma unroll
-          for (int dx = 0; dx < 4; ++dx)
-#pragma unroll
-            for (int kw = 0; kw < KS; ++kw) {
-              const int t = dx + PAD - kw;
-              if (t % ST != 0) continue;
-              acc[dy][dx] = fmaf(win[t / ST - QW0], w[kh * KS + kw], acc[dy][dx]);
-            }
-        }
+          for (int kw = 0; kw < KS; ++kw) {
+            const int t = dx + PAD - kw;
+            if (t % ST != 0) continue;
+            acc[dx] = fmaf(win[t / ST - QW0], wq[kw], acc[dx]);
+          }
       }
     }
-#pragma unroll
-    for (int dy = 0; dy < ST; ++dy)
-      if (a * ST + dy < nRows)
-        dev::storeStream4(o + (long)(a * ST + dy) * g.W + b * 4, make_float4(acc[dy][0], acc[dy][1], acc[dy][2], acc[dy][3]));
+    dev::storeStream4(o + (long)i * 4, make_float4(acc[0], acc[1], acc[2], acc[3]));
   }
 }
 

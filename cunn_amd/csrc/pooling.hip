@@ -348,12 +348,12 @@ maxPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, long *__r
           }
     }
     const long o = obase + (long)r * g.oW + b4 * 4;
-    *reinterpret_cast<float4 *>(out + o) = make_float4(mv[0], mv[1], mv[2], mv[3]);
+    dev::storeStream4(out + o, make_float4(mv[0], mv[1], mv[2], mv[3]));
     long2 i01, i23;
     i01.x = (long)mi[0] + TH_INDEX_BASE, i01.y = (long)mi[1] + TH_INDEX_BASE;
     i23.x = (long)mi[2] + TH_INDEX_BASE, i23.y = (long)mi[3] + TH_INDEX_BASE;
-    *reinterpret_cast<long2 *>(indices + o) = i01;
-    *reinterpret_cast<long2 *>(indices + o + 2) = i23;
+    dev::storeStream2(indices + o, i01.x, i01.y);
+    dev::storeStream2(indices + o + 2, i23.x, i23.y);
   }
 }
 
@@ -399,7 +399,7 @@ avgPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, PoolGeom 
         res[q] = acc[q] / avgDivisor<INCLUDE_PAD>(ph0 + r, b4 * 4 + q, g, hs, he, ws, we);
       }
     }
-    *reinterpret_cast<float4 *>(out + obase + (long)r * g.oW + b4 * 4) = make_float4(res[0], res[1], res[2], res[3]);
+    dev::storeStream4(out + obase + (long)r * g.oW + b4 * 4, make_float4(res[0], res[1], res[2], res[3]));
   }
 }
 
@@ -432,29 +432,23 @@ avgPoolFwdFlat(const float *__restrict__ in, float *__restrict__ out, int oW4, u
 #pragma unroll
       for (int q = 0; q < 4; ++q) acc[q] += row[q * KS + kw];
   }
-  reinterpret_cast<float4 *>(out)[i] = make_float4(acc[0] / (float)(KS * KS), acc[1] / (float)(KS * KS),
-                                                  acc[2] / (float)(KS * KS), acc[3] / (float)(KS * KS));
+  dev::storeStream4(out + (size_t)i * 4, make_float4(acc[0] / (float)(KS * KS), acc[1] / (float)(KS * KS),
+                                                    acc[2] / (float)(KS * KS), acc[3] / (float)(KS * KS)));
 }
 
+// total = gradInput float4s; a lane writes float4 i of gradInput (memory order: a wave's store is one
+// contiguous run) from the up to 4 gradOutput values above it.
 template <int KS>
 __global__ void __launch_bounds__(dev::kBlock)
-avgPoolBwdFlat(const float *__restrict__ gradOut, float *__restrict__ gradIn, int oW4, unsigned magicOw4, int W, unsigned total) {
+avgPoolBwdFlat(const float *__restrict__ gradOut, float *__restrict__ gradIn, int W4, unsigned magicW4, int oW, unsigned total) {
   const unsigned i = blockIdx.x * dev::kBlock + threadIdx.x;
   if (i >= total) return;
-  const unsigned R = dev::fastDiv((int)i, magicOw4), b = i - R * oW4;
-  const float4 g4 = reinterpret_cast<const float4 *>(gradOut)[i];
-  const float gq[4] = {g4.x / (float)(KS * KS), g4.y / (float)(KS * KS), g4.z / (float)(KS * KS), g4.w / (float)(KS * KS)};
-  float row[4 * KS];
+  const unsigned R = dev::fastDiv((int)i, magicW4), b = i - R * W4;  // row of the tall gradInput image, float4 within it
+  const float *gp = gradOut + (size_t)(R / KS) * oW;
+  float v[4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
-#pragma unroll
-    for (int kw = 0; kw < KS; ++kw) row[q * KS + kw] = gq[q];
-  float4 *p = reinterpret_cast<float4 *>(gradIn + (size_t)R * KS * W) + b * KS;
-  const int W4 = W >> 2;
-#pragma unroll
-  for (int kh = 0; kh < KS; ++kh)
-#pragma unroll
-    for (int k = 0; k < KS; ++k) p[kh * W4 + k] = make_float4(row[4 * k], row[4 * k + 1], row[4 * k + 2], row[4 * k + 3]);
+  for (int q = 0; q < 4; ++q) v[q] = gp[(b * 4 + q) / KS] / (float)(KS * KS);
+  dev::storeStream4(gradIn + (size_t)i * 4, make_float4(v[0], v[1], v[2], v[3]));
 }
 
 // Backward gathers. MAX: gradOutput and the argmax (narrowed to int32, base
@@ -513,46 +507,43 @@ poolBwdStrip(const float *__restrict__ gradOut, const long *__restrict__ indices
   __syncthreads();
   const int W4 = g.W >> 2;
   const unsigned magicW4 = dev::magicOf(W4);
-  const int nA = (nRows + ST - 1) / ST;
-  const int total = nA * W4;
+  // A lane produces the 4 elements i*4 .. i*4+3 of the band in memory order (a wave's store is one
+  // contiguous 1 KB run). Its row h0 + hl = ST*a + dy is covered by staged window row qh iff
+  // kh = dy + PAD - qh*ST lies inside the window; dy is a run-time value. For max pooling the argmax
+  // test alone decides (a window that does not cover the element cannot point at it).
+  const int total = nRows * W4;
   float *o = gradIn + ((long)plane * g.H + h0) * g.W;
   for (int i = threadIdx.x; i < total; i += blockDim.x) {
-    const int a = dev::fastDiv(i, magicW4), b = i - a * W4;
-    float acc[ST][4];
-#pragma unroll
-    for (int dy = 0; dy < ST; ++dy)
-#pragma unroll
-      for (int dx = 0; dx < 4; ++dx) acc[dy][dx] = 0.f;
-    const int me0 = (h0 + a * ST) * g.W + b * 4;  // flat index of patch element (0, 0)
+    const int hl = dev::fastDiv(i, magicW4), b = i - hl * W4;
+    const int a = ST == 1 ? hl : hl / ST, dy = hl - a * ST;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    const int me0 = (h0 + hl) * g.W + b * 4;  // flat index of element 0
     const int woff = dev::kStripPadL + QW0 + b * CPB;
 #pragma unroll
     for (int qh = QH0; qh <= QH1; ++qh) {
       float gw[NW], iw[NW];
       dev::readWindow<0, NW, OFF, ALIGN>(gs + (a + qh - QH0) * pitch + woff, gw);
       if (MAX) dev::readWindow<0, NW, OFF, ALIGN>(is + (a + qh - QH0) * pitch + woff, iw);
+      bool covers = false;
 #pragma unroll
-      for (int dy = 0; dy < ST; ++dy) {
-        const int kh = dy + PAD - qh * ST;
-        if (kh < 0 || kh >= KS) continue;
-#pragma unroll
-        for (int dx = 0; dx < 4; ++dx)
-#pragma unroll
-          for (int kw = KS - 1; kw >= 0; --kw) {  // descending kw = ascending window column
-            const int t = dx + PAD - kw;
-            if (t % ST != 0) continue;
-            if (MAX) {
-              if (__float_as_int(iw[t / ST - QW0]) == me0 + dy * g.W + dx) acc[dy][dx] += gw[t / ST - QW0];
-            } else {
-              acc[dy][dx] += gw[t / ST - QW0];
-            }
-          }
+      for (int dyc = 0; dyc < ST; ++dyc) {
+        const int kh = dyc + PAD - qh * ST;
+        if (kh >= 0 && kh < KS) covers = covers || dy == dyc;
       }
-    }
 #pragma unroll
-    for (int dy = 0; dy < ST; ++dy)
-      if (a * ST + dy < nRows)
-        *reinterpret_cast<float4 *>(o + (long)(a * ST + dy) * g.W + b * 4) =
-            make_float4(acc[dy][0], acc[dy][1], acc[dy][2], acc[dy][3]);
+      for (int dx = 0; dx < 4; ++dx)
+#pragma unroll
+        for (int kw = KS - 1; kw >= 0; --kw) {  // descending kw = ascending window column
+          const int t = dx + PAD - kw;
+          if (t % ST != 0) continue;
+          if (MAX) {
+            if (__float_as_int(iw[t / ST - QW0]) == me0 + dx) acc[dx] += gw[t / ST - QW0];
+          } else {
+            acc[dx] += covers ? gw[t / ST - QW0] : 0.f;
+          }
+        }
+    }
+    dev::storeStream4(o + (long)i * 4, make_float4(acc[0], acc[1], acc[2], acc[3]));
   }
 }
 
@@ -951,13 +942,13 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
   const int spitch = g.oW + dev::kStripPadL;
   auto sbytes = [&](int units) { return ((size_t)(units + extra) * spitch + dev::kStripPadL) * sizeof(float); };
   int units = 0;
-  if (avgFlatOk(g, planes) && vec && aligned16(data(gradInput))) {
-    const unsigned total = (unsigned)(planes * g.oH * (g.oW / 4));
+  if (avgFlatOk(g, planes) && vec && aligned16(data(gradInput)) && planes * g.H * (g.W / 4) * (g.W / 4) < 0xffffffffL) {
+    const unsigned total = (unsigned)(planes * g.H * (g.W / 4));
     const unsigned grid = (total + dev::kBlock - 1) / dev::kBlock;
-    const unsigned magic = dev::magicOf(g.oW / 4);
-    if (g.kH == 2) avgPoolBwdFlat<2><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.oW / 4, magic, g.W, total);
-    if (g.kH == 3) avgPoolBwdFlat<3><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.oW / 4, magic, g.W, total);
-    if (g.kH == 4) avgPoolBwdFlat<4><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.oW / 4, magic, g.W, total);
+    const unsigned magic = dev::magicOf(g.W / 4);
+    if (g.kH == 2) avgPoolBwdFlat<2><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.W / 4, magic, g.oW, total);
+    if (g.kH == 3) avgPoolBwdFlat<3><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.W / 4, magic, g.oW, total);
+    if (g.kH == 4) avgPoolBwdFlat<4><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.W / 4, magic, g.oW, total);
   } else if (stripBwdOk(g) && vec && aligned16(data(gradInput)) &&
       launch::pickBand(launch::ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
     g.tileRows = units * g.dH;

@@ -42,9 +42,9 @@ METRIC = "DW-conv fwd+bwd images/s + achieved HBM GB/s (% of peak), 1 MI355X"
 # factors); workloads without a counter run report null.
 _KIB = 1024
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg2", "dw_updateOutput"): int((50229.8 * 2.0 + 25088.0) * _KIB),
-    ("cfg2", "dw_updateGradInput"): int((12838.7 * 2.0 + 100361.2) * _KIB),
-    ("cfg2", "dw_accGradParameters"): int(((63014.7 + 189.0) * 2.0 + 321.0 + 12.0) * _KIB),
+    ("cfg2", "dw_updateOutput"): int((50220.6 * 2.0 + 25154.3) * _KIB),
+    ("cfg2", "dw_updateGradInput"): int((12841.8 * 2.0 + 100368.2) * _KIB),
+    ("cfg2", "dw_accGradParameters"): int(((63014.8 + 197.5) * 2.0 + 320.8 + 16.0) * _KIB),
 }
 
 

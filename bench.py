@@ -390,6 +390,41 @@ def wl_fullconv(nsets):
                 desc=f"SpatialFullConvolution fwd+gradInput+accGradParameters fp32 N={N} Cin={Ci} Cout={Co} {H}x{H}->{oH}x{oH} k4 s2 p1 bias")
 
 
+def wl_relu(nsets):
+    """Beyond the five configurations: Threshold (ReLU) forward + backward on the cfg2 activation tensor."""
+    from cunn_amd import CudaTensor as CT, THNN
+    from oracle import oracle as O
+    shape = (64, 128, 56, 56)
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal(shape).astype(np.float32)
+    gy = rng.standard_normal(shape).astype(np.float32)
+    sets = [dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), gx=CT()) for _ in range(nsets)]
+
+    def calls(i):
+        t = sets[i]
+        return [("threshold_updateOutput", lambda: THNN.Threshold_updateOutput(t["x"], t["y"], 0.0, 0.0, False)),
+                ("threshold_updateGradInput", lambda: THNN.Threshold_updateGradInput(t["x"], t["gy"], t["gx"], 0.0, 0.0, False))]
+
+    work = {"threshold_updateOutput": (2 * x.nbytes, "bytes"), "threshold_updateGradInput": (3 * x.nbytes, "bytes")}
+
+    def cpu(reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            O.threshold_updateOutput(x, 0.0, 0.0)
+            O.threshold_updateGradInput(x, gy, 0.0)
+        return time.perf_counter() - t0, reps * shape[0], f"{reps} full passes ({shape[0]} images each), numpy"
+
+    def verify():
+        t = sets[0]
+        for _, fn in calls(0):
+            fn()
+        assert np.array_equal(t["y"].numpy(), O.threshold_updateOutput(x, 0.0, 0.0))
+        assert np.array_equal(t["gx"].numpy(), O.threshold_updateGradInput(x, gy, 0.0))
+
+    return dict(calls=calls, work=work, images=shape[0], cpu=cpu, verify=verify, bound="hbm",
+                desc="Threshold (ReLU) fwd+bwd fp32 N=64 C=128 56x56")
+
+
 def wl_copy(nsets):
     """Calibration: plain device-to-device copy of 128 MB (2 x 128 MB of HBM traffic per launch)."""
     from cunn_amd import CudaTensor as CT
@@ -410,7 +445,7 @@ def wl_copy(nsets):
 
 
 WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda n: wl_dw("cfg2", n), "cfg3": wl_bn, "cfg4": wl_pool,
-             "cfg5": wl_conv, "dilconv": wl_dilconv, "fullconv": wl_fullconv}
+             "cfg5": wl_conv, "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu}
 
 
 def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds):

@@ -25,6 +25,7 @@ ENTRY_POINTS = [
     "SpatialFullDilatedConvolution_accGradParameters",
     "SpatialFullConvolution_updateOutput", "SpatialFullConvolution_updateGradInput",
     "SpatialFullConvolution_accGradParameters",
+    "Threshold_updateOutput", "Threshold_updateGradInput",
 ]
 
 _T = C.c_void_p  # THCudaTensor* / THCudaLongTensor* / THCState*
@@ -54,6 +55,8 @@ SIGNATURES = {
     "SpatialFullConvolution_updateOutput": [_T] * 7 + [_i] * 8,
     "SpatialFullConvolution_updateGradInput": [_T] * 6 + [_i] * 8,
     "SpatialFullConvolution_accGradParameters": [_T] * 7 + [_i] * 8 + [_f],
+    "Threshold_updateOutput": [_T] * 3 + [_f, _f, _b],
+    "Threshold_updateGradInput": [_T] * 4 + [_f, _f, _b],
 }
 
 _LP = C.POINTER(C.c_long)

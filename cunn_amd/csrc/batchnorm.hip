@@ -747,8 +747,12 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
     const int xlds = (RR > 8 && train && gxp) ? 8 : 0;                                                             \
     const size_t lds = (size_t)xlds * kResBlock * sizeof(float4);                                                  \
     if (train) {                                                                                                   \
-      if (lds) THC_HIP_CHECK(hipFuncSetAttribute((const void *)bnBwdResident<RR, true, (RR <= 8)>,                 \
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));           \
+      static bool ldsRaised = false; /* once per kernel instance: allow more than 64 KB of dynamic LDS */         \
+      if (lds && !ldsRaised) {                                                                                     \
+        THC_HIP_CHECK(hipFuncSetAttribute((const void *)bnBwdResident<RR, true, (RR <= 8)>,                        \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                  \
+        ldsRaised = true;                                                                                          \
+      }                                                                                                            \
       bnBwdResident<RR, true, (RR <= 8)><<<g.C, kResBlock, lds, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_), \
                                                         dataOrNull(gradBias_), dataOrNull(weight_), meanSrc,       \
                                                         stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, xlds);    \

@@ -190,6 +190,18 @@ void THNN_CudaSpatialFullConvolution_accGradParameters(
     THCudaTensor *columns, THCudaTensor *ones,
     int kW, int kH, int dW, int dH, int padW, int padH, int adjW, int adjH, float scale);
 
+/* ---- Threshold (ReLU): the element-wise step next to the convolution path --- */
+
+/* replaces lib/THCUNN/generic/THCUNN.h:1220-1226, lib/THCUNN/generic/Threshold.cu:7-35 */
+void THNN_CudaThreshold_updateOutput(
+    THCState *state, THCudaTensor *input, THCudaTensor *output,
+    float threshold, float val, bool inplace);
+
+/* replaces lib/THCUNN/generic/THCUNN.h:1228-1235, lib/THCUNN/generic/Threshold.cu:37-67 */
+void THNN_CudaThreshold_updateGradInput(
+    THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradInput,
+    float threshold, float val, bool inplace);
+
 #ifdef __cplusplus
 }
 #endif

@@ -323,3 +323,16 @@ def avgpool_updateGradInput(x_shape, gradOut, kW, kH, dW, dH, padW, padH, ceil_m
     lib().oracle_avgpool_updateGradInput(_p(gradOut), _p(gi), N, Cc, H, W, oH, oW, kW, kH, dW, dH,
                                          padW, padH, int(bool(count_include_pad)))
     return gi
+
+
+# ------------------------------------------------------------- Threshold ----
+def threshold_updateOutput(x, threshold, val):
+    """lib/THCUNN/Threshold.cu:6-22: out = x > threshold ? x : val (a NaN input gives val)."""
+    x = _f(x)
+    return np.where(x > np.float32(threshold), x, np.float32(val)).astype(np.float32)
+
+
+def threshold_updateGradInput(x, gradOut, threshold):
+    """lib/THCUNN/Threshold.cu:42-56: gradIn = x > threshold ? gradOut : 0."""
+    x, gradOut = _f(x), _f(gradOut)
+    return np.where(x > np.float32(threshold), gradOut.reshape(x.shape), np.float32(0)).astype(np.float32)

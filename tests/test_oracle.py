@@ -416,3 +416,27 @@ def test_avgpool_vs_torch():
         gy = rng.standard_normal(y.shape).astype(np.float32)
         ty.backward(torch.from_numpy(gy).double())
         close(O.avgpool_updateGradInput(x.shape, gy, k, k, s, s, p, p, ceil, inc), tx.grad.numpy())
+
+
+# ------------------------------------------------------------------ Threshold --
+def test_threshold_vs_torch_and_special_values():
+    """F.threshold + autograd fix the values on ordinary inputs; the comparison is a strict >
+    (lib/THCUNN/Threshold.cu:18-21, 52-55), so the threshold itself and NaN fall to `val` / 0
+    (torch's own kernels let NaN through, hence NaN is pinned here by the definition, not by torch);
+    ReLU is threshold(0, 0)."""
+    rng = np.random.default_rng(60)
+    x = rng.standard_normal((3, 5, 7)).astype(np.float32)
+    x[0, 0, :2] = [0.25, np.inf]
+    for thr, val in [(0.0, 0.0), (0.25, -1.5), (-0.5, 2.0)]:
+        tx = torch.from_numpy(x.copy()).requires_grad_()
+        ty = F.threshold(tx, thr, val)
+        y = O.threshold_updateOutput(x, thr, val)
+        assert np.array_equal(y, ty.detach().numpy())
+        gy = rng.standard_normal(x.shape).astype(np.float32)
+        ty.backward(torch.from_numpy(gy))
+        assert np.array_equal(O.threshold_updateGradInput(x, gy, thr), tx.grad.numpy())
+    assert O.threshold_updateOutput(x, 0.25, -1.5)[0, 0, 0] == -1.5            # x == threshold
+    xn = np.array([np.nan, 1.0], np.float32)
+    assert np.array_equal(O.threshold_updateOutput(xn, 0.0, -3.0), np.array([-3.0, 1.0], np.float32))
+    assert np.array_equal(O.threshold_updateGradInput(xn, np.array([5.0, 6.0], np.float32), 0.0), np.array([0.0, 6.0], np.float32))
+    assert np.array_equal(O.threshold_updateOutput(x, 0, 0), np.maximum(x, 0))

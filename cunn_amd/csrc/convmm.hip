@@ -392,13 +392,26 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
 }
 
 // taps[k] = ((c*H + kh*dilH)*W + kw*dilW) * 4 for k = (c*kH + kh)*kW + kw; g is the geometry of the padded images.
+// Entries beyond Cin*kH*kW (rows padded to a multiple of BK, spare entries) point at the position's own
+// first element: valid memory, and their weights are zero or they are never used.
 __global__ void __launch_bounds__(dev::kBlock)
 buildTapTableKernel(int *taps, int entries, ConvGeom g) {
   const int KK = g.kH * g.kW;
   for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < entries; k += gridDim.x * blockDim.x) {
     const int c = k / KK, rem = k - c * KK;
     const int kh = rem / g.kW, kw = rem - kh * g.kW;
-    taps[k] = ((c * g.H + kh * g.dilH) * g.W + kw * g.dilW) * 4;
+    taps[k] = c < g.Cin ? ((c * g.H + kh * g.dilH) * g.W + kw * g.dilW) * 4 : 0;
+  }
+}
+
+// wp(rows x Kp) = w(rows x K) with zeros in columns K .. Kp-1
+__global__ void __launch_bounds__(dev::kBlock)
+padRowsKernel(const float *__restrict__ w, float *__restrict__ wp, int rows, int K, int Kp) {
+  const long total = (long)rows * Kp;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const int k = (int)(i % Kp);
+    const long r = i / Kp;
+    wp[i] = k < K ? w[r * K + k] : 0.f;
   }
 }
 
@@ -897,7 +910,47 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   }
 }
 
-// gW[i] += scale * sum_s partial[s][i], s ascending
+// gW[i] += scale * sum_s partial[s][i] in a fixed association: a workgroup owns 64 consecutive float4
+// of gW; its 4 lane groups each sum the splits s = group, group + 4, ... with 4 independent
+// accumulators (16 16-byte loads in flight per lane), then the groups are added in order through
+// LDS. With few elements and hundreds of splits (1x1 convolutions) a one-lane-per-element loop is
+// latency bound; this form keeps enough bytes in flight to run at memory speed.
+__global__ void __launch_bounds__(dev::kBlock)
+foldPartials4Kernel(const float *__restrict__ partial, float *__restrict__ dst, long count4, int splits, float scale) {
+  __shared__ float4 part[4][64];
+  const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const long i = (long)blockIdx.x * 64 + e;
+  float4 a[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) a[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (i < count4) {
+    const float4 *p = reinterpret_cast<const float4 *>(partial) + i;
+    int s = grp;
+    for (; s + 12 < splits; s += 16) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float4 v = p[(long)(s + 4 * u) * count4];
+        a[u].x += v.x, a[u].y += v.y, a[u].z += v.z, a[u].w += v.w;
+      }
+    }
+    for (; s < splits; s += 4) {
+      const float4 v = p[(long)s * count4];
+      a[0].x += v.x, a[0].y += v.y, a[0].z += v.z, a[0].w += v.w;
+    }
+  }
+  part[grp][e] = make_float4((a[0].x + a[1].x) + (a[2].x + a[3].x), (a[0].y + a[1].y) + (a[2].y + a[3].y),
+                             (a[0].z + a[1].z) + (a[2].z + a[3].z), (a[0].w + a[1].w) + (a[2].w + a[3].w));
+  __syncthreads();
+  if (grp == 0 && i < count4) {
+    const float4 p0 = part[0][e], p1 = part[1][e], p2 = part[2][e], p3 = part[3][e];
+    float4 d = reinterpret_cast<float4 *>(dst)[i];
+    d.x += scale * ((p0.x + p1.x) + (p2.x + p3.x)), d.y += scale * ((p0.y + p1.y) + (p2.y + p3.y));
+    d.z += scale * ((p0.z + p1.z) + (p2.z + p3.z)), d.w += scale * ((p0.w + p1.w) + (p2.w + p3.w));
+    reinterpret_cast<float4 *>(dst)[i] = d;
+  }
+}
+
+// the same for any count / alignment: gW[i] += scale * sum_s partial[s][i], s ascending
 __global__ void __launch_bounds__(dev::kBlock)
 foldPartialsKernel(const float *__restrict__ partial, float *__restrict__ dst, long count, int splits, float scale) {
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (long)gridDim.x * blockDim.x) {
@@ -1137,6 +1190,7 @@ struct FwdPlan {
   int mTiles, total, full, tail, nSplit, ktPerSplit;
   int tapEntries;      // > 0: the padded kernel applies; entries of the tap table at the start of the scratch
   long paddedFloats;   // floats of the zero-bordered copy of the images (0: no border needed, or generic kernel)
+  long weightFloats;   // floats of the copy of the weights with rows padded to a multiple of BK (0: not needed)
   long scratchFloats;  // tap table, tail partials, padded images
 };
 FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
@@ -1162,31 +1216,42 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
   pl.ktPerSplit = launch::ceilDiv(nkt, nSplit);
   pl.nSplit = launch::ceilDiv(nkt, pl.ktPerSplit);
   const long padded = (long)nImages * g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW);
-  const bool fast = !forceGeneric() && g.K % BK == 0 && padded * 4 < 0x7fffffffL && (long)M * g.K * 4 < 0x7fffffffL;
-  pl.tapEntries = fast ? g.K + 2 * BK : 0;  // spare entries: the kernel reads tap offsets up to two k-tiles ahead
+  // K that is not a multiple of BK (first layers: Cin = 3) runs on the same kernel with the weight rows
+  // copied into rows of Kp = nkt * BK floats, zero beyond K
+  const int Kp = nkt * BK;
+  const bool fast = !forceGeneric() && padded * 4 < 0x7fffffffL && (long)M * Kp * 4 < 0x7fffffffL;
+  pl.tapEntries = fast ? Kp + 2 * BK : 0;  // spare entries: the kernel reads tap offsets up to two k-tiles ahead
   pl.paddedFloats = fast && (g.padH > 0 || g.padW > 0) ? padded : 0;
-  pl.scratchFloats = pl.tapEntries + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0) + pl.paddedFloats;
+  pl.weightFloats = fast && Kp != g.K ? (long)M * Kp : 0;
+  pl.scratchFloats = pl.tapEntries + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0) + (pl.paddedFloats + 3) / 4 * 4 + pl.weightFloats;
   return pl;
 }
 
 // out(nImages, M, L) = bias + W(M x K) * im2col(x); `scratch` holds plan.scratchFloats floats
 void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const float *w, const float *x, float *out,
                        const float *bias, int M, int nImages, const ConvGeom &g) {
-  const bool fast = pl.tapEntries > 0 && launch::aligned16(w) && launch::aligned16(scratch);
+  const bool fast = pl.tapEntries > 0 && launch::aligned16(scratch) && (pl.weightFloats > 0 || launch::aligned16(w));
   float *partial = scratch + pl.tapEntries;
   ConvGeom gk = g;  // geometry the kernel sees
   FwdArgs p{};
   p.x = x;
   if (fast) {
     gk.H = g.H + 2 * g.padH, gk.W = g.W + 2 * g.padW, gk.padH = gk.padW = 0;
+    float *xp = partial + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0);
     if (pl.paddedFloats > 0) {
-      float *xp = partial + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0);
       launchPadPlanes(s, x, xp, (long)nImages * g.Cin, g.H, g.W, g.padH, g.padW);
       p.x = xp;
     }
     buildTapTableKernel<<<launch::directGrid(pl.tapEntries, dev::kBlock), dev::kBlock, 0, s>>>(
         reinterpret_cast<int *>(scratch), pl.tapEntries, gk);
     THC_HIP_CHECK(hipGetLastError());
+    if (pl.weightFloats > 0) {
+      float *wp = xp + (pl.paddedFloats + 3) / 4 * 4;
+      gk.K = (int)(pl.weightFloats / M);
+      padRowsKernel<<<launch::directGrid(pl.weightFloats, dev::kBlock), dev::kBlock, 0, s>>>(w, wp, M, g.K, gk.K);
+      THC_HIP_CHECK(hipGetLastError());
+      w = wp;
+    }
   }
   p.taps = reinterpret_cast<const int *>(scratch);
   p.w = w;
@@ -1196,10 +1261,10 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
   p.Ncols = nImages * g.L;
   p.mTiles = pl.mTiles;
   p.xBytes = (int)((long)nImages * gk.Cin * gk.H * gk.W * sizeof(float));
-  p.wBytes = (int)((long)M * g.K * sizeof(float));
-  p.vecA = (g.K % 4 == 0) && launch::aligned16(w);
+  p.wBytes = (int)((long)M * gk.K * sizeof(float));
+  p.vecA = (gk.K % 4 == 0) && launch::aligned16(w);
   p.nSplit = 1;
-  p.ktPerSplit = launch::ceilDiv(g.K, BK);
+  p.ktPerSplit = launch::ceilDiv(gk.K, BK);
   if (pl.full > 0) {
     if (fast)
       convFwdPaddedKernel<<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
@@ -1457,7 +1522,10 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     convGemmKernel<kGradWeight><<<grid, dev::kBlock, 0, s>>>(p, g);
   }
   THC_HIP_CHECK(hipGetLastError());
-  foldPartialsKernel<<<launch::directGrid(count, dev::kBlock), dev::kBlock, 0, s>>>(partial, gW, count, splits, scale);
+  if (count % 4 == 0 && launch::aligned16(gW) && launch::aligned16(partial))
+    foldPartials4Kernel<<<(unsigned)((count / 4 + 63) / 64), dev::kBlock, 0, s>>>(partial, gW, count / 4, splits, scale);
+  else
+    foldPartialsKernel<<<launch::directGrid(count, dev::kBlock), dev::kBlock, 0, s>>>(partial, gW, count, splits, scale);
   THC_HIP_CHECK(hipGetLastError());
 }
 

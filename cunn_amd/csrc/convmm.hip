@@ -343,6 +343,7 @@ struct FwdArgs {
   const float *bias;  // M or null
   int M, Ncols;       // Ncols = nImages * L
   int mTiles;
+  int bm, bn;         // rows and columns of an output tile: 128 x 128, or 64 x 256 (padded kernel only)
   int xBytes;         // bytes of the nImages input images (< 2^31)
   int wBytes;         // padded kernel: bytes of the weights (< 2^31)
   bool vecA;
@@ -356,18 +357,19 @@ struct FwdArgs {
 // Epilogue shared by the forward kernels: a lane holds column (lane & 31) and rows
 // 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 accumulator tile. Split workgroups store their
 // partial tile, the others add the bias and store to out(n, row, l).
+template <int TBN = BN>
 __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g, const float16v (&acc)[2][2], int bx,
                                             int by, int m0, int j0, int wm, int wn, int grp, int idx) {
   const int rowHalf = grp * 4;
   if (p.nSplit > 1) {
-    float *dst = p.partial + ((long)bx * p.nSplit + by) * (BM * BN);
+    float *dst = p.partial + ((long)bx * p.nSplit + by) * (BM * BN);  // both tile shapes hold BM * BN elements
 #pragma unroll
     for (int tj = 0; tj < 2; ++tj)
 #pragma unroll
       for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
         for (int v = 0; v < 16; ++v)
-          dst[(wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3)) * BN + wn * 64 + tj * 32 + idx] = acc[ti][tj][v];
+          dst[(wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3)) * TBN + wn * 64 + tj * 32 + idx] = acc[ti][tj][v];
     return;
   }
 #pragma unroll
@@ -595,15 +597,21 @@ __device__ __forceinline__ void mfmaHalf(const float4 *aSrc, const float4 *bSrc,
 //  * weight rows are addressed as fixed VGPR offset + scalar k offset
 //  * the loop is unrolled over the two LDS buffers, so every LDS address is base + immediate
 // Rows past M and columns past the batch are clamped to valid ones and dropped in the epilogue.
+// WM = 2: 128 x 128 tiles, the four waves as 2 x 2; WM = 1: 64 x 256 tiles, the four waves side by side,
+// for row counts whose last 128-row tile would be at most half full. A wave multiplies 64 x 64 either way.
+template <int WM>
 __global__ void __launch_bounds__(dev::kBlock, 3)
 convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
-  __shared__ float4 As[2][BK / 4][FPITCH];
-  __shared__ float4 Bs[2][BK / 4][FPITCH];
+  constexpr int TBM = 64 * WM, TBN = 256 / WM;
+  constexpr int AP = TBM + 8, BP = TBN + 8;  // float4 per k-group row
+  constexpr int NB = WM == 2 ? 8 : 16;        // image elements a lane gathers per k-tile
+  __shared__ float4 As[2][BK / 4][AP];
+  __shared__ float4 Bs[2][BK / 4][BP];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = WM == 2 ? wave >> 1 : 0, wn = WM == 2 ? wave & 1 : wave;
   const int tileIdx = p.tile0 + blockIdx.x;
   const int mTile = tileIdx % p.mTiles, nTile = tileIdx / p.mTiles;
-  const int m0 = mTile * BM, j0 = nTile * BN;
+  const int m0 = mTile * TBM, j0 = nTile * TBN;
 
   float16v acc[2][2];
 #pragma unroll
@@ -615,9 +623,14 @@ convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
 
   const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)p.w, 0, p.wBytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.xBytes, 0x00020000);
-  const int rowA = t >> 1, colB = t & 127;
-  const int aOff = (min(m0 + rowA, p.M - 1) * g.K + (t & 1) * 8) * 4;
-  const int kB = __builtin_amdgcn_readfirstlane((t >> 7) * 8);
+  // weights: WM = 2 - a lane loads 8 consecutive k of row t / 2; WM = 1 - 4 consecutive k of row t / 4
+  // image:   WM = 2 - a lane gathers 8 taps of column t % 128; WM = 1 - all 16 taps of column t
+  const int rowA = WM == 2 ? t >> 1 : t >> 2;
+  const int kgA = WM == 2 ? (t & 1) * 2 : t & 3;
+  const int colB = WM == 2 ? t & 127 : t;
+  const int kgB = WM == 2 ? (t >> 7) * 2 : 0;
+  const int aOff = (min(m0 + rowA, p.M - 1) * g.K + kgA * 4) * 4;
+  const int kB = __builtin_amdgcn_readfirstlane(kgB * 4);
   int posOff;
   {
     const long lg = min((long)j0 + colB, (long)p.Ncols - 1);
@@ -629,41 +642,43 @@ convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
   const int ktBegin = blockIdx.y * p.ktPerSplit;
   const int nkt = min(g.K / BK, ktBegin + p.ktPerSplit);  // this workgroup reduces k-tiles [ktBegin, nkt)
 
-  u32x4 ra0, ra1;
-  unsigned rb[8];
-  // The 8 tap offsets of a wave and k-tile are fetched with scalar loads one tile ahead of their use,
-  // so that no wave waits on the scalar cache inside the loop (the table has BK spare entries at its end).
+  u32x4 ra[WM];
+  unsigned rb[NB];
+  // The tap offsets of a wave and k-tile are fetched with scalar loads one tile ahead of their use,
+  // so that no wave waits on the scalar cache inside the loop (the table has spare entries at its end).
   const int4 *tapBase = reinterpret_cast<const int4 *>(p.taps + kB);
-  int4 e0 = tapBase[ktBegin * (BK / 4)], e1 = tapBase[ktBegin * (BK / 4) + 1];
+  int4 e[NB / 4];
+  auto loadTaps = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < NB / 4; ++i) e[i] = tapBase[kt * (BK / 4) + i];
+  };
   auto loadTiles = [&](int kt) {
     const int k0 = __builtin_amdgcn_readfirstlane(kt * BK);
-    ra0 = __builtin_amdgcn_raw_buffer_load_b128(wr, aOff, k0 * 4, 0);
-    ra1 = __builtin_amdgcn_raw_buffer_load_b128(wr, aOff + 16, k0 * 4, 0);
-    rb[0] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e0.x, 0);
-    rb[1] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e0.y, 0);
-    rb[2] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e0.z, 0);
-    rb[3] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e0.w, 0);
-    rb[4] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e1.x, 0);
-    rb[5] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e1.y, 0);
-    rb[6] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e1.z, 0);
-    rb[7] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e1.w, 0);
+#pragma unroll
+    for (int i = 0; i < WM; ++i) ra[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, aOff + 16 * i, k0 * 4, 0);
+#pragma unroll
+    for (int i = 0; i < NB / 4; ++i) {
+      rb[4 * i + 0] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e[i].x, 0);
+      rb[4 * i + 1] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e[i].y, 0);
+      rb[4 * i + 2] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e[i].z, 0);
+      rb[4 * i + 3] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e[i].w, 0);
+    }
   };
-  auto loadTaps = [&](int kt) { e0 = tapBase[kt * (BK / 4)], e1 = tapBase[kt * (BK / 4) + 1]; };
-  u32x4 *aDst = reinterpret_cast<u32x4 *>(&As[0][(t & 1) * 2][rowA]);
-  u32x4 *bDst = reinterpret_cast<u32x4 *>(&Bs[0][(t >> 7) * 2][colB]);
+  u32x4 *aDst = reinterpret_cast<u32x4 *>(&As[0][kgA][rowA]);
+  u32x4 *bDst = reinterpret_cast<u32x4 *>(&Bs[0][kgB][colB]);
+  constexpr int BUFA = (BK / 4) * AP, BUFB = (BK / 4) * BP;  // float4 per LDS buffer
   auto storeTiles = [&](auto bufc) {
-    constexpr int o = decltype(bufc)::value * (BK / 4) * FPITCH;
-    aDst[o] = ra0;
-    aDst[o + FPITCH] = ra1;
-    bDst[o] = u32x4{rb[0], rb[1], rb[2], rb[3]};
-    bDst[o + FPITCH] = u32x4{rb[4], rb[5], rb[6], rb[7]};
+    constexpr int b = decltype(bufc)::value;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) aDst[b * BUFA + i * AP] = ra[i];
+#pragma unroll
+    for (int i = 0; i < NB / 4; ++i) bDst[b * BUFB + i * BP] = u32x4{rb[4 * i], rb[4 * i + 1], rb[4 * i + 2], rb[4 * i + 3]};
   };
   const int grp = lane >> 5, idx = lane & 31;
   const float4 *aSrc = &As[0][grp][wm * 64 + idx];
   const float4 *bSrc = &Bs[0][grp][wn * 64 + idx];
   using Buf0 = std::integral_constant<int, 0>;
   using Buf1 = std::integral_constant<int, 1>;
-  constexpr int BUFA = (BK / 4) * FPITCH;  // float4 per LDS buffer
 
   // Software pipeline. While tile kt is multiplied out of one LDS buffer, tile kt + 1 waits in
   // registers and tile kt + 2 is requested from memory:
@@ -673,8 +688,8 @@ convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
   // queued work while they run and the only stall left at the barrier is the LDS read latency.
   // The scheduling fences pin that order.
   auto step = [&](auto cur, auto nxt, int kt, bool store, bool load) {
-    constexpr int C = decltype(cur)::value, N = decltype(nxt)::value;
-    mfmaHalf<C * BUFA, C * BUFA>(aSrc, bSrc, acc);
+    constexpr int C = decltype(cur)::value;
+    mfmaHalf<C * BUFA, C * BUFB>(aSrc, bSrc, acc);
     __builtin_amdgcn_sched_barrier(0);
     if (store) storeTiles(nxt);
     if (load) {
@@ -682,11 +697,11 @@ convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
       loadTaps(kt + 3);
     }
     __builtin_amdgcn_sched_barrier(0);
-    mfmaHalf<C * BUFA + 2 * FPITCH, C * BUFA + 2 * FPITCH>(aSrc, bSrc, acc);
-    (void)N;
+    mfmaHalf<C * BUFA + 2 * AP, C * BUFB + 2 * BP>(aSrc, bSrc, acc);
     __syncthreads();
   };
 
+  loadTaps(ktBegin);
   loadTiles(ktBegin);
   loadTaps(ktBegin + 1);
   storeTiles(Buf0{});
@@ -704,7 +719,7 @@ convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
   step(Buf0{}, Buf1{}, kt, kt + 1 < nkt, kt + 2 < nkt);
   if (kt + 1 < nkt) step(Buf1{}, Buf0{}, kt + 1, kt + 2 < nkt, false);
   if (kt + 2 < nkt) step(Buf0{}, Buf1{}, kt + 2, false, false);
-  fwdEpilogue(p, g, acc, blockIdx.x, blockIdx.y, m0, j0, wm, wn, grp, idx);
+  fwdEpilogue<TBN>(p, g, acc, blockIdx.x, blockIdx.y, m0, j0, wm, wn, grp, idx);
 }
 
 // out tile = bias + sum over the nSplit partial tiles (ascending split order).
@@ -714,20 +729,20 @@ fwdTailFixupKernel(FwdArgs p, ConvGeom g) {
   const int tileIdx = p.tile0 + blockIdx.x;
   const int mTile = tileIdx % p.mTiles, nTile = tileIdx / p.mTiles;
   const float *src = p.partial + (long)blockIdx.x * p.nSplit * (BM * BN);
-  const int e = (blockIdx.y * dev::kBlock + threadIdx.x) * 4;  // BN % 4 == 0: the 4 elements share a row
+  const int e = (blockIdx.y * dev::kBlock + threadIdx.x) * 4;  // tile width % 4 == 0: the 4 elements share a row
   float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
   for (int s = 0; s < p.nSplit; ++s) {
     const float4 q = *reinterpret_cast<const float4 *>(src + (long)s * (BM * BN) + e);
     v.x += q.x, v.y += q.y, v.z += q.z, v.w += q.w;
   }
-  const int r = e / BN, c = e - r * BN;
-  const int row = mTile * BM + r;
+  const int r = e / p.bn, c = e - r * p.bn;
+  const int row = mTile * p.bm + r;
   if (row >= p.M) return;
   const float b = p.bias ? p.bias[row] : 0.f;
   const float vals[4] = {v.x + b, v.y + b, v.z + b, v.w + b};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const long col = (long)nTile * BN + c + i;
+    const long col = (long)nTile * p.bn + c + i;
     if (col >= p.Ncols) break;
     const int n = (int)(col / g.L);
     const int l = (int)(col - (long)n * g.L);
@@ -1187,17 +1202,26 @@ bool forceGeneric() {
 // finish one more tile, so the tiles of that round are instead split along K
 // over all CUs (partials in scratch, folded by fwdTailFixupKernel in a fixed order).
 struct FwdPlan {
+  int bm, bn;          // tile shape: 128 x 128, or 64 x 256 when that wastes fewer rows (padded kernel only)
   int mTiles, total, full, tail, nSplit, ktPerSplit;
   int tapEntries;      // > 0: the padded kernel applies; entries of the tap table at the start of the scratch
   long paddedFloats;   // floats of the zero-bordered copy of the images (0: no border needed, or generic kernel)
   long weightFloats;   // floats of the copy of the weights with rows padded to a multiple of BK (0: not needed)
   long scratchFloats;  // tap table, tail partials, padded images
 };
-FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
+// wAligned: the weights start on a 16-byte boundary (else the padded kernel works on an aligned copy)
+FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g, bool wAligned = true) {
   FwdPlan pl{};
   const int nkt = launch::ceilDiv(g.K, BK);
-  pl.mTiles = (int)tiles(M, BM);
-  pl.total = pl.mTiles * (int)tiles((long)nImages * g.L, BN);
+  const long padded = (long)nImages * g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW);
+  // K that is not a multiple of BK (first layers: Cin = 3) runs on the same kernel with the weight rows
+  // copied into rows of Kp = nkt * BK floats, zero beyond K
+  const int Kp = nkt * BK;
+  const bool fast = !forceGeneric() && padded * 4 < 0x7fffffffL && (long)M * Kp * 4 < 0x7fffffffL;
+  const bool wide = fast && tiles(M, 64) * 64 < tiles(M, BM) * BM;
+  pl.bm = wide ? 64 : BM, pl.bn = wide ? 256 : BN;
+  pl.mTiles = (int)tiles(M, pl.bm);
+  pl.total = pl.mTiles * (int)tiles((long)nImages * g.L, pl.bn);
   const int cus = residentSlots(nullptr);
   int nSplit = 1;
   if (pl.total > cus) {
@@ -1206,7 +1230,7 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
   } else {
     // fewer tiles than CUs: every tile is split along K so that the grid fills the resident slots
     pl.tail = pl.total;
-    nSplit = std::min(nkt / 4, residentSlots((const void *)convFwdPaddedKernel) / pl.total);
+    nSplit = std::min(nkt / 4, residentSlots((const void *)convFwdPaddedKernel<2>) / pl.total);
   }
   if (nSplit < 2) {
     pl.tail = 0;
@@ -1215,14 +1239,9 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
   pl.full = pl.total - pl.tail;
   pl.ktPerSplit = launch::ceilDiv(nkt, nSplit);
   pl.nSplit = launch::ceilDiv(nkt, pl.ktPerSplit);
-  const long padded = (long)nImages * g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW);
-  // K that is not a multiple of BK (first layers: Cin = 3) runs on the same kernel with the weight rows
-  // copied into rows of Kp = nkt * BK floats, zero beyond K
-  const int Kp = nkt * BK;
-  const bool fast = !forceGeneric() && padded * 4 < 0x7fffffffL && (long)M * Kp * 4 < 0x7fffffffL;
   pl.tapEntries = fast ? Kp + 2 * BK : 0;  // spare entries: the kernel reads tap offsets up to two k-tiles ahead
   pl.paddedFloats = fast && (g.padH > 0 || g.padW > 0) ? padded : 0;
-  pl.weightFloats = fast && Kp != g.K ? (long)M * Kp : 0;
+  pl.weightFloats = fast && (Kp != g.K || !wAligned) ? (long)M * Kp : 0;
   pl.scratchFloats = pl.tapEntries + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0) + (pl.paddedFloats + 3) / 4 * 4 + pl.weightFloats;
   return pl;
 }
@@ -1230,7 +1249,9 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g) {
 // out(nImages, M, L) = bias + W(M x K) * im2col(x); `scratch` holds plan.scratchFloats floats
 void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const float *w, const float *x, float *out,
                        const float *bias, int M, int nImages, const ConvGeom &g) {
-  const bool fast = pl.tapEntries > 0 && launch::aligned16(scratch) && (pl.weightFloats > 0 || launch::aligned16(w));
+  const bool fast = pl.tapEntries > 0;
+  if (fast && !(launch::aligned16(scratch) && (pl.weightFloats > 0 || launch::aligned16(w))))
+    error("SpatialConvolutionMM: internal error, convolution scratch or weights not 16-byte aligned");
   float *partial = scratch + pl.tapEntries;
   ConvGeom gk = g;  // geometry the kernel sees
   FwdArgs p{};
@@ -1260,14 +1281,17 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
   p.M = M;
   p.Ncols = nImages * g.L;
   p.mTiles = pl.mTiles;
+  p.bm = pl.bm, p.bn = pl.bn;
   p.xBytes = (int)((long)nImages * gk.Cin * gk.H * gk.W * sizeof(float));
   p.wBytes = (int)((long)M * gk.K * sizeof(float));
   p.vecA = (gk.K % 4 == 0) && launch::aligned16(w);
   p.nSplit = 1;
   p.ktPerSplit = launch::ceilDiv(gk.K, BK);
   if (pl.full > 0) {
-    if (fast)
-      convFwdPaddedKernel<<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
+    if (fast && pl.bm == 64)
+      convFwdPaddedKernel<1><<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
+    else if (fast)
+      convFwdPaddedKernel<2><<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
     else
       convFwdImplicitKernel<<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
     THC_HIP_CHECK(hipGetLastError());
@@ -1277,8 +1301,10 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
     p.ktPerSplit = pl.ktPerSplit;
     p.nSplit = pl.nSplit;
     p.partial = partial;
-    if (fast)
-      convFwdPaddedKernel<<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, gk);
+    if (fast && pl.bm == 64)
+      convFwdPaddedKernel<1><<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, gk);
+    else if (fast)
+      convFwdPaddedKernel<2><<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, gk);
     else
       convFwdImplicitKernel<<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, gk);
     THC_HIP_CHECK(hipGetLastError());
@@ -1293,7 +1319,8 @@ float *scratchFloats(THCState *state, THCudaTensor *buffer, long floats, Temp &t
   if (buffer) {
     resize(state, buffer, {floats});
     if (!isContiguous(erase(buffer))) error("%s tensor has to be contiguous", name);
-    return data(buffer);
+    if (launch::aligned16(data(buffer))) return data(buffer);
+    // a buffer tensor at an odd storage offset: its contents are unspecified anyway, work in a temporary
   }
   tmp = Temp(state->stream, (size_t)floats * sizeof(float));
   return (float *)tmp.get();
@@ -1314,12 +1341,12 @@ void convForward(THCState *state, const ConvGeom &g, const float *x, const float
   const bool implicit2 = !forceGeneric() && imgBytes < (1L << 30);
   if (implicit2) group = (int)std::min<long>(group, std::max<long>(1, ((1L << 31) - 1 - 4096) / imgBytes));
   if (implicit2) {
-    FwdPlan pl = planFwdImplicit(g.Cout, std::min(group, g.N), g);
+    FwdPlan pl = planFwdImplicit(g.Cout, std::min(group, g.N), g, launch::aligned16(w));
     Temp tmp;
     float *scratch = scratchFloats(state, scratchBuf, pl.scratchFloats, tmp, bufName);
     for (int n0 = 0; n0 < g.N; n0 += group) {
       int cnt = std::min(group, g.N - n0);
-      if (cnt != std::min(group, g.N)) pl = planFwdImplicit(g.Cout, cnt, g);  // last, smaller group: needs no more scratch
+      if (cnt != std::min(group, g.N)) pl = planFwdImplicit(g.Cout, cnt, g, launch::aligned16(w));  // last, smaller group: needs no more scratch
       launchFwdImplicit(s, pl, scratch, w, x + (long)n0 * g.Cin * g.H * g.W, out + (long)n0 * g.Cout * g.L, bias, g.Cout,
                         cnt, g);
     }

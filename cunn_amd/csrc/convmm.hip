@@ -762,8 +762,6 @@ fwdTailFixupKernel(FwdArgs p, ConvGeom g) {
 // 16 consecutive lanes gather 16 consecutive positions (64-byte runs of x).
 // L16: L % 16 == 0 - a k-tile never crosses an image, so the gradOutput offsets are a
 // fixed VGPR part plus a scalar part.
-constexpr int GPITCH = BN + 4;  // float4 per position-group row of Bs: the 4 groups of a wave's scalar stores hit disjoint banks
-
 struct GradWeightArgs {
   const float *gy;  // (N, M, L)
   const float *x;   // (N, Cin, H, W) of g: images with their zero border
@@ -775,19 +773,24 @@ struct GradWeightArgs {
   unsigned magicOW;
 };
 
-template <bool L16>
+// WM = 2: 128 x 128 tiles of gradWeight (Cout x K), WM = 1: 64 x 256 tiles (as in the forward kernel).
+template <bool L16, int WM>
 __global__ void __launch_bounds__(dev::kBlock, 3)
 convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
-  __shared__ float4 As[2][BK / 4][FPITCH];
-  __shared__ float4 Bs[2][BK / 4][GPITCH];
+  constexpr int TBM = 64 * WM, TBN = 256 / WM;
+  constexpr int AP = TBM + 8;   // float4 per position-group row of As
+  constexpr int GP = TBN + 4;   // of Bs: the 4 groups of a wave's scalar stores hit disjoint banks
+  constexpr int NB = TBN / 16;  // columns a lane gathers per k-tile
+  __shared__ float4 As[2][BK / 4][AP];
+  __shared__ float4 Bs[2][BK / 4][GP];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = WM == 2 ? wave >> 1 : 0, wn = WM == 2 ? wave & 1 : wave;
   // workgroups that reduce the same positions (one split) are neighbours in the remapped order: same XCD, same L2
   const int tilesPerSplit = p.mTiles * p.nTiles;
   const int bid = dev::xcdRemap(blockIdx.x, gridDim.x);
   const int split = bid / tilesPerSplit, tileIdx = bid - split * tilesPerSplit;
   const int mTile = tileIdx % p.mTiles, nTile = tileIdx / p.mTiles;
-  const int m0 = mTile * BM, j0 = nTile * BN;
+  const int m0 = mTile * TBM, j0 = nTile * TBN;
   const int ktBegin = split * p.ktPerSplit;
   const int ktEnd = min(p.totalKt, ktBegin + p.ktPerSplit);
   const int kOob = 0x7fffffff;
@@ -800,25 +803,27 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  // ---- A loader: row o = t >> 1, positions 8 * (t & 1) .. + 7 of the k-tile as two float4
+  // ---- A loader. WM = 2: row o = t >> 1, positions 8 * (t & 1) .. + 7 of the k-tile as two float4;
+  //                WM = 1: row o = t >> 2, positions 4 * (t & 3) .. + 3 as one float4
   const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc((void *)p.gy, 0, p.gyBytes, 0x00020000);
-  const int rowA = t >> 1;
+  const int rowA = WM == 2 ? t >> 1 : t >> 2;
+  const int pgA = WM == 2 ? (t & 1) * 2 : t & 3;  // first position group (of 4 positions) of the lane
   const int rowOffA = min(m0 + rowA, p.M - 1) * g.L * 4;  // rows past M are clamped and dropped in the epilogue
   const int imgStrideA = p.M * g.L * 4;
   int nA, lA;  // L16: scalar image and position of the k-tile; else: of this lane's first group
   {
-    const long r = (long)ktBegin * BK + (L16 ? 0 : (t & 1) * 8);
+    const long r = (long)ktBegin * BK + (L16 ? 0 : pgA * 4);
     nA = (int)(r / g.L);
     lA = (int)(r - (long)nA * g.L);
   }
   // ---- B loader: position t & 15 of the k-tile, columns (t >> 4) + 16 i
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.xBytes, 0x00020000);
   const int rB = t & 15, cB = t >> 4;
-  int tapOff[8];
+  int tapOff[NB];
   {
     const int KK = g.kH * g.kW;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < NB; ++i) {
       const int k = min(j0 + cB + 16 * i, p.Ncols - 1);  // columns past K are dropped in the epilogue
       const int c = k / KK, rem = k - c * KK;
       const int kh = rem / g.kW, kw = rem - kh * g.kW;
@@ -835,24 +840,26 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
     nOffB = n * imgStrideB;
   }
 
-  u32x4 ra0, ra1;
-  unsigned rb[8];
+  u32x4 ra[WM];
+  unsigned rb[NB];
   // loads the k-tile the position counters stand on, then advances them by BK (L >= BK: one wrap at most)
   auto loadTiles = [&]() {
     if constexpr (L16) {
       // N*L is a multiple of BK here, so every k-tile lies inside the batch (the scalar offset is not range-checked)
       const int so = __builtin_amdgcn_readfirstlane(nA * imgStrideA + lA * 4);
-      ra0 = __builtin_amdgcn_raw_buffer_load_b128(gr, rowOffA + (t & 1) * 32, so, 0);
-      ra1 = __builtin_amdgcn_raw_buffer_load_b128(gr, rowOffA + (t & 1) * 32 + 16, so, 0);
+#pragma unroll
+      for (int i = 0; i < WM; ++i) ra[i] = __builtin_amdgcn_raw_buffer_load_b128(gr, rowOffA + pgA * 16 + 16 * i, so, 0);
       lA += BK;
       if (lA >= g.L) lA -= g.L, ++nA;
     } else {
-      int n1 = nA, l1 = lA + 4;
-      if (l1 >= g.L) l1 -= g.L, ++n1;
       const int o0 = nA < g.N ? nA * imgStrideA + rowOffA + lA * 4 : kOob;
-      const int o1 = n1 < g.N ? n1 * imgStrideA + rowOffA + l1 * 4 : kOob;
-      ra0 = __builtin_amdgcn_raw_buffer_load_b128(gr, o0, 0, 0);
-      ra1 = __builtin_amdgcn_raw_buffer_load_b128(gr, o1, 0, 0);
+      ra[0] = __builtin_amdgcn_raw_buffer_load_b128(gr, o0, 0, 0);
+      if constexpr (WM == 2) {
+        int n1 = nA, l1 = lA + 4;
+        if (l1 >= g.L) l1 -= g.L, ++n1;
+        const int o1 = n1 < g.N ? n1 * imgStrideA + rowOffA + l1 * 4 : kOob;
+        ra[WM - 1] = __builtin_amdgcn_raw_buffer_load_b128(gr, o1, 0, 0);
+      }
       lA += BK;
       if (lA >= g.L) lA -= g.L, ++nA;
     }
@@ -860,27 +867,27 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
       const int oh = dev::fastDiv(lB, p.magicOW), ow = lB - oh * g.oW;
       const int posOff = nOffB + oh * rowStepB + ow * colStepB;
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
+      for (int i = 0; i < NB; ++i)
         rb[i] = __builtin_amdgcn_raw_buffer_load_b32(xr, (int)((unsigned)posOff + (unsigned)tapOff[i]), 0, 0);
       lB += BK;
       if (lB >= g.L) lB -= g.L, nOffB += imgStrideB;
     }
   };
-  u32x4 *aDst = reinterpret_cast<u32x4 *>(&As[0][(t & 1) * 2][rowA]);
+  u32x4 *aDst = reinterpret_cast<u32x4 *>(&As[0][pgA][rowA]);
   unsigned *bDst = reinterpret_cast<unsigned *>(&Bs[0][rB >> 2][cB]) + (rB & 3);
+  constexpr int BUFA = (BK / 4) * AP, BUFB = (BK / 4) * GP;  // float4 per LDS buffer
   auto storeTiles = [&](auto bufc) {
     constexpr int buf = decltype(bufc)::value;
-    aDst[buf * (BK / 4) * FPITCH] = ra0;
-    aDst[buf * (BK / 4) * FPITCH + FPITCH] = ra1;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) bDst[buf * (BK / 4) * GPITCH * 4 + 64 * i] = rb[i];  // column + 16 = 16 float4 further
+    for (int i = 0; i < WM; ++i) aDst[buf * BUFA + i * AP] = ra[i];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) bDst[buf * BUFB * 4 + 64 * i] = rb[i];  // column + 16 = 16 float4 further
   };
   const int grp = lane >> 5, idx = lane & 31;
   const float4 *aSrc = &As[0][grp][wm * 64 + idx];
   const float4 *bSrc = &Bs[0][grp][wn * 64 + idx];
   using Buf0 = std::integral_constant<int, 0>;
   using Buf1 = std::integral_constant<int, 1>;
-  constexpr int BUFA = (BK / 4) * FPITCH, BUFB = (BK / 4) * GPITCH;  // float4 per LDS buffer
 
   // same software pipeline as the forward kernel: tile kt in LDS, kt + 1 in registers, kt + 2 requested
   auto step = [&](auto cur, auto nxt, bool store, bool load) {
@@ -890,7 +897,7 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
     if (store) storeTiles(nxt);
     if (load) loadTiles();
     __builtin_amdgcn_sched_barrier(0);
-    mfmaHalf<C * BUFA + 2 * FPITCH, C * BUFB + 2 * GPITCH>(aSrc, bSrc, acc);
+    mfmaHalf<C * BUFA + 2 * AP, C * BUFB + 2 * GP>(aSrc, bSrc, acc);
     __syncthreads();
   };
   if (ktBegin < ktEnd) {
@@ -1486,7 +1493,6 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   // splits some CUs would carry one workgroup more than others for the whole
   // kernel.
   if ((long)g.N * g.L >= 0x7fffffffL) error("spatial convolution: batch too large");
-  const int mT = (int)tiles(g.Cout, BM), nT = (int)tiles(g.K, BN);
   const int totalKt = launch::ceilDiv(g.N * g.L, BK);
   // second-generation kernel: gradOutput rows loadable as float4 groups, 32-bit byte offsets into both operands
   const bool bordered = g.padH > 0 || g.padW > 0;
@@ -1495,9 +1501,12 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   const bool fast = !forceGeneric() && g.L % 4 == 0 && g.L >= BK && launch::aligned16(gy) &&
                     gyBytes < 0x7fffffffL && xpFloats * 4 < 0x7fffffffL - 65536 && (long)g.L * g.oW < 0x7fffffffL;
   const bool l16 = g.L % BK == 0;
+  // tile shape: 64 x 256 where it covers gradWeight (Cout x K) with less padding than 128 x 128
+  const bool wide = fast && tiles(g.Cout, 64) * 64 * tiles(g.K, 256) * 256 < tiles(g.Cout, BM) * BM * tiles(g.K, BN) * BN;
+  const int mT = (int)tiles(g.Cout, wide ? 64 : BM), nT = (int)tiles(g.K, wide ? 256 : BN);
   const void *kern = !fast ? (const void *)convGemmKernel<kGradWeight>
-                     : l16 ? (const void *)convGradWeightKernel<true>
-                           : (const void *)convGradWeightKernel<false>;
+                     : l16 ? (wide ? (const void *)convGradWeightKernel<true, 1> : (const void *)convGradWeightKernel<true, 2>)
+                           : (wide ? (const void *)convGradWeightKernel<false, 1> : (const void *)convGradWeightKernel<false, 2>);
   const int slots = residentSlots(kern);
   int splits = std::max(1, std::min(totalKt, slots / (mT * nT)));
   const int perSplit = launch::ceilDiv(totalKt, splits);
@@ -1529,10 +1538,15 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     q.gyBytes = (int)gyBytes;
     q.xBytes = (int)(xpFloats * 4);
     q.magicOW = dev::magicOf(g.oW);
-    if (l16)
-      convGradWeightKernel<true><<<dim3(mT * nT * splits), dev::kBlock, 0, s>>>(q, gk);
+    const dim3 grid(mT * nT * splits);
+    if (l16 && wide)
+      convGradWeightKernel<true, 1><<<grid, dev::kBlock, 0, s>>>(q, gk);
+    else if (l16)
+      convGradWeightKernel<true, 2><<<grid, dev::kBlock, 0, s>>>(q, gk);
+    else if (wide)
+      convGradWeightKernel<false, 1><<<grid, dev::kBlock, 0, s>>>(q, gk);
     else
-      convGradWeightKernel<false><<<dim3(mT * nT * splits), dev::kBlock, 0, s>>>(q, gk);
+      convGradWeightKernel<false, 2><<<grid, dev::kBlock, 0, s>>>(q, gk);
   } else {
     GemmArgs p{};
     p.a = gy;

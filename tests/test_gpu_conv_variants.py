@@ -189,13 +189,14 @@ def test_full_convolution_errors(T):
 
 
 TILE_CASES = [
-    # both output-tile shapes of the forward kernel (128 x 128, and 64 x 256 where the last 128 rows
-    # would be at most half used), for the forward pass (rows = Cout) and the stride-1 gradInput (rows = Cin)
+    # both tile shapes of the forward and weight-gradient kernels (128 x 128, and 64 x 256 where that
+    # wastes less of the tile): forward (rows = Cout), stride-1 gradInput (rows = Cin), gradWeight (Cout x K)
     (2, 40, 200, 20, 20, 3, 3, 1, 1, 1, 1, 1, 1),    # forward 128-row tiles, gradInput 64-row tiles
     (2, 192, 192, 12, 12, 3, 3, 1, 1, 1, 1, 1, 1),   # 192 rows = 3 x 64
     (2, 130, 70, 14, 18, 3, 3, 1, 1, 1, 1, 1, 1),    # gradInput: 130 rows, last 64-row tile holds 2
     (32, 16, 64, 48, 48, 3, 3, 1, 1, 1, 1, 1, 1),    # 64 rows, more tiles than CUs: full rounds + K-split tail
     (3, 3, 64, 40, 40, 7, 7, 2, 2, 3, 3, 1, 1),      # K = 147 padded to 160, stride 2
+    (2, 24, 48, 18, 22, 3, 3, 1, 1, 1, 1, 1, 1),     # 64 x 256 weight-gradient tiles with L % 16 != 0
 ]
 
 

@@ -17,8 +17,10 @@
 //   updateGradInput    gradCol[k][n,l] = sum_o W[o][k] * gy[n][o][l] for a group
 //                      of images into `gradColumns`, then the col2im gather of
 //                      lib/THCUNN/im2col.h:63-102 over the group.
+#include <cstring>
 #include <map>
 #include <mutex>
+#include <numeric>
 #include <type_traits>
 
 #include "device_utils.h"
@@ -339,7 +341,9 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 struct FwdArgs {
   const float *w;     // (M x K) row-major
   const float *x;     // images n0 .. n0 + nImages - 1 of (N, Cin, H, W)
-  float *out;         // (nImages, M, L)
+  float *out;         // element (n, row, oh, ow) at out[n * outImg + row * outRow + oh * outSH + ow * outSW]
+  long outImg;        // dense output (nImages, M, oH, oW): M * L, L, oW, 1
+  int outRow, outSH, outSW;
   const float *bias;  // M or null
   int M, Ncols;       // Ncols = nImages * L
   int mTiles;
@@ -378,7 +382,8 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
     if (col >= p.Ncols) continue;
     const int n = (int)(col / g.L);
     const int l = (int)(col - (long)n * g.L);
-    float *dst = p.out + (long)n * p.M * g.L + l;
+    const int oh = l / g.oW, ow = l - oh * g.oW;
+    float *dst = p.out + (long)n * p.outImg + (long)oh * p.outSH + ow * p.outSW;
 #pragma unroll
     for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
@@ -387,7 +392,7 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
         if (row < p.M) {
           float val = acc[ti][tj][v];
           if (p.bias) val += p.bias[row];
-          dst[(long)row * g.L] = val;
+          dst[(long)row * p.outRow] = val;
         }
       }
   }
@@ -417,19 +422,18 @@ padRowsKernel(const float *__restrict__ w, float *__restrict__ wp, int rows, int
   }
 }
 
-// xp(nc, H + 2 padH, W + 2 padW) = x(nc, H, W) inside a zero border. grid = (planes, chunks of a plane);
+// xp(nc, Hp, Wp) = x(nc, H, W) at row padTop, column padLeft inside zeros. grid = (planes, chunks of a plane);
 // VEC: a lane produces 4 consecutive floats of the bordered plane with one 16-byte store
 // (plane size a multiple of 4 floats, 16-byte aligned destination).
 template <bool VEC>
 __global__ void __launch_bounds__(dev::kBlock)
-padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int padH, int padW) {
-  const int Hp = H + 2 * padH, Wp = W + 2 * padW;
+padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int padTop, int padLeft, int Hp, int Wp) {
   const unsigned magic = dev::magicOf(Wp);
   const float *src = x + (long)blockIdx.x * H * W;
   float *dst = xp + (long)blockIdx.x * Hp * Wp;
   auto fetch = [&](int j) {
     const int hp = dev::fastDiv(j, magic), wp = j - hp * Wp;
-    const int h = hp - padH, w = wp - padW;
+    const int h = hp - padTop, w = wp - padLeft;
     return (((unsigned)h < (unsigned)H) & ((unsigned)w < (unsigned)W)) ? src[h * W + w] : 0.f;
   };
   const int i = blockIdx.y * dev::kBlock + threadIdx.x;
@@ -441,14 +445,83 @@ padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int 
   }
 }
 
-void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int H, int W, int padH, int padW) {
-  const int plane = (H + 2 * padH) * (W + 2 * padW);
+void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int H, int W, int padTop, int padLeft, int Hp,
+                     int Wp) {
+  const int plane = Hp * Wp;
   if (launch::ceilDiv(plane, dev::kBlock) > 65535) error("SpatialConvolutionMM: image plane too large");
   if (plane % 4 == 0 && launch::aligned16(xp))
-    padPlanesKernel<true><<<dim3((unsigned)planes, launch::ceilDiv(plane / 4, dev::kBlock)), dev::kBlock, 0, s>>>(x, xp, H, W, padH, padW);
+    padPlanesKernel<true><<<dim3((unsigned)planes, launch::ceilDiv(plane / 4, dev::kBlock)), dev::kBlock, 0, s>>>(
+        x, xp, H, W, padTop, padLeft, Hp, Wp);
   else
-    padPlanesKernel<false><<<dim3((unsigned)planes, launch::ceilDiv(plane, dev::kBlock)), dev::kBlock, 0, s>>>(x, xp, H, W, padH, padW);
+    padPlanesKernel<false><<<dim3((unsigned)planes, launch::ceilDiv(plane, dev::kBlock)), dev::kBlock, 0, s>>>(
+        x, xp, H, W, padTop, padLeft, Hp, Wp);
   THC_HIP_CHECK(hipGetLastError());
+}
+inline void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int H, int W, int padH, int padW) {
+  launchPadPlanes(s, x, xp, planes, H, W, padH, padW, H + 2 * padH, W + 2 * padW);
+}
+
+// ---- gradInput by output phase ------------------------------------------------------------------
+// gi[h] receives gy[oh] * w[kh] where h + pad = oh * stride + kh * dil. For the positions
+// h = ph + stride * i of one phase only the taps with kh * dil = ph + pad (mod stride) contribute,
+// they form an arithmetic sequence kh = k0 + a * kStep, and tap a reads gy row i + q0 - a * qStep:
+// per phase a stride-1 convolution of gy with a sub-kernel, written to a strided sub-grid of gi.
+struct PhaseAxis {
+  int n;                // gi positions of the phase along the axis
+  int k0, kStep, nk;    // contributing taps
+  int q0, qStep;        // gy index of tap a at position i: i + q0 - a * qStep
+};
+struct Phase {
+  PhaseAxis h, w;
+  int h0, w0;           // first gi row / column of the phase
+  int K, Kp;            // Cout * h.nk * w.nk, rounded up to a positive multiple of BK
+  int tapOfs;           // ints from the start of the tap tables
+  long wOfs;            // floats from the start of the phase weights
+};
+constexpr int kMaxPhases = 16;
+struct PhaseSet {
+  Phase ph[kMaxPhases];
+  int count;
+};
+
+// Phase weights Wp(Cin x Kp): Wp[c][(o, a, b)] = w[o][c][h.k0 + a*h.kStep][w.k0 + b*w.kStep], zero from K to Kp.
+// grid = (chunks, phases)
+__global__ void __launch_bounds__(dev::kBlock)
+phaseWeightsKernel(const float *__restrict__ w, float *__restrict__ dst, PhaseSet set, int Cin, int kH, int kW) {
+  const Phase &P = set.ph[blockIdx.y];
+  const long total = (long)Cin * P.Kp;
+  const int taps = P.h.nk * P.w.nk;
+  float *d = dst + P.wOfs;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const int k = (int)(i % P.Kp);
+    const int c = (int)(i / P.Kp);
+    float v = 0.f;
+    if (k < P.K) {
+      const int o = k / taps, r = k - o * taps;
+      const int a = r / P.w.nk, b = r - a * P.w.nk;
+      v = w[(((long)o * Cin + c) * kH + P.h.k0 + a * P.h.kStep) * kW + P.w.k0 + b * P.w.kStep];
+    }
+    d[i] = v;
+  }
+}
+
+// Tap tables of the phases: byte offset of (o, a, b) inside a bordered gy image (Hp x Wp planes, gy at
+// row top, column left), relative to the position's own (i, j); 0 for the entries beyond K.
+__global__ void __launch_bounds__(dev::kBlock)
+phaseTapsKernel(int *__restrict__ taps, PhaseSet set, int Hp, int Wp, int top, int left) {
+  const Phase &P = set.ph[blockIdx.y];
+  const int entries = P.Kp + 2 * BK;
+  const int tp = P.h.nk * P.w.nk;
+  int *d = taps + P.tapOfs;
+  for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < entries; k += gridDim.x * blockDim.x) {
+    int v = 0;
+    if (k < P.K) {
+      const int o = k / tp, r = k - o * tp;
+      const int a = r / P.w.nk, b = r - a * P.w.nk;
+      v = ((o * Hp + top + P.h.q0 - a * P.h.qStep) * Wp + left + P.w.q0 - b * P.w.qStep) * 4;
+    }
+    d[k] = v;
+  }
 }
 
 // Generic forward kernel: any K, any alignment; taps and bounds resolved in the loop.
@@ -600,8 +673,7 @@ __device__ __forceinline__ void mfmaHalf(const float4 *aSrc, const float4 *bSrc,
 // WM = 2: 128 x 128 tiles, the four waves as 2 x 2; WM = 1: 64 x 256 tiles, the four waves side by side,
 // for row counts whose last 128-row tile would be at most half full. A wave multiplies 64 x 64 either way.
 template <int WM>
-__global__ void __launch_bounds__(dev::kBlock, 3)
-convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
+__device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &g) {
   constexpr int TBM = 64 * WM, TBN = 256 / WM;
   constexpr int AP = TBM + 8, BP = TBN + 8;  // float4 per k-group row
   constexpr int NB = WM == 2 ? 8 : 16;        // image elements a lane gathers per k-tile
@@ -722,10 +794,35 @@ convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
   fwdEpilogue<TBN>(p, g, acc, blockIdx.x, blockIdx.y, m0, j0, wm, wn, grp, idx);
 }
 
+template <int WM>
+__global__ void __launch_bounds__(dev::kBlock, 3)
+convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
+  fwdPaddedBody<WM>(p, g);
+}
+
+// Several independent GEMMs of the same tile shape in one launch (the phases of a strided gradInput):
+// grid = (most tiles of an item, most splits of an item, items); workgroups beyond an item's own extent leave.
+struct FwdBatchItem {
+  FwdArgs p;
+  ConvGeom g;
+  int tiles;  // p.mTiles * column tiles
+};
+constexpr int kMaxBatch = 16;
+struct FwdBatch {
+  FwdBatchItem item[kMaxBatch];
+};
+
+template <int WM>
+__global__ void __launch_bounds__(dev::kBlock, 3)
+convFwdPaddedBatchKernel(FwdBatch b) {
+  const FwdBatchItem &it = b.item[blockIdx.z];
+  if ((int)blockIdx.x >= it.tiles || (int)blockIdx.y >= it.p.nSplit) return;
+  fwdPaddedBody<WM>(it.p, it.g);
+}
+
 // out tile = bias + sum over the nSplit partial tiles (ascending split order).
 // grid = (tail tiles, BM*BN / 1024): a workgroup folds 1024 consecutive tile elements, 4 per lane.
-__global__ void __launch_bounds__(dev::kBlock)
-fwdTailFixupKernel(FwdArgs p, ConvGeom g) {
+__device__ __forceinline__ void fwdTailFixupBody(const FwdArgs &p, const ConvGeom &g) {
   const int tileIdx = p.tile0 + blockIdx.x;
   const int mTile = tileIdx % p.mTiles, nTile = tileIdx / p.mTiles;
   const float *src = p.partial + (long)blockIdx.x * p.nSplit * (BM * BN);
@@ -746,8 +843,22 @@ fwdTailFixupKernel(FwdArgs p, ConvGeom g) {
     if (col >= p.Ncols) break;
     const int n = (int)(col / g.L);
     const int l = (int)(col - (long)n * g.L);
-    p.out[((long)n * p.M + row) * g.L + l] = vals[i];
+    const int oh = l / g.oW, ow = l - oh * g.oW;
+    p.out[(long)n * p.outImg + (long)row * p.outRow + (long)oh * p.outSH + ow * p.outSW] = vals[i];
   }
+}
+
+__global__ void __launch_bounds__(dev::kBlock)
+fwdTailFixupKernel(FwdArgs p, ConvGeom g) {
+  fwdTailFixupBody(p, g);
+}
+
+// the fold for the split items of a batch; grid = (most tiles of an item, BM*BN / 1024, items)
+__global__ void __launch_bounds__(dev::kBlock)
+fwdTailFixupBatchKernel(FwdBatch b) {
+  const FwdBatchItem &it = b.item[blockIdx.z];
+  if ((int)blockIdx.x >= it.tiles || it.p.nSplit <= 1) return;
+  fwdTailFixupBody(it.p, it.g);
 }
 
 // ---- weight gradient, second generation ------------------------------------------
@@ -1216,21 +1327,15 @@ struct FwdPlan {
   long weightFloats;   // floats of the copy of the weights with rows padded to a multiple of BK (0: not needed)
   long scratchFloats;  // tap table, tail partials, padded images
 };
-// wAligned: the weights start on a 16-byte boundary (else the padded kernel works on an aligned copy)
-FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g, bool wAligned = true) {
-  FwdPlan pl{};
-  const int nkt = launch::ceilDiv(g.K, BK);
-  const long padded = (long)nImages * g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW);
-  // K that is not a multiple of BK (first layers: Cin = 3) runs on the same kernel with the weight rows
-  // copied into rows of Kp = nkt * BK floats, zero beyond K
-  const int Kp = nkt * BK;
-  const bool fast = !forceGeneric() && padded * 4 < 0x7fffffffL && (long)M * Kp * 4 < 0x7fffffffL;
-  const bool wide = fast && tiles(M, 64) * 64 < tiles(M, BM) * BM;
+// Tiles of an M x Ncols output reduced over nkt k-tiles; wideOk: the 64 x 256 tile shape may be used.
+void planTiles(FwdPlan &pl, int M, long Ncols, int nkt, bool wideOk) {
+  const bool wide = wideOk && tiles(M, 64) * 64 < tiles(M, BM) * BM;
   pl.bm = wide ? 64 : BM, pl.bn = wide ? 256 : BN;
   pl.mTiles = (int)tiles(M, pl.bm);
-  pl.total = pl.mTiles * (int)tiles((long)nImages * g.L, pl.bn);
+  pl.total = pl.mTiles * (int)tiles(Ncols, pl.bn);
   const int cus = residentSlots(nullptr);
   int nSplit = 1;
+  pl.tail = 0;
   if (pl.total > cus) {
     pl.tail = pl.total % cus;
     if (pl.tail > 0) nSplit = std::min(nkt / 4, cus / pl.tail);  // >= 4 k-tiles per split
@@ -1246,52 +1351,32 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g, bool wAligned = t
   pl.full = pl.total - pl.tail;
   pl.ktPerSplit = launch::ceilDiv(nkt, nSplit);
   pl.nSplit = launch::ceilDiv(nkt, pl.ktPerSplit);
+}
+inline long partialFloats(const FwdPlan &pl) { return pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0; }
+
+// wAligned: the weights start on a 16-byte boundary (else the padded kernel works on an aligned copy)
+FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g, bool wAligned = true) {
+  FwdPlan pl{};
+  const int nkt = launch::ceilDiv(g.K, BK);
+  const long padded = (long)nImages * g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW);
+  // K that is not a multiple of BK (first layers: Cin = 3) runs on the same kernel with the weight rows
+  // copied into rows of Kp = nkt * BK floats, zero beyond K
+  const int Kp = nkt * BK;
+  const bool fast = !forceGeneric() && padded * 4 < 0x7fffffffL && (long)M * Kp * 4 < 0x7fffffffL;
+  planTiles(pl, M, (long)nImages * g.L, nkt, fast);
   pl.tapEntries = fast ? Kp + 2 * BK : 0;  // spare entries: the kernel reads tap offsets up to two k-tiles ahead
   pl.paddedFloats = fast && (g.padH > 0 || g.padW > 0) ? padded : 0;
   pl.weightFloats = fast && (Kp != g.K || !wAligned) ? (long)M * Kp : 0;
-  pl.scratchFloats = pl.tapEntries + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0) + (pl.paddedFloats + 3) / 4 * 4 + pl.weightFloats;
+  pl.scratchFloats = pl.tapEntries + partialFloats(pl) + (pl.paddedFloats + 3) / 4 * 4 + pl.weightFloats;
   return pl;
 }
 
-// out(nImages, M, L) = bias + W(M x K) * im2col(x); `scratch` holds plan.scratchFloats floats
-void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const float *w, const float *x, float *out,
-                       const float *bias, int M, int nImages, const ConvGeom &g) {
-  const bool fast = pl.tapEntries > 0;
-  if (fast && !(launch::aligned16(scratch) && (pl.weightFloats > 0 || launch::aligned16(w))))
-    error("SpatialConvolutionMM: internal error, convolution scratch or weights not 16-byte aligned");
-  float *partial = scratch + pl.tapEntries;
-  ConvGeom gk = g;  // geometry the kernel sees
-  FwdArgs p{};
-  p.x = x;
-  if (fast) {
-    gk.H = g.H + 2 * g.padH, gk.W = g.W + 2 * g.padW, gk.padH = gk.padW = 0;
-    float *xp = partial + (pl.tail ? (long)pl.tail * pl.nSplit * BM * BN : 0);
-    if (pl.paddedFloats > 0) {
-      launchPadPlanes(s, x, xp, (long)nImages * g.Cin, g.H, g.W, g.padH, g.padW);
-      p.x = xp;
-    }
-    buildTapTableKernel<<<launch::directGrid(pl.tapEntries, dev::kBlock), dev::kBlock, 0, s>>>(
-        reinterpret_cast<int *>(scratch), pl.tapEntries, gk);
-    THC_HIP_CHECK(hipGetLastError());
-    if (pl.weightFloats > 0) {
-      float *wp = xp + (pl.paddedFloats + 3) / 4 * 4;
-      gk.K = (int)(pl.weightFloats / M);
-      padRowsKernel<<<launch::directGrid(pl.weightFloats, dev::kBlock), dev::kBlock, 0, s>>>(w, wp, M, g.K, gk.K);
-      THC_HIP_CHECK(hipGetLastError());
-      w = wp;
-    }
-  }
-  p.taps = reinterpret_cast<const int *>(scratch);
-  p.w = w;
-  p.out = out;
-  p.bias = bias;
-  p.M = M;
-  p.Ncols = nImages * g.L;
+// The launches of one planned forward GEMM: full rounds, then the K-split tail and its fold. `p` carries the
+// operands, the output addressing, M, Ncols and the byte sizes; gk is the geometry the kernels see.
+void launchFwdKernels(hipStream_t s, const FwdPlan &pl, FwdArgs p, float *partial, const ConvGeom &gk, bool fast) {
   p.mTiles = pl.mTiles;
   p.bm = pl.bm, p.bn = pl.bn;
-  p.xBytes = (int)((long)nImages * gk.Cin * gk.H * gk.W * sizeof(float));
-  p.wBytes = (int)((long)M * gk.K * sizeof(float));
-  p.vecA = (gk.K % 4 == 0) && launch::aligned16(w);
+  p.tile0 = 0;
   p.nSplit = 1;
   p.ktPerSplit = launch::ceilDiv(gk.K, BK);
   if (pl.full > 0) {
@@ -1318,6 +1403,47 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
     fwdTailFixupKernel<<<dim3(pl.tail, BM * BN / (4 * dev::kBlock)), dev::kBlock, 0, s>>>(p, gk);
     THC_HIP_CHECK(hipGetLastError());
   }
+}
+
+// out(nImages, M, L) = bias + W(M x K) * im2col(x); `scratch` holds plan.scratchFloats floats
+void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const float *w, const float *x, float *out,
+                       const float *bias, int M, int nImages, const ConvGeom &g) {
+  const bool fast = pl.tapEntries > 0;
+  if (fast && !(launch::aligned16(scratch) && (pl.weightFloats > 0 || launch::aligned16(w))))
+    error("SpatialConvolutionMM: internal error, convolution scratch or weights not 16-byte aligned");
+  float *partial = scratch + pl.tapEntries;
+  ConvGeom gk = g;  // geometry the kernel sees
+  FwdArgs p{};
+  p.x = x;
+  if (fast) {
+    gk.H = g.H + 2 * g.padH, gk.W = g.W + 2 * g.padW, gk.padH = gk.padW = 0;
+    float *xp = partial + partialFloats(pl);
+    if (pl.paddedFloats > 0) {
+      launchPadPlanes(s, x, xp, (long)nImages * g.Cin, g.H, g.W, g.padH, g.padW);
+      p.x = xp;
+    }
+    buildTapTableKernel<<<launch::directGrid(pl.tapEntries, dev::kBlock), dev::kBlock, 0, s>>>(
+        reinterpret_cast<int *>(scratch), pl.tapEntries, gk);
+    THC_HIP_CHECK(hipGetLastError());
+    if (pl.weightFloats > 0) {
+      float *wp = xp + (pl.paddedFloats + 3) / 4 * 4;
+      gk.K = (int)(pl.weightFloats / M);
+      padRowsKernel<<<launch::directGrid(pl.weightFloats, dev::kBlock), dev::kBlock, 0, s>>>(w, wp, M, g.K, gk.K);
+      THC_HIP_CHECK(hipGetLastError());
+      w = wp;
+    }
+  }
+  p.taps = reinterpret_cast<const int *>(scratch);
+  p.w = w;
+  p.out = out;
+  p.bias = bias;
+  p.M = M;
+  p.Ncols = nImages * g.L;
+  p.outImg = (long)M * g.L, p.outRow = g.L, p.outSH = g.oW, p.outSW = 1;
+  p.xBytes = (int)((long)nImages * gk.Cin * gk.H * gk.W * sizeof(float));
+  p.wBytes = (int)((long)M * gk.K * sizeof(float));
+  p.vecA = (gk.K % 4 == 0) && launch::aligned16(w);
+  launchFwdKernels(s, pl, p, partial, gk, fast);
 }
 
 // Scratch of `floats` floats: the caller's buffer tensor (resized) or a stream-ordered temporary.
@@ -1349,11 +1475,13 @@ void convForward(THCState *state, const ConvGeom &g, const float *x, const float
   if (implicit2) group = (int)std::min<long>(group, std::max<long>(1, ((1L << 31) - 1 - 4096) / imgBytes));
   if (implicit2) {
     FwdPlan pl = planFwdImplicit(g.Cout, std::min(group, g.N), g, launch::aligned16(w));
+    long need = pl.scratchFloats;  // the last, smaller group may split differently
+    if (g.N % group != 0) need = std::max(need, planFwdImplicit(g.Cout, g.N % group, g, launch::aligned16(w)).scratchFloats);
     Temp tmp;
-    float *scratch = scratchFloats(state, scratchBuf, pl.scratchFloats, tmp, bufName);
+    float *scratch = scratchFloats(state, scratchBuf, need, tmp, bufName);
     for (int n0 = 0; n0 < g.N; n0 += group) {
       int cnt = std::min(group, g.N - n0);
-      if (cnt != std::min(group, g.N)) pl = planFwdImplicit(g.Cout, cnt, g, launch::aligned16(w));  // last, smaller group: needs no more scratch
+      if (cnt != std::min(group, g.N)) pl = planFwdImplicit(g.Cout, cnt, g, launch::aligned16(w));
       launchFwdImplicit(s, pl, scratch, w, x + (long)n0 * g.Cin * g.H * g.W, out + (long)n0 * g.Cout * g.L, bias, g.Cout,
                         cnt, g);
     }
@@ -1377,6 +1505,164 @@ void convForward(THCState *state, const ConvGeom &g, const float *x, const float
     convGemmKernel<kForward><<<grid, dev::kBlock, 0, s>>>(p, g);
     THC_HIP_CHECK(hipGetLastError());
   }
+}
+
+// Taps and gy indices of phase ph along one axis (see PhaseAxis).
+PhaseAxis phaseAxis(int ph, int size, int pad, int k, int dil, int stride) {
+  PhaseAxis a{};
+  a.n = ph < size ? (size - ph + stride - 1) / stride : 0;
+  const int d = std::gcd(dil, stride);
+  a.kStep = stride / d, a.qStep = dil / d;
+  for (int kk = 0; kk < std::min(k, a.kStep); ++kk) {  // kk * dil = ph + pad (mod stride) has period stride / d in kk
+    const int v = ph + pad - kk * dil;
+    if (((v % stride) + stride) % stride == 0) {
+      a.k0 = kk, a.nk = (k - 1 - kk) / a.kStep + 1, a.q0 = v / stride;
+      break;
+    }
+  }
+  return a;
+}
+
+// gradInput (and the transposed convolution's forward pass) for any stride, padding and dilation:
+// per phase of gi a stride-1 convolution of the zero-bordered gradOutput with the phase's sub-kernel,
+// on the forward kernels. No gradient columns reach memory and no multiply is spent on the zeros a
+// strided convolution's transpose is full of. Returns false when the geometry is outside the 32-bit
+// offsets of those kernels (the caller then takes the column path).
+bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const float *w, float *gi,
+                      THCudaTensor *scratchBuf, const char *bufName, const float *bias) {
+  if ((long)g.dH * g.dW > kMaxPhases) return false;
+  hipStream_t s = state->stream;
+  PhaseSet set{};
+  int lowH = 0, highH = g.oH - 1, lowW = 0, highW = g.oW - 1;  // gy rows / columns the phases touch
+  long wTotal = 0, tapTotal = 0, maxL = 1;
+  for (int ph = 0; ph < g.dH; ++ph)
+    for (int pw = 0; pw < g.dW; ++pw) {
+      Phase P{};
+      P.h = phaseAxis(ph, g.H, g.padH, g.kH, g.dilH, g.dH);
+      P.w = phaseAxis(pw, g.W, g.padW, g.kW, g.dilW, g.dW);
+      if (P.h.n == 0 || P.w.n == 0) continue;
+      P.h0 = ph, P.w0 = pw;
+      const long K = (long)g.Cout * P.h.nk * P.w.nk;
+      if (K >= 0x7fffffffL / 8) return false;
+      P.K = (int)K;
+      P.Kp = std::max(BK, launch::ceilDiv(P.K, BK) * BK);
+      if (P.K > 0) {
+        lowH = std::min(lowH, P.h.q0 - (P.h.nk - 1) * P.h.qStep), highH = std::max(highH, P.h.n - 1 + P.h.q0);
+        lowW = std::min(lowW, P.w.q0 - (P.w.nk - 1) * P.w.qStep), highW = std::max(highW, P.w.n - 1 + P.w.q0);
+      }
+      maxL = std::max(maxL, (long)P.h.n * P.w.n);
+      set.ph[set.count++] = P;
+    }
+  if (set.count == 0) return true;  // gi has no elements
+  // heaviest phase first: its workgroups are dispatched first
+  std::stable_sort(set.ph, set.ph + set.count, [](const Phase &a, const Phase &b) { return a.Kp > b.Kp; });
+  for (int i = 0; i < set.count; ++i) {
+    Phase &P = set.ph[i];
+    P.tapOfs = (int)tapTotal, tapTotal += P.Kp + 2 * BK;
+    P.wOfs = wTotal, wTotal += (long)g.Cin * P.Kp;
+  }
+  const int top = -lowH, left = -lowW;
+  const long Hp = (long)highH + 1 + top, Wp = (long)highW + 1 + left;
+  const long imgFloats = (long)g.Cout * Hp * Wp;
+  if (imgFloats * 4 >= (1L << 30) || wTotal * 4 >= 0x7fffffffL || tapTotal >= 0x7fffffffL / 8 ||
+      launch::ceilDiv(Hp * Wp, (long)dev::kBlock) > 65535)
+    return false;
+  const bool copy = top > 0 || left > 0 || Hp != g.oH || Wp != g.oW || !launch::aligned16(gy);
+  int group = (int)std::min<long>(g.N, std::max<long>(1, 0x7fffffffL / 2 / maxL));
+  group = (int)std::min<long>(group, std::max<long>(1, ((1L << 31) - 1 - 4096) / (imgFloats * 4)));
+
+  // All phases of a group of images run as one batched launch. The phases differ in K; the heavier ones are
+  // split along K so that a workgroup reduces about the same number of k-tiles whatever its phase and the
+  // grid holds about two workgroups per CU. Split phases leave partial tiles for the batched fold.
+  const bool wide = tiles(g.Cin, 64) * 64 < tiles(g.Cin, BM) * BM;
+  const int bm = wide ? 64 : BM, bn = wide ? 256 : BN;
+  const int mTiles = (int)tiles(g.Cin, bm);
+  struct Split {
+    int tiles, nSplit, ktPerSplit;
+    long partialOfs;
+  } split[kMaxPhases];
+  long partialTotal = 0;
+  auto planAll = [&](int cnt) {
+    long units = 0;
+    for (int i = 0; i < set.count; ++i) {
+      const Phase &P = set.ph[i];
+      split[i].tiles = mTiles * (int)tiles((long)cnt * P.h.n * P.w.n, bn);
+      units += (long)split[i].tiles * (P.Kp / BK);
+    }
+    const long target = std::max<long>(4, units / (2L * residentSlots(nullptr)));  // k-tiles per workgroup
+    long total = 0;
+    for (int i = 0; i < set.count; ++i) {
+      const int nkt = set.ph[i].Kp / BK;
+      const int n = (int)std::max<long>(1, std::min<long>(nkt / 4, (nkt + target / 2) / target));
+      split[i].ktPerSplit = launch::ceilDiv(nkt, n);
+      split[i].nSplit = launch::ceilDiv(nkt, split[i].ktPerSplit);
+      split[i].partialOfs = total;
+      if (split[i].nSplit > 1) total += (long)split[i].tiles * split[i].nSplit * BM * BN;
+    }
+    partialTotal = std::max(partialTotal, total);
+  };
+  if (g.N % group != 0) planAll(g.N % group);  // the last, smaller group may split differently
+  planAll(std::min(group, g.N));
+  const long paddedFloats = copy ? (group * imgFloats + 3) / 4 * 4 : 0;
+  Temp tmp;
+  float *buf = scratchFloats(state, scratchBuf, tapTotal + wTotal + partialTotal + paddedFloats, tmp, bufName);
+  int *taps = reinterpret_cast<int *>(buf);
+  float *wph = buf + tapTotal;
+  float *partial = wph + wTotal;
+  float *gyp = partial + partialTotal;
+  phaseTapsKernel<<<dim3(8, set.count), dev::kBlock, 0, s>>>(taps, set, (int)Hp, (int)Wp, top, left);
+  THC_HIP_CHECK(hipGetLastError());
+  phaseWeightsKernel<<<dim3(64, set.count), dev::kBlock, 0, s>>>(w, wph, set, g.Cin, g.kH, g.kW);
+  THC_HIP_CHECK(hipGetLastError());
+  for (int n0 = 0; n0 < g.N; n0 += group) {
+    const int cnt = std::min(group, g.N - n0);
+    if (cnt != std::min(group, g.N)) planAll(cnt);
+    const float *src = gy + (long)n0 * g.Cout * g.L;
+    if (copy) {
+      launchPadPlanes(s, src, gyp, (long)cnt * g.Cout, g.oH, g.oW, top, left, (int)Hp, (int)Wp);
+      src = gyp;
+    }
+    FwdBatch batch{};
+    int maxTiles = 0, maxSplit = 1;
+    for (int i = 0; i < set.count; ++i) {
+      const Phase &P = set.ph[i];
+      FwdBatchItem &it = batch.item[i];
+      ConvGeom &gk = it.g;  // what the forward kernel sees: a stride-1 pass over the bordered gy
+      gk.N = cnt, gk.Cin = g.Cout, gk.Cout = g.Cin;
+      gk.H = (int)Hp, gk.W = (int)Wp, gk.oH = P.h.n, gk.oW = P.w.n;
+      gk.kH = gk.kW = gk.dH = gk.dW = gk.dilH = gk.dilW = 1;
+      gk.K = P.Kp, gk.L = P.h.n * P.w.n;
+      FwdArgs &a = it.p;
+      a.w = wph + P.wOfs;
+      a.x = src;
+      a.taps = taps + P.tapOfs;
+      a.bias = bias;
+      a.M = g.Cin;
+      a.Ncols = cnt * gk.L;
+      a.out = gi + (long)n0 * g.Cin * g.H * g.W + (long)P.h0 * g.W + P.w0;
+      a.outImg = (long)g.Cin * g.H * g.W, a.outRow = g.H * g.W, a.outSH = g.dH * g.W, a.outSW = g.dW;
+      a.xBytes = (int)(cnt * imgFloats * 4);
+      a.wBytes = (int)((long)g.Cin * P.Kp * 4);
+      a.vecA = true;
+      a.mTiles = mTiles, a.bm = bm, a.bn = bn;
+      a.tile0 = 0;
+      a.nSplit = split[i].nSplit, a.ktPerSplit = split[i].ktPerSplit;
+      a.partial = partial + split[i].partialOfs;
+      it.tiles = split[i].tiles;
+      maxTiles = std::max(maxTiles, it.tiles), maxSplit = std::max(maxSplit, a.nSplit);
+    }
+    const dim3 grid(maxTiles, maxSplit, set.count);
+    if (wide)
+      convFwdPaddedBatchKernel<1><<<grid, dev::kBlock, 0, s>>>(batch);
+    else
+      convFwdPaddedBatchKernel<2><<<grid, dev::kBlock, 0, s>>>(batch);
+    THC_HIP_CHECK(hipGetLastError());
+    if (maxSplit > 1) {
+      fwdTailFixupBatchKernel<<<dim3(maxTiles, BM * BN / (4 * dev::kBlock), set.count), dev::kBlock, 0, s>>>(batch);
+      THC_HIP_CHECK(hipGetLastError());
+    }
+  }
+  return true;
 }
 
 // gi(N, Cin, H, W) = conv^T(gy(N, Cout, oH, oW), w(Cout, K))
@@ -1403,9 +1689,11 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
     int group = (int)std::min<long>(g.N, std::max<long>(1, 0x7fffffffL / 2 / t.L));
     group = (int)std::min<long>(group, std::max<long>(1, ((1L << 31) - 1 - 4096) / goImgBytes));
     FwdPlan pl = planFwdImplicit(t.Cout, std::min(group, g.N), t);
+    long need = pl.scratchFloats;
+    if (g.N % group != 0) need = std::max(need, planFwdImplicit(t.Cout, g.N % group, t).scratchFloats);
     const long wfFloats = ((long)g.Cout * g.K + 3) / 4 * 4;
     Temp tmp;
-    float *buf = scratchFloats(state, scratchBuf, wfFloats + pl.scratchFloats, tmp, bufName);
+    float *buf = scratchFloats(state, scratchBuf, wfFloats + need, tmp, bufName);
     flipWeightKernel<<<launch::directGrid((long)g.Cout * g.K, dev::kBlock), dev::kBlock, 0, s>>>(w, buf, g.Cout, g.Cin,
                                                                                                 g.kH, g.kW);
     THC_HIP_CHECK(hipGetLastError());
@@ -1417,6 +1705,12 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
     }
     return;
   }
+  // With few input planes the phase GEMMs would use a sliver of their 64-row tiles; the column GEMM
+  // (K rows) is the better shape then. Test switch THCUNN_CONV_GRADINPUT = "phases" / "columns" overrides.
+  const char *route = getenv("THCUNN_CONV_GRADINPUT");
+  const bool phasesPay = 2L * g.Cin >= (long)tiles(g.Cin, 64) * 64;
+  const bool tryPhases = route && !strcmp(route, "phases") ? true : route && !strcmp(route, "columns") ? false : phasesPay;
+  if (!forceGeneric() && tryPhases && gradInputByPhase(state, g, gy, w, gi, scratchBuf, bufName, bias)) return;
   // Gradient columns of a group of images at a time (<= 128 MB so the buffer stays cache resident), then
   // the col2im gather. gradCol[n][k][l] = sum_o W[o][k] * gy[n][o][l] is itself a 1x1 convolution of gy
   // with the transposed weights, so it runs on the forward kernels as well.
@@ -1436,7 +1730,9 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
     pl = planFwdImplicit(q.Cout, std::min(group, g.N), q);
     wtFloats = ((long)g.Cout * g.K + 3) / 4 * 4;
   }
-  const long fwdFloats = (pl.scratchFloats + 3) / 4 * 4;
+  long need = pl.scratchFloats;
+  if (viaForward && g.N % group != 0) need = std::max(need, planFwdImplicit(q.Cout, g.N % group, q).scratchFloats);
+  const long fwdFloats = (need + 3) / 4 * 4;
   Temp tmp;
   float *buf = scratchFloats(state, scratchBuf, wtFloats + fwdFloats + (long)group * perImg, tmp, bufName);
   float *gcol = buf + wtFloats + fwdFloats;

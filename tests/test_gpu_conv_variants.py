@@ -203,3 +203,36 @@ TILE_CASES = [
 @pytest.mark.parametrize("case", TILE_CASES)
 def test_convolution_tile_shapes(T, case):
     _dil_run(T, case)
+
+
+# gradInput (and the transposed convolution's forward pass) has two routes for geometries the flipped-weight
+# forward kernel does not cover: one stride-1 GEMM per output phase (taken when Cin fills at least half of a
+# 64-row tile) and gradient columns + col2im. Both are run on every geometry through the test switch.
+PHASE_DIL_CASES = [c for c in DIL_CASES if c[7] != 1 or c[8] != 1 or c[9] > c[11] * (c[5] - 1)] + [
+    (3, 64, 48, 23, 27, 3, 3, 2, 2, 1, 1, 1, 1),     # ResNet-style downsampling, odd extents
+    (2, 40, 24, 17, 19, 5, 4, 3, 2, 2, 1, 1, 2),     # stride 3 x 2, rectangular, dilated rows
+    (2, 33, 16, 16, 16, 1, 1, 2, 2, 0, 0, 1, 1),     # 1x1 stride 2: three of four phases have no tap at all
+    (2, 32, 16, 15, 15, 2, 2, 4, 4, 0, 0, 1, 1),     # kernel smaller than the stride
+    (2, 36, 20, 20, 21, 3, 3, 2, 2, 1, 1, 2, 2),     # stride 2 with dilation 2: only one phase per axis has taps
+    (6, 128, 160, 14, 14, 3, 3, 2, 2, 1, 1, 1, 1),   # 128-row tiles, phases split along K
+]
+
+
+@pytest.mark.parametrize("route", ["phases", "columns"])
+@pytest.mark.parametrize("case", PHASE_DIL_CASES)
+def test_gradinput_routes(T, case, route):
+    os.environ["THCUNN_CONV_GRADINPUT"] = route
+    try:
+        _dil_run(T, case, seed=83)
+    finally:
+        os.environ.pop("THCUNN_CONV_GRADINPUT", None)
+
+
+@pytest.mark.parametrize("route", ["phases", "columns"])
+@pytest.mark.parametrize("case", FULL_CASES + [(2, 24, 64, 9, 11, 4, 4, 2, 2, 1, 1, 1, 1, 0, 1)])
+def test_full_convolution_routes(T, case, route):
+    os.environ["THCUNN_CONV_GRADINPUT"] = route
+    try:
+        _full_run(T, case, seed=92)
+    finally:
+        os.environ.pop("THCUNN_CONV_GRADINPUT", None)

@@ -470,11 +470,14 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds):
         wall = time.perf_counter() - t0
         return wall, {n: [hip.elapsed_ms(a, b) for a, b in ev[n]] for n in bracket}
 
-    # warm-up: a few plain steps, then the rest instrumented per entry point - that finds the
-    # dominant kernel and times the others
+    # warm-up: a few plain steps, then the rest instrumented one entry point at a time (events around
+    # neighbouring launches would add their own few microseconds to each other's bracket) - that finds
+    # the dominant kernel and times the others
     plain = max(1, warmup // 4)
     timed(plain, [])
-    _, per_kernel = timed(max(warmup - plain, 1), names)
+    per_kernel = {}
+    for n in names:
+        per_kernel.update(timed(max((warmup - plain) // len(names), 1), [n])[1])
     dominant = max(names, key=lambda n: float(np.mean(per_kernel[n])))
     # the timed region: exactly `steps` steps; only the dominant kernel is bracketed by events,
     # so the measurement perturbs the step as little as possible

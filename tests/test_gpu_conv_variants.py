@@ -236,3 +236,32 @@ def test_full_convolution_routes(T, case, route):
         _full_run(T, case, seed=92)
     finally:
         os.environ.pop("THCUNN_CONV_GRADINPUT", None)
+
+
+def _random_geometry(rng):
+    while True:
+        Cin = int(rng.choice([3, 17, 32, 48, 70, 130]))
+        Cout = int(rng.choice([5, 33, 64, 100, 140]))
+        kW, kH = (int(v) for v in rng.integers(1, 6, 2))
+        dW, dH = (int(v) for v in rng.integers(1, 4, 2))
+        pW, pH = (int(v) for v in rng.integers(0, 3, 2))
+        dlW, dlH = (int(v) for v in rng.integers(1, 3, 2))
+        H, W = (int(v) for v in rng.integers(6, 25, 2))
+        if H + 2 * pH >= dlH * (kH - 1) + 1 and W + 2 * pW >= dlW * (kW - 1) + 1:
+            return (int(rng.integers(1, 4)), Cin, Cout, H, W, kW, kH, dW, dH, pW, pH, dlW, dlH)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_convolution_random_geometries(T, seed):
+    """Seeded draws over kernel size, stride, padding, dilation and channel counts on either side of the
+    tile-shape and gradInput-route thresholds; the gradInput route alternates between the default choice,
+    the phase route and the column route."""
+    rng = np.random.default_rng(1000 + seed)
+    case = _random_geometry(rng)
+    route = [None, "phases", "columns"][seed % 3]
+    if route:
+        os.environ["THCUNN_CONV_GRADINPUT"] = route
+    try:
+        _dil_run(T, case, seed=2000 + seed, scale=float(rng.choice([1.0, 0.5])))
+    finally:
+        os.environ.pop("THCUNN_CONV_GRADINPUT", None)

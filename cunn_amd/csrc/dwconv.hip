@@ -69,6 +69,7 @@ __device__ __forceinline__ void loadTaps(const float *__restrict__ weight, const
   }
 }
 
+#include "dwconv_small.h"
 
 // ------------------------------------------------------------------ forward --
 // KS/ST > 0: square kernel / stride known at compile time (taps in registers,
@@ -771,6 +772,71 @@ int gradInputExtraRows(int ks, int st) {
   return dev::TapSpan<5, 2, 2, 2>::hi() - dev::TapSpan<5, 2, 2, 2>::lo();
 }
 
+// ---- small planes: several planes per workgroup (dwconv_small.h) ----------------------------
+enum SmallPass { kSmallFwd, kSmallGradInput, kSmallAccGrad };
+
+// Test switch THCUNN_DW_SMALL: "0" never, "1" whenever the geometry allows; default: planes the strip
+// kernels cannot take (width or output width not a multiple of 4) and planes of at most 256 elements.
+int smallSwitch() {
+  const char *e = getenv("THCUNN_DW_SMALL");
+  return e ? atoi(e) : -1;
+}
+
+// Plans a small-plane launch; false when the geometry is outside what those kernels are compiled for.
+bool smallPlan(const DwGeom &g, SmallPass pass, SmallGeom *out, int *rw, size_t *lds) {
+  const bool sq = g.kH == g.kW && g.dH == g.dW && g.padH == g.padW;
+  if (forcedPath() != 0 || smallSwitch() == 0 || !sq || g.M != 1 || (g.kH != 3 && g.kH != 5) || (g.dH != 1 && g.dH != 2) ||
+      g.padH != g.kH / 2)
+    return false;
+  const int HW = g.H * g.W, oHW = g.oH * g.oW;
+  if (HW > 1024 || oHW < 1) return false;
+  if (smallSwitch() != 1 && stripGeometry(g) && HW > 256) return false;
+  const int PAD = g.kH / 2;
+  SmallGeom sg{};
+  sg.C = g.C, sg.planes = g.N * g.C;
+  if (pass == kSmallGradInput)
+    sg.sH = g.oH, sg.sW = g.oW, sg.oH = g.H, sg.oW = g.W;
+  else
+    sg.sH = g.H, sg.sW = g.W, sg.oH = g.oH, sg.oW = g.oW;
+  sg.LH = g.H + 2 * PAD, sg.LW = g.W + 2 * PAD;
+  const int second = pass == kSmallGradInput ? HW : oHW;  // output run (forward, gradInput) / gradOutput run (accGrad)
+  auto xsFloats = [&](int P) { return roundUp(P * sg.LH * sg.LW + 7 * 2 + g.kH, 4); };  // slack: the widest item's overrun
+  int P = 64;  // at least 4: the lanes of a plane stay inside one wave
+  while (P > 4 && (P * HW > launch::kBatchFloats || (size_t)(xsFloats(P) + P * second) * sizeof(float) > launch::kLdsMax)) P >>= 1;
+  if (P * HW > launch::kBatchFloats || (size_t)(xsFloats(P) + P * second) * sizeof(float) > launch::kLdsMax) return false;
+  if ((P * HW) % 4 != 0 || (P * oHW) % 4 != 0) return false;  // every workgroup's runs start on 16 bytes
+  sg.P = P, sg.lp = dev::kBlock / P;
+  for (sg.lpShift = 0; (1 << sg.lpShift) < sg.lp; ++sg.lpShift) {
+  }
+  sg.xsFloats = xsFloats(P);
+  // outputs per work item: 7 or 4 consecutive ones of a row, whichever needs fewer lane-steps for a plane
+  // (rounds over the plane's lanes x (outputs + the window's extra columns))
+  auto steps = [&](int r) { return ceilDiv(sg.oH * ceilDiv(sg.oW, r), sg.lp) * (r + 2); };
+  *rw = steps(7) <= steps(4) ? 7 : 4;
+  sg.nseg = ceilDiv(sg.oW, *rw);
+  sg.magicC = dev::magicOf(g.C), sg.magicSPlane = dev::magicOf(sg.sH * sg.sW), sg.magicSW = dev::magicOf(sg.sW);
+  sg.magicSeg = dev::magicOf(sg.nseg);
+  *out = sg;
+  *lds = (size_t)(sg.xsFloats + P * second) * sizeof(float);
+  return true;
+}
+
+#define DW_SMALL_CONV(CS, DS, FLIP, ...)                                                                          \
+  do {                                                                                                            \
+    if (g.kH == 3 && rw == 4) dwSmallConv<3, CS, DS, FLIP, 4><<<grid, dev::kBlock, lds, s>>>(__VA_ARGS__);        \
+    if (g.kH == 3 && rw == 7) dwSmallConv<3, CS, DS, FLIP, 7><<<grid, dev::kBlock, lds, s>>>(__VA_ARGS__);        \
+    if (g.kH == 5 && rw == 4) dwSmallConv<5, CS, DS, FLIP, 4><<<grid, dev::kBlock, lds, s>>>(__VA_ARGS__);        \
+    if (g.kH == 5 && rw == 7) dwSmallConv<5, CS, DS, FLIP, 7><<<grid, dev::kBlock, lds, s>>>(__VA_ARGS__);        \
+  } while (0)
+
+#define DW_SMALL_ACC(ST, ...)                                                                                     \
+  do {                                                                                                            \
+    if (g.kH == 3 && rw == 4) dwSmallAccGrad<3, ST, 4><<<grid, dev::kBlock, lds, s>>>(__VA_ARGS__);               \
+    if (g.kH == 3 && rw == 7) dwSmallAccGrad<3, ST, 7><<<grid, dev::kBlock, lds, s>>>(__VA_ARGS__);               \
+    if (g.kH == 5 && rw == 4) dwSmallAccGrad<5, ST, 4><<<grid, dev::kBlock, lds, s>>>(__VA_ARGS__);               \
+    if (g.kH == 5 && rw == 7) dwSmallAccGrad<5, ST, 7><<<grid, dev::kBlock, lds, s>>>(__VA_ARGS__);               \
+  } while (0)
+
 }  // namespace
 
 extern "C" {
@@ -796,6 +862,20 @@ void THNN_CudaSpatialDepthWiseConvolution_updateOutput(THCState *state, THCudaTe
   if (planes == 0) return;
   const float *bptr = bias ? data(bias) : nullptr;
 
+  {
+    SmallGeom sg;
+    int rw;
+    size_t lds;
+    if (aligned16(in.ptr()) && aligned16(data(output)) && smallPlan(g, kSmallFwd, &sg, &rw, &lds)) {
+      const dim3 grid(ceilDiv(sg.planes, sg.P));
+      if (g.dH == 1)
+        DW_SMALL_CONV(1, 1, false, in.ptr(), data(weight), strides4(weight), bptr, strides2(bias), data(output), sg);
+      else
+        DW_SMALL_CONV(2, 1, false, in.ptr(), data(weight), strides4(weight), bptr, strides2(bias), data(output), sg);
+      THC_HIP_CHECK(hipGetLastError());
+      return;
+    }
+  }
   bool vec = (g.W % 4 == 0) && aligned16(in.ptr());
   g.padL = vec ? roundUp(g.padW, 4) : g.padW;
   g.pitch = g.W + g.padL;
@@ -857,6 +937,21 @@ void THNN_CudaSpatialDepthWiseConvolution_updateGradInput(THCState *state, THCud
   const long planes = (long)g.N * g.C;
   if (planes == 0) return;
 
+  {
+    SmallGeom sg;
+    int rw;
+    size_t lds;
+    if (aligned16(go.ptr()) && aligned16(data(gradInput)) && smallPlan(g, kSmallGradInput, &sg, &rw, &lds)) {
+      const dim3 grid(ceilDiv(sg.planes, sg.P));
+      const Strides2 nob{0, 0};
+      if (g.dH == 1)
+        DW_SMALL_CONV(1, 1, true, go.ptr(), data(weight), strides4(weight), nullptr, nob, data(gradInput), sg);
+      else
+        DW_SMALL_CONV(1, 2, true, go.ptr(), data(weight), strides4(weight), nullptr, nob, data(gradInput), sg);
+      THC_HIP_CHECK(hipGetLastError());
+      return;
+    }
+  }
   // a band of `rows` gradInput rows is reached by at most (rows + kH - 2) / dH + 2 gradOutput rows
   bool vec = (g.oW % 4 == 0) && aligned16(go.ptr());
   auto ohRows = [&](int rows) { return std::min(g.oH, (rows + g.kH - 2) / g.dH + 2); };
@@ -918,6 +1013,36 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
   if (planes == 0) return;
   float *gbPtr = gradBias ? data(gradBias) : nullptr;
 
+  {
+    SmallGeom sg;
+    int rw;
+    size_t lds;
+    if (aligned16(in.ptr()) && aligned16(go.ptr()) && smallPlan(g, kSmallAccGrad, &sg, &rw, &lds)) {
+      const int T = g.kH * g.kW + 1;
+      // one partial per (channel, tap, image); scratch as in the general case below
+      Temp tmp;
+      float *partial;
+      if (columns) {
+        resize(state, columns, {(long)g.C * T, g.N});
+        if (!isContiguous(erase(columns))) error("columns tensor has to be contiguous");
+        partial = data(columns);
+      } else {
+        tmp = Temp(s, (size_t)g.C * T * g.N * sizeof(float));
+        partial = (float *)tmp.get();
+      }
+      const dim3 grid(ceilDiv(sg.planes, sg.P));
+      if (g.dH == 1)
+        DW_SMALL_ACC(1, in.ptr(), go.ptr(), partial, sg, g.N);
+      else
+        DW_SMALL_ACC(2, in.ptr(), go.ptr(), partial, sg, g.N);
+      THC_HIP_CHECK(hipGetLastError());
+      const int pairs = g.C * T;
+      dwAccGradStage2<<<ceilDiv(pairs, dev::kBlock / dev::kWave), dev::kBlock, 0, s>>>(
+          partial, data(gradWeight), strides4(gradWeight), gbPtr, strides2(gradBias), 1, g.kW, T, g.N, scale, pairs);
+      THC_HIP_CHECK(hipGetLastError());
+      return;
+    }
+  }
   bool sq = g.kH == g.kW && g.dH == g.dW;
   int ks = sq ? g.kH : 0, st = sq ? g.dH : 0;
   bool haveKernel = (ks == 3 || ks == 5) && (st == 1 || st == 2);

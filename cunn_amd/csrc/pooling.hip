@@ -403,6 +403,38 @@ avgPoolFwdStrip(const float *__restrict__ in, float *__restrict__ out, PoolGeom 
   }
 }
 
+// Global average pooling (one window = the whole plane, no padding; the last layer of most
+// classification networks, with planes of 49 elements). Forward: a wave sums one plane at a time,
+// four planes in flight, lanes over the plane's elements in memory order. Backward: a lane writes
+// elements of gradInput in memory order, each the plane's gradOutput over the plane size.
+__global__ void __launch_bounds__(dev::kBlock)
+avgPoolGlobalFwd(const float *__restrict__ in, float *__restrict__ out, long planes, int S) {
+  const int lane = threadIdx.x % dev::kWave;
+  const long nWaves = (long)gridDim.x * (dev::kBlock / dev::kWave);
+  const float div = (float)S;
+  for (long q = ((long)blockIdx.x * (dev::kBlock / dev::kWave) + threadIdx.x / dev::kWave) * 4; q < planes; q += nWaves * 4) {
+    float a[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int i = lane; i < S; i += dev::kWave) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) a[u] += q + u < planes ? in[(q + u) * S + i] : 0.f;
+    }
+    float r = 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float v = dev::waveSum(a[u]);
+      if (lane == u) r = v;
+    }
+    if (lane < 4 && q + lane < planes) out[q + lane] = r / div;
+  }
+}
+
+__global__ void __launch_bounds__(dev::kBlock)
+avgPoolGlobalBwd(const float *__restrict__ gradOut, float *__restrict__ gradIn, unsigned total, int S, unsigned magicS) {
+  const float div = (float)S;
+  for (unsigned e = blockIdx.x * dev::kBlock + threadIdx.x; e < total; e += gridDim.x * dev::kBlock)
+    gradIn[e] = gradOut[dev::fastDiv((int)e, magicS)] / div;
+}
+
 // Non-overlapping average pooling (window = stride = KS, no padding, H = KS*oH, W = KS*oW): no
 // input element is shared between windows, so nothing is staged. With these extents the planes
 // of the batch form one tall image of planes*oH output rows; a lane owns 4 consecutive outputs
@@ -587,6 +619,12 @@ bool avgFlatOk(const PoolGeom &g, long planes) {
   const long total = planes * g.oH * (g.oW / 4);
   return forcedPath() == 0 && sq && g.kH >= 2 && g.kH <= 4 && g.H == g.oH * g.kH && g.W == g.oW * g.kW && g.oW % 4 == 0 &&
          total > 0 && total * (g.oW / 4) < 0xffffffffL && total < 0x7fffffffL;
+}
+
+// One window that is exactly the plane; total elements small enough for the reciprocal division.
+bool avgGlobalOk(const PoolGeom &g, long planes) {
+  return forcedPath() == 0 && g.oH == 1 && g.oW == 1 && g.padH == 0 && g.padW == 0 && g.kH == g.H && g.kW == g.W &&
+         planes * g.H * g.W < 0x7fffffffL && planes * g.H * g.W * ((long)g.H * g.W) < 0xffffffffL;
 }
 
 bool stripFwdOk(const PoolGeom &g) {
@@ -865,7 +903,10 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
     auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.W * sizeof(float); };
     auto sbytes = [&](int rows) { return fwdStripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
     auto staged = [&](int rows) { return (size_t)((rows - 1) * g.dH + g.kH) * g.W; };
-    if (avgFlatOk(g, planes) && vec && aligned16(data(output))) {
+    if (avgGlobalOk(g, planes)) {
+      const long waves = std::min<long>((planes + 3) / 4, 8192);
+      avgPoolGlobalFwd<<<(unsigned)((waves + 3) / 4), dev::kBlock, 0, s>>>(in.ptr(), data(output), planes, g.H * g.W);
+    } else if (avgFlatOk(g, planes) && vec && aligned16(data(output))) {
       const unsigned total = (unsigned)(planes * g.oH * (g.oW / 4));
       const unsigned grid = (total + dev::kBlock - 1) / dev::kBlock;
       const unsigned magic = dev::magicOf(g.oW / 4);
@@ -942,7 +983,11 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
   const int spitch = g.oW + dev::kStripPadL;
   auto sbytes = [&](int units) { return ((size_t)(units + extra) * spitch + dev::kStripPadL) * sizeof(float); };
   int units = 0;
-  if (avgFlatOk(g, planes) && vec && aligned16(data(gradInput)) && planes * g.H * (g.W / 4) * (g.W / 4) < 0xffffffffL) {
+  if (avgGlobalOk(g, planes)) {
+    const unsigned total = (unsigned)(planes * g.H * g.W);
+    avgPoolGlobalBwd<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), total,
+                                                                                    g.H * g.W, dev::magicOf(g.H * g.W));
+  } else if (avgFlatOk(g, planes) && vec && aligned16(data(gradInput)) && planes * g.H * (g.W / 4) * (g.W / 4) < 0xffffffffL) {
     const unsigned total = (unsigned)(planes * g.H * (g.W / 4));
     const unsigned grid = (total + dev::kBlock - 1) / dev::kBlock;
     const unsigned magic = dev::magicOf(g.W / 4);

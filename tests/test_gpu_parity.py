@@ -118,6 +118,69 @@ def test_dwconv_fallback_kernels(T, case, mode):
         _dw_run(T, case, x, w, b)
 
 
+DW_SMALL_CASES = [
+    # planes of at most 1024 elements with depth multiplier 1: several planes per workgroup
+    (4, 40, 1, 14, 14, 3, 3, 1, 1, 1, 1),    # MobileNet 14x14 stage: 16 planes per workgroup, 7 outputs per item
+    (4, 40, 1, 14, 14, 3, 3, 2, 2, 1, 1),    # 14 -> 7
+    (3, 70, 1, 7, 7, 3, 3, 1, 1, 1, 1),      # 7x7: 64 planes per workgroup, last workgroup partly filled
+    (2, 24, 1, 28, 28, 3, 3, 2, 2, 1, 1),    # 28 -> 14: width fits the strip kernels, output width does not
+    (3, 10, 1, 28, 28, 5, 5, 2, 2, 2, 2),    # 5x5
+    (2, 12, 1, 14, 14, 5, 5, 1, 1, 2, 2),
+    (3, 5, 1, 13, 11, 3, 3, 1, 1, 1, 1),     # odd extents: 4 outputs per item with a masked tail
+    (2, 6, 1, 15, 18, 3, 3, 2, 2, 1, 1),     # odd height under stride 2: the last input row is never read
+    (1, 3, 1, 5, 5, 3, 3, 2, 2, 1, 1),       # three planes in all: one workgroup, mostly idle
+    (5, 16, 1, 31, 31, 3, 3, 2, 2, 1, 1),    # 961 elements: 4 planes per workgroup
+    (2, 8, 1, 9, 9, 5, 5, 2, 2, 2, 2),
+    (1, 4, 1, 2, 2, 3, 3, 1, 1, 1, 1),       # plane smaller than the kernel
+]
+
+
+@pytest.mark.parametrize("case", DW_SMALL_CASES)
+def test_dwconv_small_planes(T, case):
+    rng, x, w, b = _dw_inputs(case, 11)
+    _dw_run(T, case, x, w, b, scale=0.5, gw0=rng.standard_normal(w.shape).astype(np.float32),
+            gb0=rng.standard_normal((case[2], case[1])).astype(np.float32))
+
+
+@pytest.mark.parametrize("case", [DW_CASES[0][:2] + (1,) + DW_CASES[0][3:], (2, 6, 1, 16, 16, 3, 3, 1, 1, 1, 1),
+                                  (2, 6, 1, 32, 32, 3, 3, 2, 2, 1, 1), (2, 6, 1, 24, 32, 5, 5, 1, 1, 2, 2)])
+@pytest.mark.parametrize("switch", ["0", "1"])
+def test_dwconv_small_planes_switch(T, case, switch):
+    """Shapes both kernel families take: the switch forces the small-plane kernels on or off."""
+    _, x, w, b = _dw_inputs(case, 12)
+    with force_direct("THCUNN_DW_SMALL", switch):
+        _dw_run(T, case, x, w, b)
+
+
+def test_dwconv_small_planes_special_values(T):
+    """A work item whose last outputs are masked off (width 6, 4 outputs per item) reads past the end of its row;
+    what it finds there - here an infinity in column 0 of the next row - must not reach any sum."""
+    case = (2, 8, 1, 6, 6, 3, 3, 1, 1, 1, 1)
+    _, x, w, b = _dw_inputs(case, 13)
+    x[0, 3, 2, 0] = np.inf
+    THNN, CT = T.THNN, T.CudaTensor
+    out = CT()
+    THNN.SpatialDepthWiseConvolution_updateOutput(CT.from_numpy(x), out, CT.from_numpy(w), CT.from_numpy(b), CT(), CT(),
+                                                  3, 3, 1, 1, 1, 1)
+    y = out.numpy()
+    with np.errstate(invalid="ignore"):
+        ry = O.dwconv_updateOutput(x, w, b, 3, 3, 1, 1, 1, 1)
+    assert np.array_equal(np.isfinite(y), np.isfinite(ry))
+    close(y[np.isfinite(ry)], ry[np.isfinite(ry)])
+    gy = np.random.default_rng(14).standard_normal(y.shape).astype(np.float32)
+    gw, gb = CT.from_numpy(np.zeros_like(w)), CT.from_numpy(np.zeros_like(b))
+    THNN.SpatialDepthWiseConvolution_accGradParameters(CT.from_numpy(x), CT.from_numpy(gy), gw, gb, CT(), CT(),
+                                                       3, 3, 1, 1, 1, 1, 1.0)
+    with np.errstate(invalid="ignore"):
+        rgw, rgb = O.dwconv_accGradParameters(x, gy, np.zeros_like(w), np.zeros_like(b), 3, 3, 1, 1, 1, 1, 1.0)
+    g = gw.numpy()
+    fin = np.isfinite(rgw)
+    assert fin[0, 3, :, 2].all() and not fin[0, 3, :, 0].all()   # column 0 of the input never meets tap column 2
+    assert np.array_equal(np.isfinite(g), fin)
+    close(g[fin], rgw[fin], WG_RTOL, WG_ATOL)
+    close(gb.numpy(), rgb, WG_RTOL, WG_ATOL)
+
+
 def test_dwconv_accgrad_deterministic(T):
     """accGradParameters folds per-workgroup partials in a fixed order (no atomics): repeated
     calls on the same inputs are bit-identical."""
@@ -336,6 +399,19 @@ def test_avgpool_direct_and_noncontiguous(T, case):
             _avgpool_run(T, case, False)
     rng = np.random.default_rng(31)
     _avgpool_run(T, case, True, xt=lambda a: T.CudaTensor.noncontiguous_from_numpy(a, rng))
+
+
+@pytest.mark.parametrize("case", [
+    (5, 37, 7, 7, 7, 7, 1, 1, 0, 0, False),      # global pooling of a 7x7 plane; plane count not a multiple of 4
+    (2, 3, 13, 9, 9, 13, 1, 1, 0, 0, True),      # rectangular plane of more than 64 elements, ceil mode
+    (1, 1, 1, 1, 1, 1, 1, 1, 0, 0, False),       # a single element
+    (3, 6, 8, 8, 8, 8, 8, 8, 0, 0, False),       # stride = window
+])
+@pytest.mark.parametrize("include_pad", [True, False])
+def test_avgpool_global(T, case, include_pad):
+    _avgpool_run(T, case, include_pad, seed=33)
+    with force_direct("THCUNN_POOL_FORCE_DIRECT", "2"):
+        _avgpool_run(T, case, include_pad, seed=33)
 
 
 def test_avgpool_reference_known_answer(T):

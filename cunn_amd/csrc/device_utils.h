@@ -34,6 +34,24 @@ __device__ __forceinline__ float waveSum(float v) {
   return (r0 + r1) + (r2 + r3);
 }
 
+// Sum over each aligned group of `lanes` lanes (4, 8, 16, 32 or 64; wave-uniform), returned in
+// every lane of the group; the same DPP steps as waveSum, stopped where the group is complete.
+__device__ __forceinline__ float groupSum(float v, int lanes) {
+  v = dppAdd<0xB1>(v);
+  v = dppAdd<0x4E>(v);
+  if (lanes >= 8) v = dppAdd<0x141>(v);
+  if (lanes >= 16) v = dppAdd<0x140>(v);
+  if (lanes >= 32) {
+    const int b = __builtin_bit_cast(int, v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    v = lanes >= 64 ? (r0 + r1) + (r2 + r3) : ((threadIdx.x & 32) ? r2 + r3 : r0 + r1);
+  }
+  return v;
+}
+
 // Workgroups are handed to the XCDs round-robin (block b runs on XCD b % 8).
 // Remapping so that each XCD works on one contiguous range of logical tiles
 // keeps the tiles that share halo rows (and the planes that are neighbours in

@@ -522,7 +522,7 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
   constexpr int T = KS * KS + 1;
   constexpr int nWaves = dev::kBlock / dev::kWave;
   extern __shared__ float smem[];
-  __shared__ float red[nWaves][T];
+  __shared__ float red[nWaves * 4][T];  // one sum per row of 16 lanes
   const BlockPos bp = blockPos(g);
   const int plane = bp.plane, tile = bp.tile, c = bp.c;
   const int n = dev::fastDiv(plane, g.magicC);
@@ -578,16 +578,17 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
       }
       acc[T - 1] += (gy[0] + gy[1]) + (gy[2] + gy[3]);
     }
+    // rows of 16 lanes are folded on the VALU (4 DPP steps per sum), the 16 row sums of the workgroup through LDS
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-      float v = dev::waveSum(acc[t]);
-      if (lane == 0) red[wave][t] = v;
+      const float v = dev::groupSum(acc[t], 16);
+      if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][t] = v;
     }
     __syncthreads();
     if (threadIdx.x < T) {
       float v = 0.f;
 #pragma unroll
-      for (int w = 0; w < nWaves; ++w) v += red[w][threadIdx.x];
+      for (int w = 0; w < nWaves * 4; ++w) v += red[w][threadIdx.x];
       partial[(((long)c * nMul + j) * T + threadIdx.x) * g.nslots + slot] = v;
     }
   }
@@ -775,8 +776,8 @@ int gradInputExtraRows(int ks, int st) {
 // ---- small planes: several planes per workgroup (dwconv_small.h) ----------------------------
 enum SmallPass { kSmallFwd, kSmallGradInput, kSmallAccGrad };
 
-// Test switch THCUNN_DW_SMALL: "0" never, "1" whenever the geometry allows; default: planes the strip
-// kernels cannot take (width or output width not a multiple of 4) and planes of at most 256 elements.
+// Planes of at most 1024 elements take these kernels (measured faster than the strip kernels up to 28x28, and
+// the strip kernels need widths that are multiples of 4). Test switch THCUNN_DW_SMALL=0: never.
 int smallSwitch() {
   const char *e = getenv("THCUNN_DW_SMALL");
   return e ? atoi(e) : -1;
@@ -790,7 +791,6 @@ bool smallPlan(const DwGeom &g, SmallPass pass, SmallGeom *out, int *rw, size_t 
     return false;
   const int HW = g.H * g.W, oHW = g.oH * g.oW;
   if (HW > 1024 || oHW < 1) return false;
-  if (smallSwitch() != 1 && stripGeometry(g) && HW > 256) return false;
   const int PAD = g.kH / 2;
   SmallGeom sg{};
   sg.C = g.C, sg.planes = g.N * g.C;
@@ -798,7 +798,7 @@ bool smallPlan(const DwGeom &g, SmallPass pass, SmallGeom *out, int *rw, size_t 
     sg.sH = g.oH, sg.sW = g.oW, sg.oH = g.H, sg.oW = g.W;
   else
     sg.sH = g.H, sg.sW = g.W, sg.oH = g.oH, sg.oW = g.oW;
-  sg.LH = g.H + 2 * PAD, sg.LW = g.W + 2 * PAD;
+  sg.LH = g.H + 2 * PAD, sg.LW = (g.W + 2 * PAD) | 1;  // odd pitch: the rows a wave reads start in different banks
   const int second = pass == kSmallGradInput ? HW : oHW;  // output run (forward, gradInput) / gradOutput run (accGrad)
   auto xsFloats = [&](int P) { return roundUp(P * sg.LH * sg.LW + 7 * 2 + g.kH, 4); };  // slack: the widest item's overrun
   int P = 64;  // at least 4: the lanes of a plane stay inside one wave
@@ -1057,7 +1057,10 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
     return (band + (size_t)rows * g.oW) * sizeof(float);
   };
   auto staged = [&](int rows) { return useStrip ? (size_t)((rows - 1) * g.dH + g.kH) * g.W : (size_t)0; };
-  if (haveKernel && !forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane, staged)) {
+  // Two bands are staged here (input and gradOutput), and every workgroup pays a fixed reduction epilogue: a
+  // budget of 34 KB (4 workgroups per CU) keeps a one-batch input band and its gradOutput rows in one workgroup.
+  if (haveKernel && !forceDirect() &&
+      launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane, staged, useStrip ? 34 * 1024 : launch::kLdsBudget)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
     g.nslots = g.N * g.tilesPerPlane;
     size_t lds = bytes(g.tileRows);

@@ -16,12 +16,14 @@
 // one channel in registers. Depth multiplier 1, square kernel 3 or 5, stride 1 or 2, padding k / 2.
 #pragma once
 
+#include <type_traits>
+
 struct SmallGeom {
   int C, planes;          // channels, N * C
   int P, lp, lpShift;     // planes per workgroup, lanes per plane (kBlock / P), log2(lp)
   int sH, sW;             // plane of the tensor that is read and staged
   int oH, oW;             // plane of the tensor that is produced (accGrad: gradOutput, read linear)
-  int LH, LW;             // staged plane in LDS (zero border included); LW is the row pitch
+  int LH, LW;             // staged plane in LDS (zero border included); LW is the row pitch (odd, >= the bordered width)
   int xsFloats;           // floats of the P staged planes incl. slack, a multiple of 4
   int nseg;               // segments of RW outputs per row
   unsigned magicC, magicSPlane, magicSW, magicSeg;
@@ -191,12 +193,14 @@ dwSmallAccGrad(const float *__restrict__ in, const float *__restrict__ gradOut, 
     const float *xp = xs + pl * (g.LH * g.LW);
     const float *gp = gs + pl * oPlane;
     const int items = g.oH * g.nseg;
-    for (int it = it0; it < items; it += g.lp) {
-      const int r = dev::fastDiv(it, g.magicSeg), c0 = (it - r * g.nseg) * RW;
+    // an item whose outputs all exist needs no masking; the last item of a row may (MASK): a masked output
+    // must not multiply whatever lies past the row, which may not be finite
+    auto item = [&](auto masked, int r, int c0) {
+      constexpr bool MASK = decltype(masked)::value;
       float gv[RW];
 #pragma unroll
       for (int q = 0; q < RW; ++q) {
-        gv[q] = c0 + q < g.oW ? gp[r * g.oW + min(c0 + q, g.oW - 1)] : 0.f;
+        gv[q] = !MASK || c0 + q < g.oW ? gp[r * g.oW + (MASK ? min(c0 + q, g.oW - 1) : c0 + q)] : 0.f;
         acc[T - 1] += gv[q];
       }
 #pragma unroll
@@ -207,18 +211,23 @@ dwSmallAccGrad(const float *__restrict__ in, const float *__restrict__ gradOut, 
         for (int j = 0; j < NWIN; ++j) win[j] = row[j];
 #pragma unroll
         for (int q = 0; q < RW; ++q) {
-          const bool ok = c0 + q < g.oW;  // a masked output must not multiply whatever lies past the row
+          const bool ok = !MASK || c0 + q < g.oW;
 #pragma unroll
           for (int kw = 0; kw < KS; ++kw) acc[kh * KS + kw] = fmaf(gv[q], ok ? win[q * ST + kw] : 0.f, acc[kh * KS + kw]);
         }
       }
+    };
+    for (int it = it0; it < items; it += g.lp) {
+      const int r = dev::fastDiv(it, g.magicSeg), c0 = (it - r * g.nseg) * RW;
+      if (c0 + RW <= g.oW)
+        item(std::false_type{}, r, c0);
+      else
+        item(std::true_type{}, r, c0);
     }
   }
-  // fold over the lanes of the plane (lp is a power of two <= 64: a butterfly inside the wave, fixed order)
-  for (int off = g.lp >> 1; off > 0; off >>= 1) {
+  // fold over the lanes of the plane, returned in each of them, fixed association
 #pragma unroll
-    for (int t = 0; t < T; ++t) acc[t] += __shfl_xor(acc[t], off, dev::kWave);
-  }
+  for (int t = 0; t < T; ++t) acc[t] = dev::groupSum(acc[t], g.lp);
   if (live && it0 == 0) {
     const int q = q0 + pl;
     const int n = dev::fastDiv(q, g.magicC), c = q - n * g.C;

@@ -32,10 +32,11 @@ inline int ceilDiv(int a, int b) { return (a + b - 1) / b; }
 constexpr int kBatchFloats = 4 * 4 * 256;
 
 template <typename BytesFn, typename StagedFn>
-bool pickBand(int produced, long planes, BytesFn bytes, int *tileRows, int *tilesPerPlane, StagedFn stagedFloats) {
+bool pickBand(int produced, long planes, BytesFn bytes, int *tileRows, int *tilesPerPlane, StagedFn stagedFloats,
+              size_t budget = kLdsBudget) {
   if (produced < 1 || bytes(1) > kLdsMax) return false;
   int rows = produced;
-  while (rows > 1 && bytes(rows) > kLdsBudget) rows = (rows + 1) / 2;
+  while (rows > 1 && bytes(rows) > budget) rows = (rows + 1) / 2;
   {
     int r = rows;
     while (r > 4 && stagedFloats(r) > (size_t)kBatchFloats) --r;

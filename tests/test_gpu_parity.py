@@ -146,7 +146,7 @@ def test_dwconv_small_planes(T, case):
                                   (2, 6, 1, 32, 32, 3, 3, 2, 2, 1, 1), (2, 6, 1, 24, 32, 5, 5, 1, 1, 2, 2)])
 @pytest.mark.parametrize("switch", ["0", "1"])
 def test_dwconv_small_planes_switch(T, case, switch):
-    """Shapes both kernel families take: the switch forces the small-plane kernels on or off."""
+    """Shapes both kernel families take: "0" hands them to the strip kernels, "1" leaves the default (small-plane kernels)."""
     _, x, w, b = _dw_inputs(case, 12)
     with force_direct("THCUNN_DW_SMALL", switch):
         _dw_run(T, case, x, w, b)

@@ -560,6 +560,119 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
   }
 }
 
+// ---- resident path for small channels of any plane size -----------------------------------
+// The last stages of a network have planes of 49 elements (7x7): not a multiple of 4, so the 16-byte
+// walkers above do not apply, and a channel holds only N*L of the order of 3000 elements. One 256-lane
+// workgroup per channel keeps them in registers, RS scalar elements per lane (element e = tid + 256 u is
+// image e / L, position e % L: the lanes of a wave read runs of L consecutive floats); the formulas
+// are those of the 1024-lane kernels.
+constexpr int kSmallBlock = 256;
+
+__device__ __forceinline__ float blockSum256(float v, float *red) {
+  const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
+  v = dev::waveSum(v);
+  __syncthreads();  // red may still be read from a previous reduction
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// element offsets (in floats, from the channel's first plane) of this lane; -1 past the channel
+template <int RS>
+__device__ __forceinline__ void smallOffsets(int (&off)[RS], int N, int C, int L, unsigned magicL) {
+#pragma unroll
+  for (int u = 0; u < RS; ++u) {
+    const int e = u * kSmallBlock + (int)threadIdx.x;
+    const int n = dev::fastDiv(e, magicL);
+    off[u] = e < N * L ? n * C * L + (e - n * L) : -1;
+  }
+}
+
+template <int RS>
+__global__ void __launch_bounds__(kSmallBlock)
+bnFwdSmall(const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ weight,
+           const float *__restrict__ bias, float *__restrict__ runningMean, float *__restrict__ runningVar,
+           float *__restrict__ saveMean, float *__restrict__ saveStd, int N, int C, int L, unsigned magicL,
+           float momentum, float eps) {
+  __shared__ float red[kSmallBlock / dev::kWave];
+  const int ch = blockIdx.x;
+  const float *xc = x + (long)ch * L;
+  float *yc = y + (long)ch * L;
+  int off[RS];
+  smallOffsets<RS>(off, N, C, L, magicL);
+  float v[RS];
+#pragma unroll
+  for (int u = 0; u < RS; ++u) v[u] = off[u] >= 0 ? xc[off[u]] : 0.f;
+  const float cnt = (float)N * (float)L, norm = 1.f / cnt;
+  float s = 0.f;
+#pragma unroll
+  for (int u = 0; u < RS; ++u) s += v[u];
+  const float mean = blockSum256(s, red) * norm;
+  float q = 0.f;
+#pragma unroll
+  for (int u = 0; u < RS; ++u)
+    if (off[u] >= 0) q += (v[u] - mean) * (v[u] - mean);
+  const float varN = blockSum256(q, red);
+  float invStd = 0.f;
+  if (varN != 0.f || eps != 0.f) invStd = 1.f / sqrtf(varN * norm + eps);
+  if (threadIdx.x == 0) {
+    float unbiased = varN / (cnt - 1.f);
+    saveMean[ch] = mean;
+    saveStd[ch] = invStd;
+    runningMean[ch] = (1.f - momentum) * runningMean[ch] + momentum * mean;
+    runningVar[ch] = (1.f - momentum) * runningVar[ch] + momentum * unbiased;
+  }
+  const float gamma = weight ? weight[ch] : 1.f, beta = bias ? bias[ch] : 0.f;
+#pragma unroll
+  for (int u = 0; u < RS; ++u)
+    if (off[u] >= 0) yc[off[u]] = gamma * (v[u] - mean) * invStd + beta;
+}
+
+template <int RS, bool TRAIN>
+__global__ void __launch_bounds__(kSmallBlock)
+bnBwdSmall(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
+           float *__restrict__ gradWeight, float *__restrict__ gradBias, const float *__restrict__ weight,
+           const float *__restrict__ meanSrc, const float *__restrict__ stdSrc, int N, int C, int L, unsigned magicL,
+           float scale, float eps) {
+  __shared__ float red[kSmallBlock / dev::kWave];
+  const int ch = blockIdx.x;
+  const float *xc = x + (long)ch * L, *gc = gy + (long)ch * L;
+  const float mean = meanSrc[ch];
+  const float stdVal = TRAIN ? stdSrc[ch] : 1.f / sqrtf(stdSrc[ch] + eps);
+  const float weightVal = weight ? weight[ch] : 1.f;
+  int off[RS];
+  smallOffsets<RS>(off, N, C, L, magicL);
+  float d[RS], xm[RS];
+#pragma unroll
+  for (int u = 0; u < RS; ++u) {
+    d[u] = off[u] >= 0 ? gc[off[u]] : 0.f;
+    xm[u] = off[u] >= 0 ? xc[off[u]] : mean;
+  }
+  float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+  for (int u = 0; u < RS; ++u) {
+    xm[u] -= mean;
+    s0 += d[u];
+    s1 += d[u] * xm[u];
+  }
+  const float gradOutputSum = blockSum256(s0, red);
+  const float dotP = blockSum256(s1, red);
+  const float norm = 1.f / ((float)N * (float)L);
+  const float gradMean = gradOutputSum * norm;
+  const float projScale = dotP * norm * stdVal * stdVal;
+  const float gradScale = stdVal * weightVal;
+  if (gx) {
+    float *oc = gx + (long)ch * L;
+#pragma unroll
+    for (int u = 0; u < RS; ++u)
+      if (off[u] >= 0) oc[off[u]] = TRAIN ? (d[u] - xm[u] * projScale - gradMean) * gradScale : d[u] * gradScale;
+  }
+  if (threadIdx.x == 0) {
+    if (gradWeight) gradWeight[ch] += scale * dotP * stdVal;
+    if (gradBias) gradBias[ch] += scale * gradOutputSum;
+  }
+}
+
 // -------------------------------------------------------------- host side ----
 struct BnView {
   BnGeom g;
@@ -627,6 +740,21 @@ int residentR(const BnView &v, int maxR) {
   return 0;
 }
 
+// Elements per lane of the small-channel kernels (0: not applicable): planes whose size is not a multiple of 4
+// (the 16-byte kernels take the others), channels of at most 32 * 256 elements, enough channels to occupy the chip.
+int smallR(const BnView &v) {
+  const char *e = getenv("THCUNN_BN_FORCE_CHUNKED");
+  if (e && e[0] == '1') return 0;
+  const BnGeom &g = v.g;
+  const long NL = (long)g.N * g.L;
+  if (g.L % 4 == 0 || g.C < 96 || NL > 32 * kSmallBlock || (long)g.N * g.C * g.L >= 0x7fffffffL) return 0;
+  const int need = (int)((NL + kSmallBlock - 1) / kSmallBlock);
+  const int sizes[] = {4, 8, 16, 32};
+  for (int r : sizes)
+    if (need <= r) return r;
+  return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -664,6 +792,18 @@ void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *inp
                                                 data(saveStd_), g.N, g.C, g.L, (float)momentum, (float)eps);
     BN_FWD_RES(2) BN_FWD_RES(4) BN_FWD_RES(8) BN_FWD_RES(12) BN_FWD_RES(13) BN_FWD_RES(14)
 #undef BN_FWD_RES
+    THC_HIP_CHECK(hipGetLastError());
+    return;
+  }
+  if (int RS = train ? smallR(v) : 0) {
+#define BN_FWD_SMALL(RR)                                                                                            \
+  if (RS == RR)                                                                                                     \
+    bnFwdSmall<RR><<<g.C, kSmallBlock, 0, s>>>(in.ptr(), data(output_), dataOrNull(weight_), dataOrNull(bias_),     \
+                                               data(runningMean_), data(runningVar_), data(saveMean_),              \
+                                               data(saveStd_), g.N, g.C, g.L, dev::magicOf(g.L), (float)momentum,   \
+                                               (float)eps);
+    BN_FWD_SMALL(4) BN_FWD_SMALL(8) BN_FWD_SMALL(16) BN_FWD_SMALL(32)
+#undef BN_FWD_SMALL
     THC_HIP_CHECK(hipGetLastError());
     return;
   }
@@ -764,6 +904,24 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
   }
     BN_BWD_RES(2) BN_BWD_RES(4) BN_BWD_RES(8) BN_BWD_RES(12) BN_BWD_RES(13)
 #undef BN_BWD_RES
+    THC_HIP_CHECK(hipGetLastError());
+    return;
+  }
+  if (int RS = needSums ? smallR(v) : 0) {
+    float *gxp = gradInput_ ? data(gradInput_) : nullptr;
+#define BN_BWD_SMALL(RR)                                                                                          \
+  if (RS == RR) {                                                                                                 \
+    if (train)                                                                                                    \
+      bnBwdSmall<RR, true><<<g.C, kSmallBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),          \
+                                                       dataOrNull(gradBias_), dataOrNull(weight_), meanSrc, stdSrc, \
+                                                       g.N, g.C, g.L, dev::magicOf(g.L), (float)scale, (float)eps); \
+    else                                                                                                          \
+      bnBwdSmall<RR, false><<<g.C, kSmallBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),         \
+                                                        dataOrNull(gradBias_), dataOrNull(weight_), meanSrc, stdSrc, \
+                                                        g.N, g.C, g.L, dev::magicOf(g.L), (float)scale, (float)eps); \
+  }
+    BN_BWD_SMALL(4) BN_BWD_SMALL(8) BN_BWD_SMALL(16) BN_BWD_SMALL(32)
+#undef BN_BWD_SMALL
     THC_HIP_CHECK(hipGetLastError());
     return;
   }

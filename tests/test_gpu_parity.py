@@ -429,7 +429,9 @@ def test_avgpool_reference_known_answer(T):
 # ------------------------------------------------------------------------- BN --
 BN_SHAPES = [(8, 16, 28, 28), (4, 3, 7, 5), (32, 64), (2, 5, 33), (3, 2, 4, 5, 6), (2, 2, 150, 120), (1, 3, 9000),
              # channel-resident kernels (C >= 96, a channel fits one workgroup's registers)
-             (64, 100, 28, 28), (40, 96, 20, 20), (33, 97, 12, 12), (4, 128, 14, 14), (57, 96, 24, 28)]
+             (64, 100, 28, 28), (40, 96, 20, 20), (33, 97, 12, 12), (4, 128, 14, 14), (57, 96, 24, 28),
+             # small channels with planes that are not a multiple of 4 elements (scalar resident kernels)
+             (16, 130, 7, 7), (64, 96, 7, 7), (5, 100, 3, 3), (160, 97, 7, 7), (3, 128, 1, 1), (2, 96, 13, 11)]
 
 
 def _bn_run(T, shape, affine, seed=40):

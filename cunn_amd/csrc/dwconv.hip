@@ -423,7 +423,7 @@ dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strid
 #pragma unroll
       for (int kh = 0; kh < KS; ++kh) {
         float win[NW];
-        S::loadWin(p + kh * pitch, b4, g.W, win);
+        S::loadWinShared(p + kh * pitch, b4, oW4, g.W, win);
 #pragma unroll
         for (int kw = 0; kw < KS; ++kw)
 #pragma unroll
@@ -474,7 +474,8 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
   // a run-time value, so those taps are selected into per-lane weights instead of being resolved at compile time.
   const int total = nRows * W4;
   float *o = gradIn + ((long)plane * g.H + h0) * g.W;
-#pragma unroll 2
+  constexpr int kUnroll = ST == 1 ? 1 : 2;  // the wave shifts of the stride-1 window do not unroll
+#pragma unroll kUnroll
   for (int i = threadIdx.x; i < total; i += blockDim.x) {
     const int hl = dev::fastDiv(i, magicW4), b = i - hl * W4;
     const int a = ST == 1 ? hl : hl >> (ST == 2 ? 1 : 0), dy = hl - a * ST;
@@ -495,7 +496,10 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
           }
         }
         float win[NW];
-        dev::readWindow<0, NW, OFF, ALIGN>(gj + (a + qh - QH0) * pitch, win);
+        if constexpr (ST == 1)
+          dev::loadWindowShared<PAD>(gj - QW0 + (a + qh - QH0) * pitch, b, W4, win);  // NW = 4 + 2 PAD, QW0 = -PAD
+        else
+          dev::readWindow<0, NW, OFF, ALIGN>(gj + (a + qh - QH0) * pitch, win);
 #pragma unroll
         for (int dx = 0; dx < 4; ++dx)
 #pragma unroll
@@ -570,7 +574,7 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
 #pragma unroll
       for (int kh = 0; kh < KS; ++kh) {
         float win[NW];
-        S::loadWin(p + kh * pitch, b4, g.W, win);
+        S::loadWinShared(p + kh * pitch, b4, oW4, g.W, win);
 #pragma unroll
         for (int kw = 0; kw < KS; ++kw)
 #pragma unroll

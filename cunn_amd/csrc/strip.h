@@ -35,6 +35,35 @@ struct TapSpan {
   }
 };
 
+// Window of a stride-1 item: columns 4*b4 - PAD .. 4*b4 + 3 + PAD of a staged row, p pointing at column 4*b4.
+// For loops in which the lanes of a wave hold consecutive items (b4, then the next row): the window is the
+// lane's own 4 columns (one aligned 16-byte read) plus PAD columns on either side, and those are the last /
+// first columns of the neighbouring lanes' reads - they come over the wave shift of the DPP unit instead of
+// 4-byte LDS reads, which hit only 16 of the 64 banks (stride of 4 floats between lanes). The first and
+// last group of a row take the zero border instead; lanes 0 and 63 of a wave have no neighbour on one
+// side and read LDS (the cells around a row hold the border or the neighbouring group).
+template <int PAD>
+__device__ __forceinline__ void loadWindowShared(const float *__restrict__ p, int b4, int W4, float (&win)[4 + 2 * PAD]) {
+  static_assert(PAD >= 1 && PAD <= 2, "kernel 3 or 5");
+  const float4 c = *reinterpret_cast<const float4 *>(p);
+  const int lane = threadIdx.x % kWave;
+  auto fromLeft = [](float v) {   // value of lane - 1
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x138, 0xF, 0xF, true));
+  };
+  auto fromRight = [](float v) {  // value of lane + 1
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x130, 0xF, 0xF, true));
+  };
+  float l[2] = {fromLeft(c.z), fromLeft(c.w)};
+  float r[2] = {fromRight(c.x), fromRight(c.y)};
+  if (lane == 0) l[0] = p[-2], l[1] = p[-1];
+  if (lane == kWave - 1) r[0] = p[4], r[1] = p[5];
+  if (b4 == 0) l[0] = l[1] = 0.f;
+  if (b4 == W4 - 1) r[0] = r[1] = 0.f;
+#pragma unroll
+  for (int j = 0; j < PAD; ++j) win[j] = l[2 - PAD + j], win[PAD + 4 + j] = r[j];
+  win[PAD] = c.x, win[PAD + 1] = c.y, win[PAD + 2] = c.z, win[PAD + 3] = c.w;
+}
+
 // How the input band of a strip kernel is laid out in LDS and how a lane reads
 // the NW = 3*ST + KS consecutive input columns its 4 outputs need.
 //   ST == 1: plain rows, pitch W + 4, element (r, col) at r*pitch + 4 + col.
@@ -118,6 +147,37 @@ struct Strip {
     for (int j = 0; j < NW; ++j)
       if (even(j) == e && half(j) > m) m = half(j);
     return m;
+  }
+  // The same window with its edge columns taken from the neighbouring lanes (see loadWindowShared), for rows
+  // whose border cells hold zeros: a lane reads its own 4 columns (ST == 1) or its 4 even and 4 odd columns
+  // (ST == 2) with aligned 16-byte reads only. nb4 = groups per row.
+  __device__ static void loadWinShared(const float *__restrict__ row, int b4, int nb4, int W, float (&win)[NW]) {
+    if constexpr (ST == 1) {
+      static_assert(NW == 4 + 2 * PAD, "stride 1");
+      loadWindowShared<PAD>(row + kStripPadL + b4 * 4, b4, nb4, win);
+    } else {
+      constexpr int ELO = lo(true), EHI = hi(true), OLO = lo(false), OHI = hi(false);
+      static_assert(ELO >= -2 && OLO >= -2 && EHI <= 5 && OHI <= 5, "at most two columns from a neighbour");
+      const float *pe = row + 4 + b4 * 4, *po = row + (W >> 1) + 8 + b4 * 4;
+      const float4 e = *reinterpret_cast<const float4 *>(pe), o = *reinterpret_cast<const float4 *>(po);
+      const int lane = threadIdx.x % kWave;
+      const bool first = b4 == 0, last = b4 == nb4 - 1;
+      // half-index k of the even (odd) columns: 0..3 own, negative from lane - 1, above 3 from lane + 1
+      auto pick = [&](const float4 &v, const float *p, int k) -> float {
+        const float own[4] = {v.x, v.y, v.z, v.w};
+        if (k >= 0 && k < 4) return own[k];
+        if (k < 0) {
+          float t = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, own[4 + k]), 0x138, 0xF, 0xF, true));
+          if (lane == 0) t = p[k];
+          return first ? 0.f : t;
+        }
+        float t = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, own[k - 4]), 0x130, 0xF, 0xF, true));
+        if (lane == kWave - 1) t = p[k];
+        return last ? 0.f : t;
+      };
+#pragma unroll
+      for (int j = 0; j < NW; ++j) win[j] = even(j) ? pick(e, pe, half(j)) : pick(o, po, half(j));
+    }
   }
   __device__ static void loadWin(const float *__restrict__ row, int b4, int W, float (&win)[NW]) {
     if constexpr (ST == 1) {

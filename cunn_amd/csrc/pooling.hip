@@ -27,6 +27,7 @@ struct PoolGeom {
   int maxStageRows;  // rows of the staged tensor per band (upper bound)
   unsigned magicTiles;  // dev::magicOf(tilesPerPlane), used by the strip kernels
   int constDiv;         // average pooling: every window has the divisor kH*kW (no window is clipped)
+  unsigned magicDH, magicDW;  // dev::magicOf(dH), dev::magicOf(dW): the backward gathers divide by the strides
 };
 
 // (plane, tile) of a workgroup of the strip kernels
@@ -255,10 +256,10 @@ avgPoolFwdDirect(const float *__restrict__ in, float *__restrict__ out, PoolGeom
 template <bool INCLUDE_PAD>
 __device__ __forceinline__ float avgGather(const float *__restrict__ gp, int rowOff, int h, int w, const PoolGeom &g) {
   const int hp = h + g.padH, wp = w + g.padW;
-  const int phstart = (hp < g.kH) ? 0 : (hp - g.kH) / g.dH + 1;
-  const int phend = min(hp / g.dH + 1, g.oH);
-  const int pwstart = (wp < g.kW) ? 0 : (wp - g.kW) / g.dW + 1;
-  const int pwend = min(wp / g.dW + 1, g.oW);
+  const int phstart = (hp < g.kH) ? 0 : dev::fastDiv(hp - g.kH, g.magicDH) + 1;
+  const int phend = min(dev::fastDiv(hp, g.magicDH) + 1, g.oH);
+  const int pwstart = (wp < g.kW) ? 0 : dev::fastDiv(wp - g.kW, g.magicDW) + 1;
+  const int pwend = min(dev::fastDiv(wp, g.magicDW) + 1, g.oW);
   float grad = 0.f;
   for (int ph = phstart; ph < phend; ++ph)
     for (int pw = pwstart; pw < pwend; ++pw) {
@@ -299,6 +300,123 @@ avgPoolBwdDirect(const float *__restrict__ gradOut, float *__restrict__ gradIn, 
     int h = (int)(t % g.H);
     long plane = t / g.H;
     gradIn[i] = avgGather<INCLUDE_PAD>(gradOut + plane * g.oH * g.oW, 0, h, w, g);
+  }
+}
+
+// ===================================================== small planes, any geometry ==
+// Planes of at most 1024 elements (the 28x28 / 14x14 / 7x7 stages) that the strip kernels do not take:
+// a plane per workgroup would leave most lanes idle, so a workgroup takes P consecutive planes - one
+// contiguous run of memory - stages what it reads in LDS and produces its results in memory order
+// (a lane per output element forward, 4 consecutive gradInput elements backward), so every global
+// access of a wave is one contiguous run. Window geometry is run-time (the reference's loops).
+struct SmallPool {
+  int planes, P;          // N * C, planes per workgroup
+  unsigned magicHW, magicW, magicOHW, magicOW;
+  bool vec;               // runs start on 16-byte boundaries: 16-byte accesses allowed
+};
+
+template <bool MAX, bool INCLUDE_PAD>
+__global__ void __launch_bounds__(dev::kBlock)
+poolFwdSmall(const float *__restrict__ in, float *__restrict__ out, long *__restrict__ indices, PoolGeom g, SmallPool sp) {
+  extern __shared__ float smem[];
+  const int HW = g.H * g.W, oHW = g.oH * g.oW;
+  const int q0 = blockIdx.x * sp.P;
+  const int np = min(sp.P, sp.planes - q0);
+  const int nIn = np * HW, nOut = np * oHW;
+  const float *src = in + (long)q0 * HW;
+  if (sp.vec) {
+    for (int i = threadIdx.x * 4; i < nIn; i += dev::kBlock * 4) {
+      if (i + 4 <= nIn) {
+        *reinterpret_cast<float4 *>(smem + i) = *reinterpret_cast<const float4 *>(src + i);
+      } else {
+        for (int k = i; k < nIn; ++k) smem[k] = src[k];
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < nIn; i += dev::kBlock) smem[i] = src[i];
+  }
+  __syncthreads();
+  float *o = out + (long)q0 * oHW;
+  long *ix = MAX ? indices + (long)q0 * oHW : nullptr;
+  for (int i = threadIdx.x; i < nOut; i += dev::kBlock) {
+    const int pl = dev::fastDiv(i, sp.magicOHW), r = i - pl * oHW;
+    const int ph = dev::fastDiv(r, sp.magicOW), pw = r - ph * g.oW;
+    const float *ip = smem + pl * HW;
+    if (MAX) {
+      int hstart = ph * g.dH - g.padH, wstart = pw * g.dW - g.padW;
+      const int hend = min(hstart + (g.kH - 1) * g.dilH + 1, g.H);
+      const int wend = min(wstart + (g.kW - 1) * g.dilW + 1, g.W);
+      while (hstart < 0) hstart += g.dilH;
+      while (wstart < 0) wstart += g.dilW;
+      float maxval = -FLT_MAX;
+      int maxidx = -1;
+      for (int h = hstart; h < hend; h += g.dilH)
+        for (int w = wstart; w < wend; w += g.dilW) {
+          const float v = ip[h * g.W + w];
+          if (v > maxval) maxval = v, maxidx = h * g.W + w;
+        }
+      o[i] = maxval;
+      ix[i] = (long)maxidx + TH_INDEX_BASE;
+    } else {
+      int hs, he, ws, we;
+      const float div = avgDivisor<INCLUDE_PAD>(ph, pw, g, hs, he, ws, we);
+      float sum = 0.f;
+      for (int h = hs; h < he; ++h)
+        for (int w = ws; w < we; ++w) sum += ip[h * g.W + w];
+      o[i] = sum / div;
+    }
+  }
+}
+
+template <bool MAX, bool INCLUDE_PAD>
+__global__ void __launch_bounds__(dev::kBlock)
+poolBwdSmall(const float *__restrict__ gradOut, const long *__restrict__ indices, float *__restrict__ gradIn, PoolGeom g,
+             SmallPool sp) {
+  extern __shared__ float smem[];
+  const int HW = g.H * g.W, oHW = g.oH * g.oW;
+  const int q0 = blockIdx.x * sp.P;
+  const int np = min(sp.P, sp.planes - q0);
+  const int nIn = np * HW, nOut = np * oHW;
+  float *gs = smem;
+  int *is = reinterpret_cast<int *>(smem + sp.P * oHW);  // max: argmax positions inside their plane, 0-based
+  for (int i = threadIdx.x; i < nOut; i += dev::kBlock) {
+    gs[i] = gradOut[(long)q0 * oHW + i];
+    if (MAX) is[i] = (int)(indices[(long)q0 * oHW + i] - TH_INDEX_BASE);
+  }
+  __syncthreads();
+  const int extH = (g.kH - 1) * g.dilH + 1, extW = (g.kW - 1) * g.dilW + 1;
+  float *o = gradIn + (long)q0 * HW;
+  for (int i4 = threadIdx.x * 4; i4 < nIn; i4 += dev::kBlock * 4) {
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int i = i4 + k;
+      v[k] = 0.f;
+      if (i < nIn) {
+        const int pl = dev::fastDiv(i, sp.magicHW), r = i - pl * HW;
+        const int h = dev::fastDiv(r, sp.magicW), w = r - h * g.W;
+        if (MAX) {
+          const int phstart = (h + g.padH < extH) ? 0 : dev::fastDiv(h + g.padH - extH, g.magicDH) + 1;
+          const int phend = min(dev::fastDiv(h + g.padH, g.magicDH) + 1, g.oH);
+          const int pwstart = (w + g.padW < extW) ? 0 : dev::fastDiv(w + g.padW - extW, g.magicDW) + 1;
+          const int pwend = min(dev::fastDiv(w + g.padW, g.magicDW) + 1, g.oW);
+          float grad = 0.f;
+          for (int ph = phstart; ph < phend; ++ph)
+            for (int pw = pwstart; pw < pwend; ++pw)
+              if (is[pl * oHW + ph * g.oW + pw] == r) grad += gs[pl * oHW + ph * g.oW + pw];
+          v[k] = grad;
+        } else {
+          v[k] = avgGather<INCLUDE_PAD>(gs + pl * oHW, 0, h, w, g);
+        }
+      }
+    }
+    if (sp.vec && i4 + 4 <= nIn) {
+      dev::storeStream4(o + i4, make_float4(v[0], v[1], v[2], v[3]));
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (i4 + k < nIn) o[i4 + k] = v[k];
+    }
   }
 }
 
@@ -621,6 +739,30 @@ bool avgFlatOk(const PoolGeom &g, long planes) {
          total > 0 && total * (g.oW / 4) < 0xffffffffL && total < 0x7fffffffL;
 }
 
+// Plans the small-plane kernels: planes of at most 1024 elements; `staged` = elements per plane held in LDS
+// (forward: the input plane; backward: gradOutput and, for max pooling, its indices), `produced` = elements
+// per plane written. P planes per workgroup: about 8192 produced elements, at most 32 KB of LDS.
+bool smallPoolPlan(const PoolGeom &g, long planes, bool backward, bool max, const void *a, const void *b, SmallPool *sp,
+                   size_t *lds) {
+  const long HW = (long)g.H * g.W, oHW = (long)g.oH * g.oW;
+  // forward: measured faster than the band kernels up to about 20x20 planes; backward up to 32x32
+  if (forcedPath() != 0 || HW > (backward ? 1024 : 400) || HW < 1 || oHW < 1 || oHW > 4096 || planes >= 0x7fffffffL)
+    return false;
+  const long ldsPerPlane = backward ? oHW * (max ? 8 : 4) : HW * 4;
+  const long produced = backward ? HW : oHW;
+  long P = std::max<long>(1, std::min<long>(8192 / std::max<long>(produced, 1), (32 * 1024) / ldsPerPlane));
+  P = std::min(P, planes);
+  if (P < 1 || P * ldsPerPlane > (long)launch::kLdsMax) return false;
+  // enough workgroups to occupy the chip
+  while (P > 1 && planes / P < launch::kMinBlocks) P = (P + 1) / 2;
+  sp->planes = (int)planes, sp->P = (int)P;
+  sp->magicHW = dev::magicOf((int)HW), sp->magicW = dev::magicOf(g.W);
+  sp->magicOHW = dev::magicOf((int)oHW), sp->magicOW = dev::magicOf(g.oW);
+  sp->vec = (P * HW) % 4 == 0 && aligned16(a) && aligned16(b);
+  *lds = (size_t)(P * ldsPerPlane);
+  return true;
+}
+
 // One window that is exactly the plane; total elements small enough for the reciprocal division.
 bool avgGlobalOk(const PoolGeom &g, long planes) {
   return forcedPath() == 0 && g.oH == 1 && g.oW == 1 && g.padH == 0 && g.padW == 0 && g.kH == g.H && g.kW == g.W &&
@@ -724,6 +866,7 @@ PoolCall poolSetup(THCudaTensor *input, THCudaTensor *gradOutput, THCudaLongTens
   g.tileRows = g.tilesPerPlane = g.nblk = g.maxStageRows = 0;
   g.magicTiles = 0;
   g.constDiv = 0;
+  g.magicDH = dev::magicOf(dH), g.magicDW = dev::magicOf(dW);
   return c;
 }
 
@@ -760,6 +903,8 @@ void maxPoolUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *out
     auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.W * sizeof(float); };
     auto sbytes = [&](int rows) { return fwdStripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
     auto staged = [&](int rows) { return (size_t)((rows - 1) * g.dH + g.kH) * g.W; };
+    SmallPool sp;
+    size_t slds;
     if (stripFwdOk(g) && vec && aligned16(data(output)) && aligned16(data(indices)) &&
         launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane, staged)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
@@ -771,6 +916,9 @@ void maxPoolUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *out
     maxPoolFwdStrip<K, S, P><<<grid, block, lds, s>>>(in.ptr(), data(output), data(indices), g);
       POOL_STRIP_COMBOS(X)
 #undef X
+    } else if (smallPoolPlan(g, planes, false, true, in.ptr(), in.ptr(), &sp, &slds)) {
+      poolFwdSmall<true, false><<<launch::ceilDiv(sp.planes, sp.P), dev::kBlock, slds, s>>>(in.ptr(), data(output),
+                                                                                           data(indices), g, sp);
     } else if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
       g.magicTiles = dev::magicOf(g.tilesPerPlane);
@@ -814,6 +962,8 @@ void maxPoolUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *
   const int spitch = g.oW + dev::kStripPadL;
   auto sbytes = [&](int units) { return 2 * ((size_t)(units + extra) * spitch + dev::kStripPadL) * sizeof(float); };
   int units = 0;
+  SmallPool sp;
+  size_t slds;
   if (stripBwdOk(g) && vec && aligned16(data(gradInput)) &&
       launch::pickBand(launch::ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
     g.tileRows = units * g.dH;
@@ -826,6 +976,9 @@ void maxPoolUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *
     poolBwdStrip<K, S, P, true, true><<<grid, block, lds, s>>>(go.ptr(), data(indices), data(gradInput), g, units + extra);
     POOL_STRIP_COMBOS(X)
 #undef X
+  } else if (smallPoolPlan(g, planes, true, true, data(gradInput), data(gradInput), &sp, &slds)) {
+    poolBwdSmall<true, false><<<launch::ceilDiv(sp.planes, sp.P), dev::kBlock, slds, s>>>(go.ptr(), data(indices),
+                                                                                         data(gradInput), g, sp);
   } else if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
       g.magicTiles = dev::magicOf(g.tilesPerPlane);
@@ -903,6 +1056,8 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
     auto bytes = [&](int rows) { return (size_t)stageRows(rows) * g.W * sizeof(float); };
     auto sbytes = [&](int rows) { return fwdStripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
     auto staged = [&](int rows) { return (size_t)((rows - 1) * g.dH + g.kH) * g.W; };
+    SmallPool sp;
+    size_t slds;
     if (avgGlobalOk(g, planes)) {
       const long waves = std::min<long>((planes + 3) / 4, 8192);
       avgPoolGlobalFwd<<<(unsigned)((waves + 3) / 4), dev::kBlock, 0, s>>>(in.ptr(), data(output), planes, g.H * g.W);
@@ -928,6 +1083,12 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
   }
       POOL_STRIP_COMBOS(X)
 #undef X
+    } else if (smallPoolPlan(g, planes, false, false, in.ptr(), in.ptr(), &sp, &slds)) {
+      const unsigned grid = launch::ceilDiv(sp.planes, sp.P);
+      if (count_include_pad)
+        poolFwdSmall<false, true><<<grid, dev::kBlock, slds, s>>>(in.ptr(), data(output), nullptr, g, sp);
+      else
+        poolFwdSmall<false, false><<<grid, dev::kBlock, slds, s>>>(in.ptr(), data(output), nullptr, g, sp);
     } else if (!forceDirect() && launch::pickBand(g.oH, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
       g.magicTiles = dev::magicOf(g.tilesPerPlane);
@@ -983,6 +1144,8 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
   const int spitch = g.oW + dev::kStripPadL;
   auto sbytes = [&](int units) { return ((size_t)(units + extra) * spitch + dev::kStripPadL) * sizeof(float); };
   int units = 0;
+  SmallPool sp;
+  size_t slds;
   if (avgGlobalOk(g, planes)) {
     const unsigned total = (unsigned)(planes * g.H * g.W);
     avgPoolGlobalBwd<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), total,
@@ -1010,6 +1173,12 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
   }
     POOL_STRIP_COMBOS(X)
 #undef X
+  } else if (smallPoolPlan(g, planes, true, false, data(gradInput), data(gradInput), &sp, &slds)) {
+    const unsigned grid = launch::ceilDiv(sp.planes, sp.P);
+    if (count_include_pad)
+      poolBwdSmall<false, true><<<grid, dev::kBlock, slds, s>>>(go.ptr(), nullptr, data(gradInput), g, sp);
+    else
+      poolBwdSmall<false, false><<<grid, dev::kBlock, slds, s>>>(go.ptr(), nullptr, data(gradInput), g, sp);
   } else if (!forceDirect() && launch::pickBand(g.H, planes, bytes, &g.tileRows, &g.tilesPerPlane)) {
     g.nblk = (int)(planes * g.tilesPerPlane);
       g.magicTiles = dev::magicOf(g.tilesPerPlane);

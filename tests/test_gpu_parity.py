@@ -340,6 +340,33 @@ def test_maxpool_fallback_kernels(T, case, mode):
         _maxpool_run(T, case, _tied_input(case[:4], 21, q=8))
 
 
+POOL_SMALL_CASES = [
+    # planes of at most 1024 elements outside the strip kernels' geometries: several planes per workgroup
+    (4, 40, 14, 14, 2, 2, 2, 2, 0, 0, False),    # VGG-style 14 -> 7
+    (3, 33, 28, 28, 2, 2, 2, 2, 0, 0, False),    # 28 -> 14: plane count not a multiple of the group
+    (2, 20, 13, 13, 3, 3, 2, 2, 0, 0, False),    # overlapping 3x3 stride 2, odd plane
+    (2, 12, 27, 27, 3, 3, 2, 2, 0, 0, True),     # ceil mode
+    (2, 9, 7, 7, 3, 3, 1, 1, 1, 1, False),       # padded, stride 1
+    (3, 5, 15, 9, 2, 3, 1, 2, 1, 0, True),       # rectangular everything
+    (1, 3, 6, 6, 3, 3, 2, 2, 1, 1, False),       # three planes in all
+    (2, 70, 5, 5, 2, 2, 2, 2, 0, 0, True),       # ceil mode with a clipped last window
+    (300, 9, 3, 3, 2, 2, 1, 1, 0, 0, False),     # many tiny planes
+]
+
+
+@pytest.mark.parametrize("case", POOL_SMALL_CASES)
+def test_maxpool_small_planes(T, case):
+    _maxpool_run(T, case, _tied_input(case[:4], 25, q=8))
+    if case[4] > 1 and case[5] > 1 and case[2] >= 9 and case[3] >= 9:
+        _maxpool_run(T, case, _tied_input(case[:4], 26, q=8), dil=(2, 2))
+
+
+@pytest.mark.parametrize("case", POOL_SMALL_CASES)
+@pytest.mark.parametrize("include_pad", [True, False])
+def test_avgpool_small_planes(T, case, include_pad):
+    _avgpool_run(T, case, include_pad, seed=34)
+
+
 def test_maxpool_dilated_and_noncontiguous(T):
     case = (2, 3, 30, 34, 3, 2, 2, 1, 1, 1, False)
     x = _tied_input(case[:4], 22, q=16)

@@ -7,7 +7,7 @@ A step is one pass of the workload's entry points over one synthetic batch,
 called through the C ABI of libTHCUNN.so. The default workload is the one the
 headline metric is quoted on: SpatialDepthWiseConvolution forward +
 updateGradInput + accGradParameters, fp32, N=64 C=128 56x56 -> 28x28, 3x3
-stride 2 pad 1 (BASELINE.json configs[1]). Inputs live in HBM before the timed
+stride 2 pad 1 (the MobileNet stride-2 layer). Inputs live in HBM before the timed
 region; four buffer sets are rotated so that no step finds its inputs in the
 256 MB Infinity Cache from the step before.
 
@@ -523,7 +523,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
-              "(the path shards by batch, see DESIGN.md)", file=sys.stderr)
+              "(the path would shard by batch; nothing multi-GPU is built)", file=sys.stderr)
         sys.exit(2)
 
     import cunn_amd

@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at their full sizes on the GPU: compared with
+"""The five benchmark configurations at their full sizes on the GPU: compared with
 the CPU oracle where it finishes in seconds, and through size-independent
 properties (adjoint identities, index round trips, gradient orthogonality)."""
 import numpy as np

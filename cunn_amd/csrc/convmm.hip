@@ -376,26 +376,41 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
           dst[(wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3)) * TBN + wn * 64 + tj * 32 + idx] = acc[ti][tj][v];
     return;
   }
+  auto store = [&](auto withBias) {
+    constexpr bool BIAS = decltype(withBias)::value;
+    // the lane's 32 bias values first, all requested together: a load between the stores would wait for
+    // each store before it (the compiler must assume that out and bias overlap)
+    float bv[2][16];
+    if (BIAS) {
 #pragma unroll
-  for (int tj = 0; tj < 2; ++tj) {
-    const long col = (long)j0 + wn * 64 + tj * 32 + idx;
-    if (col >= p.Ncols) continue;
-    const int n = (int)(col / g.L);
-    const int l = (int)(col - (long)n * g.L);
-    const int oh = l / g.oW, ow = l - oh * g.oW;
-    float *dst = p.out + (long)n * p.outImg + (long)oh * p.outSH + ow * p.outSW;
+      for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
-    for (int ti = 0; ti < 2; ++ti)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
-        if (row < p.M) {
-          float val = acc[ti][tj][v];
-          if (p.bias) val += p.bias[row];
-          dst[(long)row * p.outRow] = val;
+        for (int v = 0; v < 16; ++v) {
+          const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
+          bv[ti][v] = row < p.M ? p.bias[row] : 0.f;
         }
-      }
-  }
+    }
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+      const unsigned col = (unsigned)j0 + wn * 64 + tj * 32 + idx;  // Ncols < 2^31
+      if (col >= (unsigned)p.Ncols) continue;
+      const unsigned n = col / (unsigned)g.L;
+      const int l = (int)(col - n * (unsigned)g.L);
+      const int oh = l / g.oW, ow = l - oh * g.oW;
+      float *dst = p.out + (long)n * p.outImg + (long)oh * p.outSH + ow * p.outSW;
+#pragma unroll
+      for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
+          if (row < p.M) dst[(long)row * p.outRow] = BIAS ? acc[ti][tj][v] + bv[ti][v] : acc[ti][tj][v];
+        }
+    }
+  };
+  if (p.bias)
+    store(std::true_type{});
+  else
+    store(std::false_type{});
 }
 
 // taps[k] = ((c*H + kh*dilH)*W + kw*dilW) * 4 for k = (c*kH + kh)*kW + kw; g is the geometry of the padded images.
@@ -705,9 +720,9 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   const int kB = __builtin_amdgcn_readfirstlane(kgB * 4);
   int posOff;
   {
-    const long lg = min((long)j0 + colB, (long)p.Ncols - 1);
-    const int n = (int)(lg / g.L);
-    const int l = (int)(lg - (long)n * g.L);
+    const unsigned lg = min((unsigned)j0 + colB, (unsigned)p.Ncols - 1);  // Ncols < 2^31
+    const int n = (int)(lg / (unsigned)g.L);
+    const int l = (int)(lg - (unsigned)n * (unsigned)g.L);
     const int oh = l / g.oW, ow = l - oh * g.oW;
     posOff = ((n * g.Cin * g.H + oh * g.dH) * g.W + ow * g.dW) * 4;
   }

@@ -361,9 +361,11 @@ struct FwdArgs {
 // Epilogue shared by the forward kernels: a lane holds column (lane & 31) and rows
 // 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 accumulator tile. Split workgroups store their
 // partial tile, the others add the bias and store to out(n, row, l).
+// biasLds: the tile's bias values in LDS (index = row - m0, zeros where there is no bias or row), or null.
 template <int TBN = BN>
 __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g, const float16v (&acc)[2][2], int bx,
-                                            int by, int m0, int j0, int wm, int wn, int grp, int idx) {
+                                            int by, int m0, int j0, int wm, int wn, int grp, int idx,
+                                            const float *biasLds = nullptr) {
   const int rowHalf = grp * 4;
   if (p.nSplit > 1) {
     float *dst = p.partial + ((long)bx * p.nSplit + by) * (BM * BN);  // both tile shapes hold BM * BN elements
@@ -378,16 +380,24 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
   }
   auto store = [&](auto withBias) {
     constexpr bool BIAS = decltype(withBias)::value;
-    // the lane's 32 bias values first, all requested together: a load between the stores would wait for
-    // each store before it (the compiler must assume that out and bias overlap)
+    // the lane's 32 bias values first: a load between the stores would wait for each store before it
+    // (the compiler must assume that out and bias overlap)
     float bv[2][16];
     if (BIAS) {
 #pragma unroll
       for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
-          bv[ti][v] = row < p.M ? p.bias[row] : 0.f;
+        for (int q = 0; q < 4; ++q) {
+          if (biasLds) {  // 4 consecutive rows: one 16-byte LDS read
+            const float4 b4 = *reinterpret_cast<const float4 *>(biasLds + wm * 64 + ti * 32 + 8 * q + rowHalf);
+            bv[ti][4 * q] = b4.x, bv[ti][4 * q + 1] = b4.y, bv[ti][4 * q + 2] = b4.z, bv[ti][4 * q + 3] = b4.w;
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int row = m0 + wm * 64 + ti * 32 + 8 * q + rowHalf + r;
+              bv[ti][4 * q + r] = row < p.M ? p.bias[row] : 0.f;
+            }
+          }
         }
     }
 #pragma unroll
@@ -694,11 +704,13 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   constexpr int NB = WM == 2 ? 8 : 16;        // image elements a lane gathers per k-tile
   __shared__ float4 As[2][BK / 4][AP];
   __shared__ float4 Bs[2][BK / 4][BP];
+  __shared__ __attribute__((aligned(16))) float biasS[TBM];  // the tile's bias values: the epilogue reads them from here
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm = WM == 2 ? wave >> 1 : 0, wn = WM == 2 ? wave & 1 : wave;
   const int tileIdx = p.tile0 + blockIdx.x;
   const int mTile = tileIdx % p.mTiles, nTile = tileIdx / p.mTiles;
   const int m0 = mTile * TBM, j0 = nTile * TBN;
+  if (t < TBM) biasS[t] = p.bias && m0 + t < p.M ? p.bias[m0 + t] : 0.f;  // visible after the first barrier
 
   float16v acc[2][2];
 #pragma unroll
@@ -806,7 +818,7 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   step(Buf0{}, Buf1{}, kt, kt + 1 < nkt, kt + 2 < nkt);
   if (kt + 1 < nkt) step(Buf1{}, Buf0{}, kt + 1, kt + 2 < nkt, false);
   if (kt + 2 < nkt) step(Buf0{}, Buf1{}, kt + 2, false, false);
-  fwdEpilogue<TBN>(p, g, acc, blockIdx.x, blockIdx.y, m0, j0, wm, wn, grp, idx);
+  fwdEpilogue<TBN>(p, g, acc, blockIdx.x, blockIdx.y, m0, j0, wm, wn, grp, idx, biasS);
 }
 
 template <int WM>

@@ -1830,7 +1830,11 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   const void *kern = !fast ? (const void *)convGemmKernel<kGradWeight>
                      : l16 ? (wide ? (const void *)convGradWeightKernel<true, 1> : (const void *)convGradWeightKernel<true, 2>)
                            : (wide ? (const void *)convGradWeightKernel<false, 1> : (const void *)convGradWeightKernel<false, 2>);
-  const int slots = residentSlots(kern);
+  // Every split leaves a partial copy of gradWeight (64 KB per tile) for the fold: three workgroups per CU
+  // measured better than the four that fit (less partial traffic for the same matrix-pipe load), two when
+  // gradWeight is one or two tiles and the partials are most of the traffic.
+  const int perCu = mT * nT <= 2 ? 2 : 3;
+  const int slots = std::min(residentSlots(kern), residentSlots(nullptr) * perCu);
   int splits = std::max(1, std::min(totalKt, slots / (mT * nT)));
   const int perSplit = launch::ceilDiv(totalKt, splits);
   splits = launch::ceilDiv(totalKt, perSplit);

@@ -904,6 +904,7 @@ struct GradWeightArgs {
   const float *gy;  // (N, M, L)
   const float *x;   // (N, Cin, H, W) of g: images with their zero border
   float *partial;   // (splits, M, Ncols)
+  float *biasPartial;  // (splits, M) row sums of gy per split, or null: the bias gradient comes out of the same pass
   int M, Ncols;     // Cout, K
   int mTiles, nTiles;
   int totalKt, ktPerSplit;  // k-tiles of BK positions over the N*L positions; per split
@@ -1014,10 +1015,23 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   u32x4 *aDst = reinterpret_cast<u32x4 *>(&As[0][pgA][rowA]);
   unsigned *bDst = reinterpret_cast<unsigned *>(&Bs[0][rB >> 2][cB]) + (rB & 3);
   constexpr int BUFA = (BK / 4) * AP, BUFB = (BK / 4) * GP;  // float4 per LDS buffer
+  // The workgroups of the first column tile also sum the gradOutput elements they pass on (each element of a
+  // row is loaded by exactly one lane of exactly one of them): the bias gradient without a second pass over gy.
+  const bool rowSums = nTile == 0 && p.biasPartial != nullptr;
+  float rowSum = 0.f;
   auto storeTiles = [&](auto bufc) {
     constexpr int buf = decltype(bufc)::value;
 #pragma unroll
     for (int i = 0; i < WM; ++i) aDst[buf * BUFA + i * AP] = ra[i];
+    if (rowSums) {
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+      {
+        // (element by element: a bit cast applied to a vector element expression reads element 0 here)
+        const unsigned ex = ra[i].x, ey = ra[i].y, ez = ra[i].z, ew = ra[i].w;
+        rowSum += (__uint_as_float(ex) + __uint_as_float(ey)) + (__uint_as_float(ez) + __uint_as_float(ew));
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NB; ++i) bDst[buf * BUFB * 4 + 64 * i] = rb[i];  // column + 16 = 16 float4 further
   };
@@ -1068,6 +1082,12 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
         if (row < p.M) dst[(long)row * p.Ncols + col] = acc[ti][tj][v];
       }
   }
+  if (rowSums) {
+    // the 2 (WM = 2) or 4 (WM = 1) lanes that loaded parts of a row are neighbours inside a quad
+    rowSum = dev::dppAdd<0xB1>(rowSum);
+    if (WM == 1) rowSum = dev::dppAdd<0x4E>(rowSum);
+    if ((t & (WM == 2 ? 1 : 3)) == 0 && m0 + rowA < p.M) p.biasPartial[(long)split * p.M + m0 + rowA] = rowSum;
+  }
 }
 
 // gW[i] += scale * sum_s partial[s][i] in a fixed association: a workgroup owns 64 consecutive float4
@@ -1075,11 +1095,15 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
 // accumulators (16 16-byte loads in flight per lane), then the groups are added in order through
 // LDS. With few elements and hundreds of splits (1x1 convolutions) a one-lane-per-element loop is
 // latency bound; this form keeps enough bytes in flight to run at memory speed.
+// Blocks past the last float4 of gW do the same for the bias partials (biasPartial(splits, M), M % 4 == 0), when given.
 __global__ void __launch_bounds__(dev::kBlock)
-foldPartials4Kernel(const float *__restrict__ partial, float *__restrict__ dst, long count4, int splits, float scale) {
+foldPartials4Kernel(const float *__restrict__ partial, float *__restrict__ dst, long count4, int splits, float scale,
+                    const float *__restrict__ biasPartial, float *__restrict__ gradBias, int M, int gwBlocks) {
   __shared__ float4 part[4][64];
+  int blk = blockIdx.x;
+  if (blk >= gwBlocks) blk -= gwBlocks, partial = biasPartial, dst = gradBias, count4 = M >> 2;
   const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
-  const long i = (long)blockIdx.x * 64 + e;
+  const long i = (long)blk * 64 + e;
   float4 a[4];
 #pragma unroll
   for (int u = 0; u < 4; ++u) a[u] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -1806,8 +1830,9 @@ void convGradBias(hipStream_t s, const float *gy, float *gB, int N, int C, int L
 }
 
 // gW(Cout, K) += scale * sum_n gy_n(Cout x L) * im2col(x_n)^T
+// gB(Cout) += scale * sum_{n,l} gy when gB is given (the bias gradient of the ordinary convolution)
 void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const float *gy, float *gW,
-                    THCudaTensor *scratchBuf, float scale) {
+                    THCudaTensor *scratchBuf, float scale, float *gB = nullptr) {
   if ((long)g.N * g.Cout * g.K == 0) return;
   hipStream_t s = state->stream;
 
@@ -1841,13 +1866,19 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   const long count = (long)g.Cout * g.K;
   // scratch: the splits' partial products, then (second-generation kernel) the images with their zero border
   const long partialFloats = (splits * count + 3) / 4 * 4;
+  // the bias gradient rides along when the fold below has the 16-byte form; else it is a pass of its own
+  const bool fold4 = count % 4 == 0 && launch::aligned16(gW);
+  const bool fusedBias = gB && fast && fold4 && g.Cout % 4 == 0 && launch::aligned16(gB);
+  const long biasFloats = fusedBias ? ((long)splits * g.Cout + 3) / 4 * 4 : 0;
   Temp tmp;
-  float *partial = scratchFloats(state, scratchBuf, partialFloats + (fast && bordered ? xpFloats : 0), tmp, "columns");
+  float *partial =
+      scratchFloats(state, scratchBuf, partialFloats + biasFloats + (fast && bordered ? xpFloats : 0), tmp, "columns");
+  float *biasPartial = fusedBias ? partial + partialFloats : nullptr;
   if (fast) {
     ConvGeom gk = g;
     const float *xk = x;
     if (bordered) {
-      float *xp = partial + partialFloats;
+      float *xp = partial + partialFloats + biasFloats;
       launchPadPlanes(s, x, xp, (long)g.N * g.Cin, g.H, g.W, g.padH, g.padW);
       gk.H = g.H + 2 * g.padH, gk.W = g.W + 2 * g.padW, gk.padH = gk.padW = 0;
       xk = xp;
@@ -1856,6 +1887,7 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     q.gy = gy;
     q.x = xk;
     q.partial = partial;
+    q.biasPartial = biasPartial;
     q.M = g.Cout;
     q.Ncols = g.K;
     q.mTiles = mT;
@@ -1890,11 +1922,16 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     convGemmKernel<kGradWeight><<<grid, dev::kBlock, 0, s>>>(p, g);
   }
   THC_HIP_CHECK(hipGetLastError());
-  if (count % 4 == 0 && launch::aligned16(gW) && launch::aligned16(partial))
-    foldPartials4Kernel<<<(unsigned)((count / 4 + 63) / 64), dev::kBlock, 0, s>>>(partial, gW, count / 4, splits, scale);
-  else
+  if (fold4) {  // (the scratch starts on a 16-byte boundary)
+    const int gwBlocks = (int)((count / 4 + 63) / 64);
+    const int biasBlocks = fusedBias ? launch::ceilDiv(g.Cout / 4, 64) : 0;
+    foldPartials4Kernel<<<gwBlocks + biasBlocks, dev::kBlock, 0, s>>>(partial, gW, count / 4, splits, scale, biasPartial,
+                                                                       gB, g.Cout, gwBlocks);
+  } else {
     foldPartialsKernel<<<launch::directGrid(count, dev::kBlock), dev::kBlock, 0, s>>>(partial, gW, count, splits, scale);
+  }
   THC_HIP_CHECK(hipGetLastError());
+  if (gB && !fusedBias) convGradBias(s, gy, gB, g.N, g.Cout, g.L, scale);
 }
 
 // ---- entry-point bodies shared by SpatialConvolutionMM and SpatialDilatedConvolution --------
@@ -1939,8 +1976,7 @@ void convAccGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *g
   ConvGeom &g = call.g;
   Contiguous in(state, input);
   Contiguous go(state, gradOutput);
-  convGradWeight(state, g, in.ptr(), go.ptr(), data(gradWeight), columns, scale);
-  if (gradBias) convGradBias(state->stream, go.ptr(), data(gradBias), g.N, g.Cout, g.L, scale);
+  convGradWeight(state, g, in.ptr(), go.ptr(), data(gradWeight), columns, scale, gradBias ? data(gradBias) : nullptr);
 }
 
 // ---- transposed ("full") convolution -----------------------------------------------------------

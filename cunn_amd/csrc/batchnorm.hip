@@ -16,6 +16,8 @@
 // lib/THCUNN/BatchNormalization.cu:214-283.
 #include <cmath>
 
+#include <atomic>
+
 #include "device_utils.h"
 #include "launch_utils.h"
 #include "thc_internal.h"
@@ -725,6 +727,14 @@ void checkVector(const THCudaTensor *t, const char *name, int C, bool required) 
 
 inline float *dataOrNull(const THCudaTensor *t) { return t ? data(t) : nullptr; }
 
+constexpr int kMaxDevices = 64;
+inline int currentDevice() {
+  int dv = 0;
+  THC_HIP_CHECK(hipGetDevice(&dv));
+  if (dv < 0 || dv >= kMaxDevices) error("BatchNormalization: device ordinal %d not supported", dv);
+  return dv;
+}
+
 // The resident kernels hold a channel in the registers of one 1024-lane
 // workgroup: at most maxR float4 per lane, and enough channels to occupy the chip.
 int residentR(const BnView &v, int maxR) {
@@ -887,11 +897,13 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
     const int xlds = (RR > 8 && train && gxp) ? 8 : 0;                                                             \
     const size_t lds = (size_t)xlds * kResBlock * sizeof(float4);                                                  \
     if (train) {                                                                                                   \
-      static bool ldsRaised = false; /* once per kernel instance: allow more than 64 KB of dynamic LDS */         \
-      if (lds && !ldsRaised) {                                                                                     \
+      /* once per kernel instance and device: allow more than 64 KB of dynamic LDS */                             \
+      static std::atomic<bool> ldsRaised[kMaxDevices];                                                             \
+      const int dv = currentDevice();                                                                              \
+      if (lds && !ldsRaised[dv].load()) {                                                                          \
         THC_HIP_CHECK(hipFuncSetAttribute((const void *)bnBwdResident<RR, true, (RR <= 8)>,                        \
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                  \
-        ldsRaised = true;                                                                                          \
+        ldsRaised[dv].store(true);                                                                                 \
       }                                                                                                            \
       bnBwdResident<RR, true, (RR <= 8)><<<g.C, kResBlock, lds, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_), \
                                                         dataOrNull(gradBias_), dataOrNull(weight_), meanSrc,       \

@@ -1346,16 +1346,16 @@ inline unsigned tiles(long n, int b) { return (unsigned)((n + b - 1) / b); }
 // kernel == nullptr: the number of CUs.
 int residentSlots(const void *kernel) {
   static std::mutex mu;
-  static std::map<const void *, int> cache;
-  std::lock_guard<std::mutex> lock(mu);
-  auto it = cache.find(kernel);
-  if (it != cache.end()) return it->second;
+  static std::map<std::pair<int, const void *>, int> cache;  // per (device, kernel)
   int dev = 0, cus = 0, perCu = 1;
   THC_HIP_CHECK(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = cache.find({dev, kernel});
+  if (it != cache.end()) return it->second;
   THC_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
   if (kernel) THC_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, kernel, dev::kBlock, 0));
   int v = std::max(1, cus) * std::max(1, perCu);
-  cache[kernel] = v;
+  cache[{dev, kernel}] = v;
   return v;
 }
 

@@ -264,6 +264,44 @@ def test_dwconv_transposed_gradweight_view(T):
     close(base.numpy().transpose(1, 0, 2, 3), rgw, WG_RTOL, WG_ATOL)
 
 
+def test_dwconv_small_planes_variants(T):
+    """The several-planes-per-workgroup kernels behind the other ways of calling the module: no bias, a
+    non-contiguous input, a 3-D input with a 2-D weight, gradWeight and gradBias through transposed views."""
+    THNN, CT = T.THNN, T.CudaTensor
+    case = (3, 20, 1, 14, 14, 3, 3, 2, 2, 1, 1)
+    rng, x, w, _ = _dw_inputs(case, 15, bias=False)
+    _dw_run(T, case, x, w, None, scale=2.0, gw0=rng.standard_normal(w.shape).astype(np.float32))
+    rng, x, w, b = _dw_inputs(case, 16)
+    _dw_run(T, case, x, w, b, xt=CT.noncontiguous_from_numpy(x, rng))
+    # 3-D input, 2-D weight
+    C, H, W, k = 20, 7, 7, 3
+    x3 = rng.standard_normal((C, H, W)).astype(np.float32)
+    w4 = rng.standard_normal((1, C, k, k)).astype(np.float32)
+    b2 = rng.standard_normal((1, C)).astype(np.float32)
+    tw, out = CT.from_numpy(w4.reshape(1, C * k * k)), CT()
+    THNN.SpatialDepthWiseConvolution_updateOutput(CT.from_numpy(x3), out, tw, CT.from_numpy(b2), CT(), CT(), k, k, 1, 1, 1, 1)
+    assert out.size() == (C, H, W)
+    close(out.numpy(), O.dwconv_updateOutput(x3[None], w4, b2, k, k, 1, 1, 1, 1)[0])
+    gy3 = rng.standard_normal((C, H, W)).astype(np.float32)
+    gi = CT()
+    THNN.SpatialDepthWiseConvolution_updateGradInput(CT.from_numpy(x3), CT.from_numpy(gy3), gi, tw, CT(), CT(), k, k, 1, 1, 1, 1)
+    assert gi.size() == (C, H, W)
+    close(gi.numpy(), O.dwconv_updateGradInput((1, C, H, W), gy3[None], w4, k, k, 1, 1, 1, 1)[0])
+    # gradWeight as a (1, C, k, k) view of memory in (C, k, k) order with a gap between channels; gradBias likewise
+    gw0 = rng.standard_normal((1, C, k, k)).astype(np.float32)
+    basew = CT.from_numpy(np.zeros((C, 2 * k * k), np.float32))
+    hw = basew.numpy(); hw[:, :k * k] = gw0[0].reshape(C, k * k)
+    basew = CT.from_numpy(hw)
+    vieww = basew.view(0, (1, C, k, k), (0, 2 * k * k, k, 1))
+    gb0 = rng.standard_normal((1, C)).astype(np.float32)
+    THNN.SpatialDepthWiseConvolution_accGradParameters(CT.from_numpy(x3), CT.from_numpy(gy3), vieww, CT.from_numpy(gb0.copy()),
+                                                       CT(), CT(), k, k, 1, 1, 1, 1, 0.5)
+    rgw, _ = O.dwconv_accGradParameters(x3[None], gy3[None], gw0.copy(), gb0.copy(), k, k, 1, 1, 1, 1, 0.5)
+    got = basew.numpy()
+    close(got[:, :k * k].reshape(1, C, k, k), rgw, WG_RTOL, WG_ATOL)
+    assert np.all(got[:, k * k:] == 0)
+
+
 def test_dwconv_shape_errors(T):
     THNN, CT = T.THNN, T.CudaTensor
     x = CT.from_numpy(np.zeros((2, 3, 8, 8), np.float32))

@@ -1,0 +1,49 @@
+"""Seeded random geometries for the kernels that put several small planes in one workgroup
+(depthwise convolution, pooling, batch normalization with plane sizes that are not a multiple
+of 4): plane sizes 1..32 on either side of every internal threshold, plane counts that leave the
+last workgroup partly filled. Same tolerances as the fixed cases."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from oracle import oracle as O  # noqa: E402
+from test_gpu_parity import (T, close, _dw_run, _dw_inputs, _maxpool_run, _avgpool_run, _tied_input,  # noqa: E402,F401
+                             _bn_run)
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_dwconv_small_random(T, seed):
+    rng = np.random.default_rng(3000 + seed)
+    k = int(rng.choice([3, 5]))
+    s = int(rng.choice([1, 2]))
+    H, W = (int(v) for v in rng.integers(1, 33, 2))
+    N, C = int(rng.integers(1, 6)), int(rng.integers(1, 90))
+    case = (N, C, 1, H, W, k, k, s, s, k // 2, k // 2)
+    _, x, w, b = _dw_inputs(case, 3100 + seed)
+    _dw_run(T, case, x, w, b if seed % 3 else None, scale=float(rng.choice([1.0, 0.25])))
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_pool_small_random(T, seed):
+    rng = np.random.default_rng(4000 + seed)
+    while True:
+        kW, kH = (int(v) for v in rng.integers(1, 5, 2))
+        dW, dH = (int(v) for v in rng.integers(1, 4, 2))
+        pW, pH = int(rng.integers(0, kW // 2 + 1)), int(rng.integers(0, kH // 2 + 1))
+        H, W = (int(v) for v in rng.integers(1, 33, 2))
+        if H + 2 * pH >= kH and W + 2 * pW >= kW:
+            break
+    ceil = bool(rng.integers(0, 2))
+    N, C = int(rng.integers(1, 5)), int(rng.integers(1, 70))
+    case = (N, C, H, W, kW, kH, dW, dH, pW, pH, ceil)
+    _maxpool_run(T, case, _tied_input(case[:4], 4100 + seed, q=8))
+    _avgpool_run(T, case, bool(seed % 2), seed=4200 + seed)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_batchnorm_small_random(T, seed):
+    rng = np.random.default_rng(5000 + seed)
+    H, W = (int(v) for v in rng.integers(1, 12, 2))
+    N, C = int(rng.integers(1, 80)), int(rng.integers(96, 140))
+    _bn_run(T, (N, C, H, W), bool(seed % 2), seed=5100 + seed)

@@ -780,12 +780,16 @@ int gradInputExtraRows(int ks, int st) {
 // ---- small planes: several planes per workgroup (dwconv_small.h) ----------------------------
 enum SmallPass { kSmallFwd, kSmallGradInput, kSmallAccGrad };
 
-// Planes of at most 1024 elements take these kernels (measured faster than the strip kernels up to 28x28, and
-// the strip kernels need widths that are multiples of 4). Test switch THCUNN_DW_SMALL=0: never.
+// Planes of at most 1024 elements take these kernels, several per workgroup (measured faster than the strip
+// kernels up to 28x28), and so do larger planes whose width or output width is not a multiple of 4 (which
+// the strip kernels need): two per workgroup up to 2048 elements, a band of rows per workgroup beyond. Test switch THCUNN_DW_SMALL: 0 never, 1 also for
+// the larger planes that the strip kernels could take.
 int smallSwitch() {
   const char *e = getenv("THCUNN_DW_SMALL");
   return e ? atoi(e) : -1;
 }
+
+constexpr int kSmallPlane = 1024;
 
 // Plans a small-plane launch; false when the geometry is outside what those kernels are compiled for.
 bool smallPlan(const DwGeom &g, SmallPass pass, SmallGeom *out, int *rw, size_t *lds) {
@@ -794,35 +798,107 @@ bool smallPlan(const DwGeom &g, SmallPass pass, SmallGeom *out, int *rw, size_t 
       g.padH != g.kH / 2)
     return false;
   const int HW = g.H * g.W, oHW = g.oH * g.oW;
-  if (HW > 1024 || oHW < 1) return false;
-  const int PAD = g.kH / 2;
+  if (oHW < 1 || (long)g.N * g.C >= 0x7fffffffL / 64) return false;
+  const int PAD = g.kH / 2, KS = g.kH, st = g.dH;
   SmallGeom sg{};
   sg.C = g.C, sg.planes = g.N * g.C;
   if (pass == kSmallGradInput)
     sg.sH = g.oH, sg.sW = g.oW, sg.oH = g.H, sg.oW = g.W;
   else
     sg.sH = g.H, sg.sW = g.W, sg.oH = g.oH, sg.oW = g.oW;
-  sg.LH = g.H + 2 * PAD, sg.LW = (g.W + 2 * PAD) | 1;  // odd pitch: the rows a wave reads start in different banks
-  const int second = pass == kSmallGradInput ? HW : oHW;  // output run (forward, gradInput) / gradOutput run (accGrad)
-  auto xsFloats = [&](int P) { return roundUp(P * sg.LH * sg.LW + 7 * 2 + g.kH, 4); };  // slack: the widest item's overrun
-  int P = 64;  // at least 4: the lanes of a plane stay inside one wave
-  while (P > 4 && (P * HW > launch::kBatchFloats || (size_t)(xsFloats(P) + P * second) * sizeof(float) > launch::kLdsMax)) P >>= 1;
-  if (P * HW > launch::kBatchFloats || (size_t)(xsFloats(P) + P * second) * sizeof(float) > launch::kLdsMax) return false;
-  if ((P * HW) % 4 != 0 || (P * oHW) % 4 != 0) return false;  // every workgroup's runs start on 16 bytes
-  sg.P = P, sg.lp = dev::kBlock / P;
+  sg.srcFloats = (long)sg.planes * sg.sH * sg.sW, sg.outFloats = (long)sg.planes * sg.oH * sg.oW;
+  sg.LW = (g.W + 2 * PAD) | 1;  // row pitch for sizing; the final one (up to 8 more) is chosen below
+  const int CS = pass == kSmallGradInput ? 1 : st, DS = pass == kSmallGradInput ? st : 1;  // compute stride, staging dilation
+  const int kRun = launch::kBatchFloats - 3;  // floats of a run (one batch of 16-byte loads, incl. up to 3 in front of it)
+  const int kSlack = 7 * 2 + KS;              // LDS floats the widest work item may read past the last staged row
+  int secondFloats = 0;                       // second LDS buffer: output run (forward, gradInput) / gradOutput run (accGrad)
+  if (HW <= kSmallPlane || (HW <= 2 * kSmallPlane && !stripGeometry(g))) {
+    // several whole planes per workgroup, at least 2
+    sg.bands = 1, sg.rowsPerBand = sg.oH;
+    sg.LH = g.H + 2 * PAD;
+    const int second = pass == kSmallGradInput ? HW : oHW;
+    auto bytes = [&](int P) { return (size_t)(roundUp(P * sg.LH * sg.LW + kSlack, 4) + roundUp(P * second + 4, 4)) * sizeof(float); };
+    // a workgroup's runs start at multiples of P planes: on a 16-byte boundary if P planes are a multiple of 4 floats
+    auto fetched = [&](int n) { return n + (n % 4 ? 3 : 0); };
+    auto fits = [&](int P) { return fetched(P * HW) <= launch::kBatchFloats && fetched(P * oHW) <= launch::kBatchFloats && bytes(P) <= launch::kLdsMax; };
+    int P = 64;
+    while (P > 2 && !fits(P)) P >>= 1;
+    if (fits(P)) {
+      sg.P = P;
+      sg.xsFloats = roundUp(P * sg.LH * sg.LW + kSlack, 4);
+      secondFloats = roundUp(P * second + 4, 4);
+    }
+  }
+  if (sg.P == 0) {
+    // a band of rows of one plane per workgroup: for the widths the strip kernels do not take
+    if (smallSwitch() != 1 && stripGeometry(g)) return false;
+    sg.P = 1;
+    // produced rows per band: the source rows behind them and the produced rows themselves are one run each
+    auto srcRows = [&](int rows) { return ((rows - 1) * CS + KS - 1) / DS + 1; };
+    auto fits = [&](int rows) {
+      const int LHb = (rows - 1) * CS + KS;
+      const size_t b = (size_t)(roundUp(LHb * sg.LW + kSlack, 4) + roundUp(rows * sg.oW + 4, 4)) * sizeof(float);
+      return srcRows(rows) * sg.sW <= kRun && rows * sg.oW <= kRun && b <= 48 * 1024;
+    };
+    if (!fits(1)) return false;
+    int rows = 1;
+    while (rows < sg.oH && fits(rows + 1)) ++rows;
+    sg.bands = ceilDiv(sg.oH, rows);
+    sg.rowsPerBand = ceilDiv(sg.oH, sg.bands);
+    if ((long)sg.planes * sg.bands >= 0x7fffffffL) return false;
+    sg.LH = (sg.rowsPerBand - 1) * CS + KS;
+    sg.xsFloats = roundUp(sg.LH * sg.LW + kSlack, 4);
+    secondFloats = roundUp(sg.rowsPerBand * sg.oW + 4, 4);
+  }
+  sg.lp = dev::kBlock / sg.P;
   for (sg.lpShift = 0; (1 << sg.lpShift) < sg.lp; ++sg.lpShift) {
   }
-  sg.xsFloats = xsFloats(P);
-  // outputs per work item: 7 or 4 consecutive ones of a row, whichever needs fewer lane-steps for a plane
-  // (rounds over the plane's lanes x (outputs + the window's extra columns))
-  auto steps = [&](int r) { return ceilDiv(sg.oH * ceilDiv(sg.oW, r), sg.lp) * (r + 2); };
-  *rw = steps(7) <= steps(4) ? 7 : 4;
-  sg.nseg = ceilDiv(sg.oW, *rw);
+  // Outputs per work item (7 or 4 consecutive ones of a row) and row pitch in LDS: the pair with the fewest
+  // LDS read cycles = lane-steps (rounds over the lanes that share a plane x (outputs + the window's extra
+  // columns)) x the most lanes of a wave that read the same bank at one window column. The last choice
+  // is kept per pass and thread: the search costs a few microseconds.
+  struct Choice {
+    int oW, rows, lp, LH, CS, base, room, rw, LW;
+  };
+  static thread_local Choice last[3] = {};
+  const int base = g.W + 2 * PAD;
+  const int room = (int)((launch::kLdsMax / sizeof(float) - secondFloats - kSlack - 4) / ((size_t)sg.P * sg.LH));  // widest pitch that fits
+  Choice &ch = last[pass];
+  if (ch.rw == 0 || ch.oW != sg.oW || ch.rows != sg.rowsPerBand || ch.lp != sg.lp || ch.LH != sg.LH || ch.CS != CS || ch.base != base ||
+      ch.room != room) {
+    ch = Choice{sg.oW, sg.rowsPerBand, sg.lp, sg.LH, CS, base, room, 0, 0};
+    long best = 0;
+    for (int LW = base; LW <= std::min(base + 8, std::max(room, sg.LW)); ++LW)
+      for (int r : {7, 4}) {
+        // accGradParameters runs the items that end past the row in a pass of their own
+        const bool split = pass == kSmallAccGrad && sg.oW % r != 0 && sg.oW > r;
+        const int nseg = split ? sg.oW / r : ceilDiv(sg.oW, r), items = sg.rowsPerBand * nseg;
+        unsigned char lanes[64] = {};
+        int worst = 1;
+        for (int tid = 0; tid < dev::kWave; ++tid) {
+          const int pl = tid >> sg.lpShift, it = tid & (sg.lp - 1);
+          if (it >= items) continue;
+          const int row = it / nseg, c0 = (it - row * nseg) * r;
+          worst = std::max(worst, (int)++lanes[(pl * sg.LH * LW + row * CS * LW + c0 * CS) & 63]);
+        }
+        const long cost = (long)(ceilDiv(items, sg.lp) + (split ? ceilDiv(sg.rowsPerBand, sg.lp) : 0)) * (r + 2) * worst;
+        if (ch.rw == 0 || cost < best) best = cost, ch.rw = r, ch.LW = LW;
+      }
+  }
+  *rw = ch.rw;
+  sg.LW = ch.LW;
+  sg.xsFloats = roundUp(sg.P * sg.LH * sg.LW + kSlack, 4);
+  sg.nseg = ceilDiv(sg.oW, *rw), sg.nfull = sg.oW / *rw;
   sg.magicC = dev::magicOf(g.C), sg.magicSPlane = dev::magicOf(sg.sH * sg.sW), sg.magicSW = dev::magicOf(sg.sW);
-  sg.magicSeg = dev::magicOf(sg.nseg);
+  sg.magicSeg = dev::magicOf(sg.nseg), sg.magicFull = dev::magicOf(std::max(sg.nfull, 1)), sg.magicBands = dev::magicOf(sg.bands);
   *out = sg;
-  *lds = (size_t)(sg.xsFloats + P * second) * sizeof(float);
+  *lds = (size_t)(sg.xsFloats + secondFloats) * sizeof(float);
   return true;
+}
+
+// workgroups of a small-plane launch
+inline unsigned smallGrid(const SmallGeom &sg) {
+  return sg.bands == 1 ? (unsigned)ceilDiv(sg.planes, sg.P) : (unsigned)((long)sg.planes * sg.bands);
 }
 
 #define DW_SMALL_CONV(CS, DS, FLIP, ...)                                                                          \
@@ -871,7 +947,7 @@ void THNN_CudaSpatialDepthWiseConvolution_updateOutput(THCState *state, THCudaTe
     int rw;
     size_t lds;
     if (aligned16(in.ptr()) && aligned16(data(output)) && smallPlan(g, kSmallFwd, &sg, &rw, &lds)) {
-      const dim3 grid(ceilDiv(sg.planes, sg.P));
+      const dim3 grid(smallGrid(sg));
       if (g.dH == 1)
         DW_SMALL_CONV(1, 1, false, in.ptr(), data(weight), strides4(weight), bptr, strides2(bias), data(output), sg);
       else
@@ -946,7 +1022,7 @@ void THNN_CudaSpatialDepthWiseConvolution_updateGradInput(THCState *state, THCud
     int rw;
     size_t lds;
     if (aligned16(go.ptr()) && aligned16(data(gradInput)) && smallPlan(g, kSmallGradInput, &sg, &rw, &lds)) {
-      const dim3 grid(ceilDiv(sg.planes, sg.P));
+      const dim3 grid(smallGrid(sg));
       const Strides2 nob{0, 0};
       if (g.dH == 1)
         DW_SMALL_CONV(1, 1, true, go.ptr(), data(weight), strides4(weight), nullptr, nob, data(gradInput), sg);
@@ -1026,15 +1102,17 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
       // one partial per (channel, tap, image); scratch as in the general case below
       Temp tmp;
       float *partial;
+      const long nslots = (long)g.N * sg.bands;
+      if (nslots >= 0x7fffffffL) error("SpatialDepthWiseConvolution: batch too large");
       if (columns) {
-        resize(state, columns, {(long)g.C * T, g.N});
+        resize(state, columns, {(long)g.C * T, nslots});
         if (!isContiguous(erase(columns))) error("columns tensor has to be contiguous");
         partial = data(columns);
       } else {
-        tmp = Temp(s, (size_t)g.C * T * g.N * sizeof(float));
+        tmp = Temp(s, (size_t)g.C * T * nslots * sizeof(float));
         partial = (float *)tmp.get();
       }
-      const dim3 grid(ceilDiv(sg.planes, sg.P));
+      const dim3 grid(smallGrid(sg));
       if (g.dH == 1)
         DW_SMALL_ACC(1, in.ptr(), go.ptr(), partial, sg, g.N);
       else
@@ -1042,7 +1120,7 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
       THC_HIP_CHECK(hipGetLastError());
       const int pairs = g.C * T;
       dwAccGradStage2<<<ceilDiv(pairs, dev::kBlock / dev::kWave), dev::kBlock, 0, s>>>(
-          partial, data(gradWeight), strides4(gradWeight), gbPtr, strides2(gradBias), 1, g.kW, T, g.N, scale, pairs);
+          partial, data(gradWeight), strides4(gradWeight), gbPtr, strides2(gradBias), 1, g.kW, T, (int)nslots, scale, pairs);
       THC_HIP_CHECK(hipGetLastError());
       return;
     }

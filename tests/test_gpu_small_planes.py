@@ -1,7 +1,8 @@
 """Seeded random geometries for the kernels that put several small planes in one workgroup
 (depthwise convolution, pooling, batch normalization with plane sizes that are not a multiple
 of 4): plane sizes 1..32 on either side of every internal threshold, plane counts that leave the
-last workgroup partly filled. Same tolerances as the fixed cases."""
+last workgroup partly filled; and for the depthwise kernels that cut a larger plane of any width into
+bands of rows. Same tolerances as the fixed cases."""
 import numpy as np
 import pytest
 
@@ -22,6 +23,42 @@ def test_dwconv_small_random(T, seed):
     case = (N, C, 1, H, W, k, k, s, s, k // 2, k // 2)
     _, x, w, b = _dw_inputs(case, 3100 + seed)
     _dw_run(T, case, x, w, b if seed % 3 else None, scale=float(rng.choice([1.0, 0.25])))
+
+
+# fixed shapes: network planes of odd width, a plane one row over the several-planes limit, rows so wide
+# that a band is a single row, and the 5x5 window where a band's first rows lie in the border
+DW_BAND_CASES = [
+    (2, 3, 1, 147, 147, 3, 3, 1, 1, 1, 1),
+    (1, 4, 1, 150, 150, 3, 3, 2, 2, 1, 1),
+    (2, 2, 1, 75, 75, 5, 5, 2, 2, 2, 2),
+    (1, 5, 1, 37, 37, 5, 5, 1, 1, 2, 2),
+    (1, 3, 1, 33, 32, 3, 3, 1, 1, 1, 1),      # oW % 4 == 0 but taken as bands only if the strip kernels do not
+    (1, 2, 1, 3, 2045, 3, 3, 1, 1, 1, 1),
+    (1, 2, 1, 5, 1366, 5, 5, 2, 2, 2, 2),
+    (1, 2, 1, 600, 3, 5, 5, 2, 2, 2, 2),
+    (1, 1, 1, 1, 1025, 3, 3, 2, 2, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", DW_BAND_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_dwconv_bands(T, case):
+    _, x, w, b = _dw_inputs(case, 3500)
+    _dw_run(T, case, x, w, b)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_dwconv_bands_random(T, seed, monkeypatch):
+    rng = np.random.default_rng(3600 + seed)
+    k = int(rng.choice([3, 5]))
+    s = int(rng.choice([1, 2]))
+    H, W = (int(v) for v in rng.integers(20, 260, 2))
+    if seed % 4 == 3:  # also the widths the strip kernels would take
+        monkeypatch.setenv("THCUNN_DW_SMALL", "1")
+        W = W // 8 * 8 + 8
+    N, C = int(rng.integers(1, 3)), int(rng.integers(1, 5))
+    case = (N, C, 1, H, W, k, k, s, s, k // 2, k // 2)
+    _, x, w, b = _dw_inputs(case, 3700 + seed)
+    _dw_run(T, case, x, w, b if seed % 3 else None, scale=float(rng.choice([1.0, 0.5])))
 
 
 @pytest.mark.parametrize("seed", range(30))

@@ -853,38 +853,10 @@ bool smallPlan(const DwGeom &g, SmallPass pass, SmallGeom *out, int *rw, size_t 
   sg.lp = dev::kBlock / sg.P;
   for (sg.lpShift = 0; (1 << sg.lpShift) < sg.lp; ++sg.lpShift) {
   }
-  // Outputs per work item (7 or 4 consecutive ones of a row) and row pitch in LDS: the pair with the fewest
-  // LDS read cycles = lane-steps (rounds over the lanes that share a plane x (outputs + the window's extra
-  // columns)) x the most lanes of a wave that read the same bank at one window column. The last choice
-  // is kept per pass and thread: the search costs a few microseconds.
-  struct Choice {
-    int oW, rows, lp, LH, CS, base, room, rw, LW;
-  };
-  static thread_local Choice last[3] = {};
   const int base = g.W + 2 * PAD;
   const int room = (int)((launch::kLdsMax / sizeof(float) - secondFloats - kSlack - 4) / ((size_t)sg.P * sg.LH));  // widest pitch that fits
-  Choice &ch = last[pass];
-  if (ch.rw == 0 || ch.oW != sg.oW || ch.rows != sg.rowsPerBand || ch.lp != sg.lp || ch.LH != sg.LH || ch.CS != CS || ch.base != base ||
-      ch.room != room) {
-    ch = Choice{sg.oW, sg.rowsPerBand, sg.lp, sg.LH, CS, base, room, 0, 0};
-    long best = 0;
-    for (int LW = base; LW <= std::min(base + 8, std::max(room, sg.LW)); ++LW)
-      for (int r : {7, 4}) {
-        // accGradParameters runs the items that end past the row in a pass of their own
-        const bool split = pass == kSmallAccGrad && sg.oW % r != 0 && sg.oW > r;
-        const int nseg = split ? sg.oW / r : ceilDiv(sg.oW, r), items = sg.rowsPerBand * nseg;
-        unsigned char lanes[64] = {};
-        int worst = 1;
-        for (int tid = 0; tid < dev::kWave; ++tid) {
-          const int pl = tid >> sg.lpShift, it = tid & (sg.lp - 1);
-          if (it >= items) continue;
-          const int row = it / nseg, c0 = (it - row * nseg) * r;
-          worst = std::max(worst, (int)++lanes[(pl * sg.LH * LW + row * CS * LW + c0 * CS) & 63]);
-        }
-        const long cost = (long)(ceilDiv(items, sg.lp) + (split ? ceilDiv(sg.rowsPerBand, sg.lp) : 0)) * (r + 2) * worst;
-        if (ch.rw == 0 || cost < best) best = cost, ch.rw = r, ch.LW = LW;
-      }
-  }
+  const launch::ItemChoice ch = launch::pickItem(pass, sg.oW, sg.rowsPerBand, sg.lp, sg.lpShift, sg.LH, CS, base,
+                                                 std::max(room, sg.LW), pass == kSmallAccGrad);
   *rw = ch.rw;
   sg.LW = ch.LW;
   sg.xsFloats = roundUp(sg.P * sg.LH * sg.LW + kSlack, 4);

@@ -420,6 +420,8 @@ poolBwdSmall(const float *__restrict__ gradOut, const long *__restrict__ indices
   }
 }
 
+#include "pooling_runs.h"
+
 // ============================================================ strip kernels ==
 // Fast paths for square windows without dilation whose geometry (KS, ST, PAD) is
 // known at compile time and whose rows are multiples of 4 (see strip.h). A lane
@@ -794,6 +796,145 @@ size_t fwdStripFloats(const PoolGeom &g, int rows) {
   return 0;
 }
 
+// ---- runs of memory (pooling_runs.h) ------------------------------------------------
+// The strip kernels' window geometries on planes of any width: several whole planes per workgroup
+// (planes of at most 2048 elements) or a band of rows of a larger plane. Test switch
+// THCUNN_POOL_RUNS: 0 never, 1 also where the strip kernels would be chosen.
+struct PoolRunPlan {
+  SmallGeom sg;
+  int rw, secondFloats;
+  size_t lds;
+};
+
+template <int KS, int ST, int PAD>
+bool poolRunPlanFor(const PoolGeom &g, long planes, bool backward, bool max, PoolRunPlan *out) {
+  using R = PoolReach<KS, ST, PAD>;
+  using launch::ceilDiv;
+  using launch::roundUp;
+  const int HW = g.H * g.W, oHW = g.oH * g.oW;
+  if (planes >= 0x7fffffffL / 64 || HW < 1 || oHW < 1) return false;
+  SmallGeom sg{};
+  sg.C = 1, sg.planes = (int)planes;
+  if (backward)
+    sg.sH = g.oH, sg.sW = g.oW, sg.oH = g.H, sg.oW = g.W;
+  else
+    sg.sH = g.H, sg.sW = g.W, sg.oH = g.oH, sg.oW = g.oW;
+  sg.srcFloats = planes * sg.sH * sg.sW, sg.outFloats = planes * sg.oH * sg.oW;
+  const int kRun = launch::kBatchFloats - 3;  // a run and up to 3 floats in front of it are one batch of 16-byte loads
+  const int nIdx = max ? 2 : 1;               // max pooling keeps a 32-bit plane of argmax positions beside the values
+  auto fetched = [&](int n) { return n + (n % 4 ? 3 : 0); };  // runs of whole planes start on 16-byte boundaries if P planes do
+  const int kSlack = backward ? 4 : 7 * ST + KS;  // floats the widest forward item may read past the last staged row
+  // staged plane (or band of `rows` produced rows) with its border
+  const int LW0 = backward ? std::max(R::BT + sg.sW, (4 * (ceilDiv(g.W, 4) - 1)) / ST + R::first(3) + R::NC) | 1
+                           : std::max(PAD + g.W, (g.oW - 1) * ST + KS) | 1;
+  const int LHplanes = backward ? std::max(R::BT + sg.sH, R::first(g.H - 1) + R::NC) : std::max(PAD + g.H, (g.oH - 1) * ST + KS);
+  auto LHband = [&](int rows) { return backward ? (rows + ST - 2) / ST + R::NC : (rows - 1) * ST + KS; };
+  // LDS floats: forward staged planes | values | argmax; backward staged gradOutput | staged argmax | gradInput run
+  auto ldsFloats = [&](int P, int LH, int producedPerPlane) {
+    const int staged = roundUp(P * LH * LW0 + kSlack, 4), second = roundUp(P * producedPerPlane + 4, 4);
+    return (size_t)(backward ? nIdx * staged + second : staged + nIdx * second);
+  };
+  const int producedPlane = sg.oH * sg.oW, srcPlane = sg.sH * sg.sW;
+  if (std::max(HW, oHW) <= 2048) {
+    auto fits = [&](int P) {
+      return fetched(P * srcPlane) <= launch::kBatchFloats && fetched(P * producedPlane) <= launch::kBatchFloats &&
+             ldsFloats(P, LHplanes, producedPlane) * sizeof(float) <= launch::kLdsMax;
+    };
+    int P = 64;
+    while (P > 2 && !fits(P)) P >>= 1;
+    if (fits(P)) {
+      sg.P = P, sg.bands = 1, sg.rowsPerBand = sg.oH, sg.LH = LHplanes;
+    }
+  }
+  if (sg.P == 0) {
+    auto fits = [&](int rows) {
+      const int srcRows = std::min(sg.sH, LHband(rows));
+      return srcRows * sg.sW <= kRun && rows * sg.oW <= kRun &&
+             ldsFloats(1, LHband(rows), rows * sg.oW) * sizeof(float) <= 48 * 1024;
+    };
+    if (!fits(1)) return false;
+    int rows = 1;
+    while (rows < sg.oH && fits(rows + 1)) ++rows;
+    sg.P = 1, sg.bands = ceilDiv(sg.oH, rows);
+    sg.rowsPerBand = ceilDiv(sg.oH, sg.bands);
+    if (planes * sg.bands >= 0x7fffffffL) return false;
+    sg.LH = LHband(sg.rowsPerBand);
+  }
+  sg.lp = dev::kBlock / sg.P;
+  for (sg.lpShift = 0; (1 << sg.lpShift) < sg.lp; ++sg.lpShift) {
+  }
+  const int second = roundUp(sg.P * sg.rowsPerBand * sg.oW + 4, 4);
+  sg.LW = LW0;
+  int rw = 4;
+  if (!backward) {
+    const int room = (int)((launch::kLdsMax / sizeof(float) - nIdx * second - kSlack - 4) / ((size_t)sg.P * sg.LH));
+    const launch::ItemChoice ch = launch::pickItem(3 + (max ? 1 : 0), sg.oW, sg.rowsPerBand, sg.lp, sg.lpShift, sg.LH, ST,
+                                                   LW0 & ~1, std::max(room, LW0), false);
+    rw = ch.rw, sg.LW = std::max(ch.LW, std::max(PAD + g.W, (g.oW - 1) * ST + KS));
+  }
+  sg.xsFloats = roundUp(sg.P * sg.LH * sg.LW + kSlack, 4);
+  sg.nseg = ceilDiv(sg.oW, rw), sg.nfull = sg.oW / rw;
+  sg.magicC = dev::magicOf(1), sg.magicSPlane = dev::magicOf(srcPlane), sg.magicSW = dev::magicOf(sg.sW);
+  sg.magicSeg = dev::magicOf(sg.nseg), sg.magicFull = dev::magicOf(std::max(sg.nfull, 1)), sg.magicBands = dev::magicOf(sg.bands);
+  out->sg = sg, out->rw = rw, out->secondFloats = second;
+  out->lds = (size_t)(backward ? nIdx * sg.xsFloats + second : sg.xsFloats + nIdx * second) * sizeof(float);
+  return out->lds <= launch::kLdsMax;
+}
+
+int runSwitch() {
+  const char *e = getenv("THCUNN_POOL_RUNS");
+  return e ? atoi(e) : -1;
+}
+// Where both families apply (widths that are multiples of 4), measured on 8x8 ... 224x224 planes: the run
+// kernels' max forward is never slower (16x16: 44 -> 12 us, 112x112: 64 -> 62 us); the average forward wins
+// up to 28x28 and the backward passes up to about 36x36 (a plane per workgroup leaves the strip kernels'
+// lanes idle there), beyond that the strip kernels' backward is 10-20 % faster.
+bool runsFirst(const PoolGeom &g, bool backward, bool max) {
+  if (runSwitch() >= 0) return runSwitch() == 1;
+  const long plane = std::max((long)g.H * g.W, (long)g.oH * g.oW);
+  if (backward) return plane <= 2048;
+  return max || plane <= 1024;
+}
+
+bool poolRunPlan(const PoolGeom &g, long planes, bool backward, bool max, PoolRunPlan *out) {
+  if (forcedPath() != 0 || runSwitch() == 0 || !stripCombo(g)) return false;
+#define X(K, S, P) \
+  if (g.kH == K && g.dH == S && g.padH == P) return poolRunPlanFor<K, S, P>(g, planes, backward, max, out);
+  POOL_STRIP_COMBOS(X)
+#undef X
+  return false;
+}
+
+inline unsigned poolRunGrid(const SmallGeom &sg) {
+  return sg.bands == 1 ? (unsigned)launch::ceilDiv(sg.planes, sg.P) : (unsigned)((long)sg.planes * sg.bands);
+}
+
+template <bool MAX>
+void launchPoolRunFwd(hipStream_t s, const PoolGeom &g, const PoolRunPlan &pl, const float *in, float *out, long *indices,
+                      bool includePad) {
+  const dim3 grid(poolRunGrid(pl.sg));
+#define X(K, S, P)                                                                                                        \
+  if (g.kH == K && g.dH == S && g.padH == P) {                                                                            \
+    if (pl.rw == 7)                                                                                                       \
+      poolRunFwd<K, S, P, MAX, 7><<<grid, dev::kBlock, pl.lds, s>>>(in, out, indices, pl.sg, pl.secondFloats, includePad); \
+    else                                                                                                                  \
+      poolRunFwd<K, S, P, MAX, 4><<<grid, dev::kBlock, pl.lds, s>>>(in, out, indices, pl.sg, pl.secondFloats, includePad); \
+  }
+  POOL_STRIP_COMBOS(X)
+#undef X
+}
+
+template <bool MAX>
+void launchPoolRunBwd(hipStream_t s, const PoolGeom &g, const PoolRunPlan &pl, const float *gradOut, const long *indices,
+                      float *gradIn, bool includePad) {
+  const dim3 grid(poolRunGrid(pl.sg));
+#define X(K, S, P)                            \
+  if (g.kH == K && g.dH == S && g.padH == P) \
+    poolRunBwd<K, S, P, MAX><<<grid, dev::kBlock, pl.lds, s>>>(gradOut, indices, gradIn, pl.sg, includePad);
+  POOL_STRIP_COMBOS(X)
+#undef X
+}
+
 // Output extent rule shared by max and average pooling
 // (lib/THCUNN/generic/SpatialDilatedMaxPooling.cu:47-64,
 //  lib/THCUNN/generic/SpatialAveragePooling.cu:41-58): float division,
@@ -904,8 +1045,11 @@ void maxPoolUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *out
     auto sbytes = [&](int rows) { return fwdStripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
     auto staged = [&](int rows) { return (size_t)((rows - 1) * g.dH + g.kH) * g.W; };
     SmallPool sp;
+    PoolRunPlan rp;
     size_t slds;
-    if (stripFwdOk(g) && vec && aligned16(data(output)) && aligned16(data(indices)) &&
+    const bool haveRuns = aligned16(in.ptr()) && aligned16(data(output)) && aligned16(data(indices)) &&
+                          poolRunPlan(g, planes, false, true, &rp);
+    if (stripFwdOk(g) && !(haveRuns && runsFirst(g, false, true)) && vec && aligned16(data(output)) && aligned16(data(indices)) &&
         launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane, staged)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
       g.magicTiles = dev::magicOf(g.tilesPerPlane);
@@ -916,6 +1060,8 @@ void maxPoolUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *out
     maxPoolFwdStrip<K, S, P><<<grid, block, lds, s>>>(in.ptr(), data(output), data(indices), g);
       POOL_STRIP_COMBOS(X)
 #undef X
+    } else if (haveRuns) {
+      launchPoolRunFwd<true>(s, g, rp, in.ptr(), data(output), data(indices), false);
     } else if (smallPoolPlan(g, planes, false, true, in.ptr(), in.ptr(), &sp, &slds)) {
       poolFwdSmall<true, false><<<launch::ceilDiv(sp.planes, sp.P), dev::kBlock, slds, s>>>(in.ptr(), data(output),
                                                                                            data(indices), g, sp);
@@ -963,8 +1109,11 @@ void maxPoolUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *
   auto sbytes = [&](int units) { return 2 * ((size_t)(units + extra) * spitch + dev::kStripPadL) * sizeof(float); };
   int units = 0;
   SmallPool sp;
+    PoolRunPlan rp;
   size_t slds;
-  if (stripBwdOk(g) && vec && aligned16(data(gradInput)) &&
+  const bool haveRuns = aligned16(go.ptr()) && aligned16(data(gradInput)) && aligned16(data(indices)) &&
+                        poolRunPlan(g, planes, true, true, &rp);
+  if (stripBwdOk(g) && !(haveRuns && runsFirst(g, true, true)) && vec && aligned16(data(gradInput)) &&
       launch::pickBand(launch::ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
     g.tileRows = units * g.dH;
     g.nblk = (int)(planes * g.tilesPerPlane);
@@ -976,6 +1125,8 @@ void maxPoolUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *
     poolBwdStrip<K, S, P, true, true><<<grid, block, lds, s>>>(go.ptr(), data(indices), data(gradInput), g, units + extra);
     POOL_STRIP_COMBOS(X)
 #undef X
+  } else if (haveRuns) {
+    launchPoolRunBwd<true>(s, g, rp, go.ptr(), data(indices), data(gradInput), false);
   } else if (smallPoolPlan(g, planes, true, true, data(gradInput), data(gradInput), &sp, &slds)) {
     poolBwdSmall<true, false><<<launch::ceilDiv(sp.planes, sp.P), dev::kBlock, slds, s>>>(go.ptr(), data(indices),
                                                                                          data(gradInput), g, sp);
@@ -1057,7 +1208,9 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
     auto sbytes = [&](int rows) { return fwdStripFloats(g, (rows - 1) * g.dH + g.kH) * sizeof(float); };
     auto staged = [&](int rows) { return (size_t)((rows - 1) * g.dH + g.kH) * g.W; };
     SmallPool sp;
+    PoolRunPlan rp;
     size_t slds;
+    const bool haveRuns = aligned16(in.ptr()) && aligned16(data(output)) && poolRunPlan(g, planes, false, false, &rp);
     if (avgGlobalOk(g, planes)) {
       const long waves = std::min<long>((planes + 3) / 4, 8192);
       avgPoolGlobalFwd<<<(unsigned)((waves + 3) / 4), dev::kBlock, 0, s>>>(in.ptr(), data(output), planes, g.H * g.W);
@@ -1068,7 +1221,7 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
       if (g.kH == 2) avgPoolFwdFlat<2><<<grid, dev::kBlock, 0, s>>>(in.ptr(), data(output), g.oW / 4, magic, g.W, total);
       if (g.kH == 3) avgPoolFwdFlat<3><<<grid, dev::kBlock, 0, s>>>(in.ptr(), data(output), g.oW / 4, magic, g.W, total);
       if (g.kH == 4) avgPoolFwdFlat<4><<<grid, dev::kBlock, 0, s>>>(in.ptr(), data(output), g.oW / 4, magic, g.W, total);
-    } else if (stripFwdOk(g) && vec && aligned16(data(output)) &&
+    } else if (stripFwdOk(g) && !(haveRuns && runsFirst(g, false, false)) && vec && aligned16(data(output)) &&
         launch::pickBand(g.oH, planes, sbytes, &g.tileRows, &g.tilesPerPlane, staged)) {
       g.nblk = (int)(planes * g.tilesPerPlane);
       g.magicTiles = dev::magicOf(g.tilesPerPlane);
@@ -1083,6 +1236,8 @@ void THNN_CudaSpatialAveragePooling_updateOutput(THCState *state, THCudaTensor *
   }
       POOL_STRIP_COMBOS(X)
 #undef X
+    } else if (haveRuns) {
+      launchPoolRunFwd<false>(s, g, rp, in.ptr(), data(output), nullptr, count_include_pad);
     } else if (smallPoolPlan(g, planes, false, false, in.ptr(), in.ptr(), &sp, &slds)) {
       const unsigned grid = launch::ceilDiv(sp.planes, sp.P);
       if (count_include_pad)
@@ -1145,7 +1300,9 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
   auto sbytes = [&](int units) { return ((size_t)(units + extra) * spitch + dev::kStripPadL) * sizeof(float); };
   int units = 0;
   SmallPool sp;
+    PoolRunPlan rp;
   size_t slds;
+  const bool haveRuns = aligned16(go.ptr()) && aligned16(data(gradInput)) && poolRunPlan(g, planes, true, false, &rp);
   if (avgGlobalOk(g, planes)) {
     const unsigned total = (unsigned)(planes * g.H * g.W);
     avgPoolGlobalBwd<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), total,
@@ -1157,7 +1314,7 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
     if (g.kH == 2) avgPoolBwdFlat<2><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.W / 4, magic, g.oW, total);
     if (g.kH == 3) avgPoolBwdFlat<3><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.W / 4, magic, g.oW, total);
     if (g.kH == 4) avgPoolBwdFlat<4><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.W / 4, magic, g.oW, total);
-  } else if (stripBwdOk(g) && vec && aligned16(data(gradInput)) &&
+  } else if (stripBwdOk(g) && !(haveRuns && runsFirst(g, true, false)) && vec && aligned16(data(gradInput)) &&
       launch::pickBand(launch::ceilDiv(g.H, g.dH), planes, sbytes, &units, &g.tilesPerPlane)) {
     g.tileRows = units * g.dH;
     g.nblk = (int)(planes * g.tilesPerPlane);
@@ -1173,6 +1330,8 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
   }
     POOL_STRIP_COMBOS(X)
 #undef X
+  } else if (haveRuns) {
+    launchPoolRunBwd<false>(s, g, rp, go.ptr(), nullptr, data(gradInput), count_include_pad);
   } else if (smallPoolPlan(g, planes, true, false, data(gradInput), data(gradInput), &sp, &slds)) {
     const unsigned grid = launch::ceilDiv(sp.planes, sp.P);
     if (count_include_pad)

@@ -9,8 +9,8 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 from oracle import oracle as O  # noqa: E402
-from test_gpu_parity import (T, close, _dw_run, _dw_inputs, _maxpool_run, _avgpool_run, _tied_input,  # noqa: E402,F401
-                             _bn_run)
+from test_gpu_parity import (T, close, force_direct, _dw_run, _dw_inputs, _maxpool_run, _avgpool_run,  # noqa: E402,F401
+                             _tied_input, _bn_run)
 
 
 @pytest.mark.parametrize("seed", range(30))
@@ -76,6 +76,57 @@ def test_pool_small_random(T, seed):
     case = (N, C, H, W, kW, kH, dW, dH, pW, pH, ceil)
     _maxpool_run(T, case, _tied_input(case[:4], 4100 + seed, q=8))
     _avgpool_run(T, case, bool(seed % 2), seed=4200 + seed)
+
+
+# window geometries of the pooling kernels that work on runs of memory: (k, stride, pad)
+POOL_RUN_COMBOS = [(3, 2, 1), (2, 2, 0), (3, 2, 0), (3, 1, 1)]
+# network planes of odd width, planes on either side of the several-planes limit, single-row bands
+POOL_RUN_PLANES = [(2, 3, 147, 147), (1, 5, 71, 71), (3, 7, 35, 35), (2, 70, 17, 17), (2, 9, 27, 27), (1, 66, 8, 8),
+                   (2, 5, 28, 28), (1, 3, 45, 46), (1, 2, 3, 2045), (1, 2, 300, 3), (1, 3, 1, 1025), (2, 2, 55, 55)]
+
+
+@pytest.mark.parametrize("combo", POOL_RUN_COMBOS, ids=lambda c: "k%ds%dp%d" % c)
+@pytest.mark.parametrize("plane", POOL_RUN_PLANES, ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("ceil", [False, True])
+def test_pool_runs(T, combo, plane, ceil):
+    k, s, p = combo
+    N, C, H, W = plane
+    if H + 2 * p < k or W + 2 * p < k:
+        pytest.skip("window larger than the padded plane")
+    case = (N, C, H, W, k, k, s, s, p, p, ceil)
+    _maxpool_run(T, case, _tied_input(case[:4], 4500, q=8))
+    _avgpool_run(T, case, True, seed=4501)
+    _avgpool_run(T, case, False, seed=4502)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_pool_runs_random(T, seed):
+    rng = np.random.default_rng(4600 + seed)
+    k, s, p = POOL_RUN_COMBOS[seed % 4]
+    H, W = (int(v) for v in rng.integers(max(1, k - 2 * p), 200, 2))
+    N, C = int(rng.integers(1, 4)), int(rng.integers(1, 40))
+    case = (N, C, H, W, k, k, s, s, p, p, bool(rng.integers(0, 2)))
+    _maxpool_run(T, case, _tied_input(case[:4], 4700 + seed, q=8))
+    _avgpool_run(T, case, bool(seed % 2), seed=4800 + seed)
+
+
+# widths that are multiples of 4: the strip kernels and the run kernels both apply, the library picks by size
+POOL_BOTH_PLANES = [(2, 9, 27, 27), (1, 5, 71, 71), (2, 70, 17, 17), (2, 6, 56, 56), (1, 4, 112, 112), (2, 8, 16, 16),
+                    (1, 3, 32, 64), (1, 2, 8, 8)]
+
+
+@pytest.mark.parametrize("combo", POOL_RUN_COMBOS, ids=lambda c: "k%ds%dp%d" % c)
+@pytest.mark.parametrize("switch", ["0", "1"])
+def test_pool_runs_switch(T, combo, switch):
+    """THCUNN_POOL_RUNS=0: never the run kernels (strip kernels, small-plane kernels, tiled kernels as before);
+    1: the run kernels wherever their window geometry matches."""
+    k, s, p = combo
+    with force_direct("THCUNN_POOL_RUNS", switch):
+        for plane in POOL_BOTH_PLANES:
+            for ceil in (False, True):
+                case = plane + (k, k, s, s, p, p, ceil)
+                _maxpool_run(T, case, _tied_input(case[:4], 4900, q=8))
+                _avgpool_run(T, case, not ceil, seed=4901)
 
 
 @pytest.mark.parametrize("seed", range(16))

@@ -18,6 +18,8 @@
 
 #include <atomic>
 
+#include <type_traits>
+
 #include "device_utils.h"
 #include "launch_utils.h"
 #include "thc_internal.h"
@@ -49,23 +51,43 @@ __device__ __forceinline__ Chunk chunkOf(const BnGeom &g, int chunk) {
   return c;
 }
 
-// Visits every element of a chunk of channel `ch`: f(offset, width) is called
-// with the flat offset into the (N,C,L) tensor of `width` (4 or 1) consecutive
-// elements.
-template <bool VEC, typename F>
+// Visits every element of a chunk of channel `ch`: f(offset, width) is called with the flat offset into the
+// (N,C,L) tensor of `width` (W4 or W1) consecutive elements. MODE 1: plane segments start on 16-byte
+// boundaries and are multiples of 4 long (16-byte accesses only); MODE 2: any plane size in a 16-byte aligned
+// tensor - per plane segment the elements in front of the first boundary, the 16-byte groups, and the
+// elements behind the last boundary are three kinds of work items; MODE 0: element by element.
+using W1 = std::integral_constant<int, 1>;
+using W4 = std::integral_constant<int, 4>;
+template <int MODE, typename F>
 __device__ __forceinline__ void forChunk(const BnGeom &g, int ch, const Chunk &c, F f) {
-  if (VEC) {
+  if (MODE == 1) {
     const int seg4 = c.lN >> 2;
     const int total = c.nN * seg4;
     for (int i = threadIdx.x; i < total; i += blockDim.x) {
       int n = i / seg4, l4 = i - n * seg4;
-      f(((long)(c.n0 + n) * g.C + ch) * g.L + c.l0 + (l4 << 2));
+      f(((long)(c.n0 + n) * g.C + ch) * g.L + c.l0 + (l4 << 2), W4{});
+    }
+  } else if (MODE == 2) {
+    const int slots = (c.lN >> 2) + 2;  // head, at most lN / 4 groups, tail
+    const int total = c.nN * slots;
+    for (int i = threadIdx.x; i < total; i += blockDim.x) {
+      const int n = i / slots, k = i - n * slots;
+      const long off0 = ((long)(c.n0 + n) * g.C + ch) * g.L + c.l0;
+      const int head = min((int)(-off0 & 3), c.lN);
+      const int body4 = (c.lN - head) >> 2, tail = (c.lN - head) & 3;
+      if (k == 0) {
+        for (int j = 0; j < head; ++j) f(off0 + j, W1{});
+      } else if (k <= body4) {
+        f(off0 + head + ((k - 1) << 2), W4{});
+      } else if (k == body4 + 1) {
+        for (int j = 0; j < tail; ++j) f(off0 + head + (body4 << 2) + j, W1{});
+      }
     }
   } else {
     const int total = c.nN * c.lN;
     for (int i = threadIdx.x; i < total; i += blockDim.x) {
       int n = i / c.lN, l = i - n * c.lN;
-      f(((long)(c.n0 + n) * g.C + ch) * g.L + c.l0 + l);
+      f(((long)(c.n0 + n) * g.C + ch) * g.L + c.l0 + l, W1{});
     }
   }
 }
@@ -90,7 +112,7 @@ __device__ __forceinline__ void blockSum(float (&v)[NV], float (*red)[NV]) {
 
 // ------------------------------------------------------ forward statistics ----
 // partial[(ch * chunks + chunk) * 3 + {0,1,2}] = count, mean, M2 of the chunk
-template <bool VEC>
+template <int VEC>
 __global__ void __launch_bounds__(dev::kBlock)
 bnStatsKernel(const float *__restrict__ x, float *__restrict__ partial, BnGeom g) {
   __shared__ float red[dev::kBlock / dev::kWave][2];
@@ -100,8 +122,8 @@ bnStatsKernel(const float *__restrict__ x, float *__restrict__ partial, BnGeom g
   // not cancel when |mean| >> sigma
   const float shift = x[((long)c.n0 * g.C + ch) * g.L + c.l0];
   float v[2] = {0.f, 0.f};
-  forChunk<VEC>(g, ch, c, [&](long off) {
-    if (VEC) {
+  forChunk<VEC>(g, ch, c, [&](long off, auto width) {
+    if constexpr (decltype(width)::value == 4) {
       float4 q = *reinterpret_cast<const float4 *>(x + off);
       float d0 = q.x - shift, d1 = q.y - shift, d2 = q.z - shift, d3 = q.w - shift;
       v[0] += (d0 + d1) + (d2 + d3);
@@ -153,7 +175,7 @@ __device__ __forceinline__ void mergeStats(const float *__restrict__ p, int chun
 // ------------------------------------------------------------ forward apply ----
 // TRAIN: merges the chunk statistics, publishes saveMean/saveStd/running stats
 // (chunk 0 only) and normalises; otherwise uses the running statistics.
-template <bool TRAIN, bool VEC>
+template <bool TRAIN, int VEC>
 __global__ void __launch_bounds__(dev::kBlock)
 bnApplyKernel(const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ partial,
               const float *__restrict__ weight, const float *__restrict__ bias, float *__restrict__ runningMean,
@@ -191,8 +213,8 @@ bnApplyKernel(const float *__restrict__ x, float *__restrict__ y, const float *_
   }
   const float gamma = weight ? weight[ch] : 1.f, beta = bias ? bias[ch] : 0.f;
   const Chunk c = chunkOf(g, chunk);
-  forChunk<VEC>(g, ch, c, [&](long off) {
-    if (VEC) {
+  forChunk<VEC>(g, ch, c, [&](long off, auto width) {
+    if constexpr (decltype(width)::value == 4) {
       float4 q = *reinterpret_cast<const float4 *>(x + off), r;
       r.x = gamma * (q.x - mean) * invStd + beta;
       r.y = gamma * (q.y - mean) * invStd + beta;
@@ -207,7 +229,7 @@ bnApplyKernel(const float *__restrict__ x, float *__restrict__ y, const float *_
 
 // ----------------------------------------------------------- backward sums ----
 // partial[(ch * chunks + chunk) * 2 + {0,1}] = sum gy, sum gy * (x - mean)
-template <bool VEC>
+template <int VEC>
 __global__ void __launch_bounds__(dev::kBlock)
 bnGradSumsKernel(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ partial,
                  const float *__restrict__ meanSrc, BnGeom g) {
@@ -216,8 +238,8 @@ bnGradSumsKernel(const float *__restrict__ x, const float *__restrict__ gy, floa
   const Chunk c = chunkOf(g, chunk);
   const float mean = meanSrc[ch];
   float v[2] = {0.f, 0.f};
-  forChunk<VEC>(g, ch, c, [&](long off) {
-    if (VEC) {
+  forChunk<VEC>(g, ch, c, [&](long off, auto width) {
+    if constexpr (decltype(width)::value == 4) {
       float4 q = *reinterpret_cast<const float4 *>(x + off);
       float4 d = *reinterpret_cast<const float4 *>(gy + off);
       v[0] += (d.x + d.y) + (d.z + d.w);
@@ -253,7 +275,7 @@ __device__ __forceinline__ void mergeSums(const float *__restrict__ p, int chunk
 // ---------------------------------------------------------- backward apply ----
 // lib/THCUNN/BatchNormalization.cu:253-282. HAVE_SUMS: partial holds the chunk
 // sums (needed for train-mode gradInput and for gradWeight/gradBias).
-template <bool TRAIN, bool VEC>
+template <bool TRAIN, int VEC>
 __global__ void __launch_bounds__(dev::kBlock)
 bnBackwardKernel(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
                  const float *__restrict__ partial, float *__restrict__ gradWeight, float *__restrict__ gradBias,
@@ -284,8 +306,8 @@ bnBackwardKernel(const float *__restrict__ x, const float *__restrict__ gy, floa
   const float gradScale = stdVal * weightVal;
   if (gx) {
     const Chunk c = chunkOf(g, chunk);
-    forChunk<VEC>(g, ch, c, [&](long off) {
-      if (VEC) {
+    forChunk<VEC>(g, ch, c, [&](long off, auto width) {
+      if constexpr (decltype(width)::value == 4) {
         float4 d = *reinterpret_cast<const float4 *>(gy + off), r;
         if (TRAIN) {
           float4 q = *reinterpret_cast<const float4 *>(x + off);
@@ -568,40 +590,44 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
 // workgroup per channel keeps them in registers, RS scalar elements per lane (element e = tid + 256 u is
 // image e / L, position e % L: the lanes of a wave read runs of L consecutive floats); the formulas
 // are those of the 1024-lane kernels.
-constexpr int kSmallBlock = 256;
+constexpr int kSmallBlock = 256;  // channels of up to 32 * 256 elements; up to 32 * 1024 take 1024 lanes
 
-__device__ __forceinline__ float blockSum256(float v, float *red) {
+template <int BS>
+__device__ __forceinline__ float blockSumSmall(float v, float *red) {
   const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
   v = dev::waveSum(v);
   __syncthreads();  // red may still be read from a previous reduction
   if (lane == 0) red[wave] = v;
   __syncthreads();
-  return (red[0] + red[1]) + (red[2] + red[3]);
+  float s = 0.f;
+#pragma unroll
+  for (int w = 0; w < BS / dev::kWave; w += 4) s += (red[w] + red[w + 1]) + (red[w + 2] + red[w + 3]);
+  return s;
 }
 
 // element offsets (in floats, from the channel's first plane) of this lane; -1 past the channel
-template <int RS>
+template <int RS, int BS>
 __device__ __forceinline__ void smallOffsets(int (&off)[RS], int N, int C, int L, unsigned magicL) {
 #pragma unroll
   for (int u = 0; u < RS; ++u) {
-    const int e = u * kSmallBlock + (int)threadIdx.x;
+    const int e = u * BS + (int)threadIdx.x;
     const int n = dev::fastDiv(e, magicL);
     off[u] = e < N * L ? n * C * L + (e - n * L) : -1;
   }
 }
 
-template <int RS>
-__global__ void __launch_bounds__(kSmallBlock)
+template <int RS, int BS>
+__global__ void __launch_bounds__(BS)
 bnFwdSmall(const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ weight,
            const float *__restrict__ bias, float *__restrict__ runningMean, float *__restrict__ runningVar,
            float *__restrict__ saveMean, float *__restrict__ saveStd, int N, int C, int L, unsigned magicL,
            float momentum, float eps) {
-  __shared__ float red[kSmallBlock / dev::kWave];
+  __shared__ float red[BS / dev::kWave];
   const int ch = blockIdx.x;
   const float *xc = x + (long)ch * L;
   float *yc = y + (long)ch * L;
   int off[RS];
-  smallOffsets<RS>(off, N, C, L, magicL);
+  smallOffsets<RS, BS>(off, N, C, L, magicL);
   float v[RS];
 #pragma unroll
   for (int u = 0; u < RS; ++u) v[u] = off[u] >= 0 ? xc[off[u]] : 0.f;
@@ -609,12 +635,12 @@ bnFwdSmall(const float *__restrict__ x, float *__restrict__ y, const float *__re
   float s = 0.f;
 #pragma unroll
   for (int u = 0; u < RS; ++u) s += v[u];
-  const float mean = blockSum256(s, red) * norm;
+  const float mean = blockSumSmall<BS>(s, red) * norm;
   float q = 0.f;
 #pragma unroll
   for (int u = 0; u < RS; ++u)
     if (off[u] >= 0) q += (v[u] - mean) * (v[u] - mean);
-  const float varN = blockSum256(q, red);
+  const float varN = blockSumSmall<BS>(q, red);
   float invStd = 0.f;
   if (varN != 0.f || eps != 0.f) invStd = 1.f / sqrtf(varN * norm + eps);
   if (threadIdx.x == 0) {
@@ -630,20 +656,20 @@ bnFwdSmall(const float *__restrict__ x, float *__restrict__ y, const float *__re
     if (off[u] >= 0) yc[off[u]] = gamma * (v[u] - mean) * invStd + beta;
 }
 
-template <int RS, bool TRAIN>
-__global__ void __launch_bounds__(kSmallBlock)
+template <int RS, bool TRAIN, int BS>
+__global__ void __launch_bounds__(BS)
 bnBwdSmall(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
            float *__restrict__ gradWeight, float *__restrict__ gradBias, const float *__restrict__ weight,
            const float *__restrict__ meanSrc, const float *__restrict__ stdSrc, int N, int C, int L, unsigned magicL,
            float scale, float eps) {
-  __shared__ float red[kSmallBlock / dev::kWave];
+  __shared__ float red[BS / dev::kWave];
   const int ch = blockIdx.x;
   const float *xc = x + (long)ch * L, *gc = gy + (long)ch * L;
   const float mean = meanSrc[ch];
   const float stdVal = TRAIN ? stdSrc[ch] : 1.f / sqrtf(stdSrc[ch] + eps);
   const float weightVal = weight ? weight[ch] : 1.f;
   int off[RS];
-  smallOffsets<RS>(off, N, C, L, magicL);
+  smallOffsets<RS, BS>(off, N, C, L, magicL);
   float d[RS], xm[RS];
 #pragma unroll
   for (int u = 0; u < RS; ++u) {
@@ -657,8 +683,8 @@ bnBwdSmall(const float *__restrict__ x, const float *__restrict__ gy, float *__r
     s0 += d[u];
     s1 += d[u] * xm[u];
   }
-  const float gradOutputSum = blockSum256(s0, red);
-  const float dotP = blockSum256(s1, red);
+  const float gradOutputSum = blockSumSmall<BS>(s0, red);
+  const float dotP = blockSumSmall<BS>(s1, red);
   const float norm = 1.f / ((float)N * (float)L);
   const float gradMean = gradOutputSum * norm;
   const float projScale = dotP * norm * stdVal * stdVal;
@@ -678,7 +704,8 @@ bnBwdSmall(const float *__restrict__ x, const float *__restrict__ gy, float *__r
 // -------------------------------------------------------------- host side ----
 struct BnView {
   BnGeom g;
-  bool vec;
+  bool vec;  // plane size a multiple of 4 and every tensor 16-byte aligned
+  int mode;  // forChunk: 1 = vec, 2 = 16-byte accesses around unaligned plane starts, 0 = element by element
 };
 
 // N x C x L view of the input (lib/THCUNN/generic/BatchNormalization.cu:8-32)
@@ -695,7 +722,10 @@ BnView bnView(const THCudaTensor *t, std::initializer_list<const void *> ptrs) {
     error("BatchNormalization: dimensions of 2^31 or more elements are not supported");
   g.N = (int)e->size[0], g.C = (int)e->size[1], g.L = (int)L;
   v.vec = g.L % 4 == 0;
-  for (const void *p : ptrs) v.vec = v.vec && (p == nullptr || launch::aligned16(p));
+  bool aligned = true;
+  for (const void *p : ptrs) aligned = aligned && (p == nullptr || launch::aligned16(p));
+  v.vec = v.vec && aligned;
+  v.mode = v.vec ? 1 : (aligned && g.L >= 8 ? 2 : 0);
   // ~8K elements (32 KB) per workgroup: 8 x 16-byte loads per lane
   const int target = 8192;
   if (g.L >= target) {
@@ -750,19 +780,24 @@ int residentR(const BnView &v, int maxR) {
   return 0;
 }
 
-// Elements per lane of the small-channel kernels (0: not applicable): planes whose size is not a multiple of 4
-// (the 16-byte kernels take the others), channels of at most 32 * 256 elements, enough channels to occupy the chip.
-int smallR(const BnView &v) {
+// Elements per lane and lanes per workgroup of the small-channel kernels (rs 0: not applicable): planes whose
+// size is not a multiple of 4 (the 16-byte kernels take the others), channels of at most 32 * 1024 elements,
+// enough channels to occupy the chip.
+struct SmallChoice {
+  int rs, bs;
+};
+SmallChoice smallR(const BnView &v) {
   const char *e = getenv("THCUNN_BN_FORCE_CHUNKED");
-  if (e && e[0] == '1') return 0;
+  if (e && e[0] == '1') return {0, 0};
   const BnGeom &g = v.g;
   const long NL = (long)g.N * g.L;
-  if (g.L % 4 == 0 || g.C < 96 || NL > 32 * kSmallBlock || (long)g.N * g.C * g.L >= 0x7fffffffL) return 0;
-  const int need = (int)((NL + kSmallBlock - 1) / kSmallBlock);
+  if (g.L % 4 == 0 || g.C < 96 || NL > 32 * kResBlock || (long)g.N * g.C * g.L >= 0x7fffffffL) return {0, 0};
+  const int bs = NL <= 32 * kSmallBlock ? kSmallBlock : kResBlock;
+  const int need = (int)((NL + bs - 1) / bs);
   const int sizes[] = {4, 8, 16, 32};
   for (int r : sizes)
-    if (need <= r) return r;
-  return 0;
+    if (need <= r) return {r, bs};
+  return {0, 0};
 }
 
 }  // namespace
@@ -805,14 +840,14 @@ void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *inp
     THC_HIP_CHECK(hipGetLastError());
     return;
   }
-  if (int RS = train ? smallR(v) : 0) {
-#define BN_FWD_SMALL(RR)                                                                                            \
-  if (RS == RR)                                                                                                     \
-    bnFwdSmall<RR><<<g.C, kSmallBlock, 0, s>>>(in.ptr(), data(output_), dataOrNull(weight_), dataOrNull(bias_),     \
-                                               data(runningMean_), data(runningVar_), data(saveMean_),              \
-                                               data(saveStd_), g.N, g.C, g.L, dev::magicOf(g.L), (float)momentum,   \
-                                               (float)eps);
-    BN_FWD_SMALL(4) BN_FWD_SMALL(8) BN_FWD_SMALL(16) BN_FWD_SMALL(32)
+  if (const SmallChoice sc = train ? smallR(v) : SmallChoice{0, 0}; sc.rs) {
+#define BN_FWD_SMALL(RR, BS)                                                                                        \
+  if (sc.rs == RR && sc.bs == BS)                                                                                   \
+    bnFwdSmall<RR, BS><<<g.C, BS, 0, s>>>(in.ptr(), data(output_), dataOrNull(weight_), dataOrNull(bias_),          \
+                                          data(runningMean_), data(runningVar_), data(saveMean_), data(saveStd_),   \
+                                          g.N, g.C, g.L, dev::magicOf(g.L), (float)momentum, (float)eps);
+    BN_FWD_SMALL(4, kSmallBlock) BN_FWD_SMALL(8, kSmallBlock) BN_FWD_SMALL(16, kSmallBlock) BN_FWD_SMALL(32, kSmallBlock)
+    BN_FWD_SMALL(16, kResBlock) BN_FWD_SMALL(32, kResBlock)
 #undef BN_FWD_SMALL
     THC_HIP_CHECK(hipGetLastError());
     return;
@@ -820,28 +855,23 @@ void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *inp
   if (train) {
     Temp partial(s, (size_t)g.C * g.chunks * 3 * sizeof(float));
     float *p = (float *)partial.get();
-    if (v.vec) {
-      bnStatsKernel<true><<<grid, block, 0, s>>>(in.ptr(), p, g);
-      bnApplyKernel<true, true><<<grid, block, 0, s>>>(in.ptr(), data(output_), p, dataOrNull(weight_),
-                                                       dataOrNull(bias_), data(runningMean_), data(runningVar_),
-                                                       data(saveMean_), data(saveStd_), g, (float)momentum,
-                                                       (float)eps);
-    } else {
-      bnStatsKernel<false><<<grid, block, 0, s>>>(in.ptr(), p, g);
-      bnApplyKernel<true, false><<<grid, block, 0, s>>>(in.ptr(), data(output_), p, dataOrNull(weight_),
-                                                        dataOrNull(bias_), data(runningMean_), data(runningVar_),
-                                                        data(saveMean_), data(saveStd_), g, (float)momentum,
-                                                        (float)eps);
-    }
+#define BN_FWD_TRAIN(MODE)                                                                                        \
+  {                                                                                                               \
+    bnStatsKernel<MODE><<<grid, block, 0, s>>>(in.ptr(), p, g);                                                   \
+    bnApplyKernel<true, MODE><<<grid, block, 0, s>>>(in.ptr(), data(output_), p, dataOrNull(weight_),             \
+                                                     dataOrNull(bias_), data(runningMean_), data(runningVar_),    \
+                                                     data(saveMean_), data(saveStd_), g, (float)momentum,         \
+                                                     (float)eps);                                                 \
+  }
+    if (v.mode == 1) BN_FWD_TRAIN(1) else if (v.mode == 2) BN_FWD_TRAIN(2) else BN_FWD_TRAIN(0)
+#undef BN_FWD_TRAIN
   } else {
-    if (v.vec)
-      bnApplyKernel<false, true><<<grid, block, 0, s>>>(in.ptr(), data(output_), nullptr, dataOrNull(weight_),
-                                                        dataOrNull(bias_), data(runningMean_), data(runningVar_),
-                                                        nullptr, nullptr, g, (float)momentum, (float)eps);
-    else
-      bnApplyKernel<false, false><<<grid, block, 0, s>>>(in.ptr(), data(output_), nullptr, dataOrNull(weight_),
-                                                         dataOrNull(bias_), data(runningMean_), data(runningVar_),
-                                                         nullptr, nullptr, g, (float)momentum, (float)eps);
+#define BN_FWD_EVAL(MODE)                                                                                         \
+  bnApplyKernel<false, MODE><<<grid, block, 0, s>>>(in.ptr(), data(output_), nullptr, dataOrNull(weight_),        \
+                                                    dataOrNull(bias_), data(runningMean_), data(runningVar_),     \
+                                                    nullptr, nullptr, g, (float)momentum, (float)eps);
+    if (v.mode == 1) BN_FWD_EVAL(1) else if (v.mode == 2) BN_FWD_EVAL(2) else BN_FWD_EVAL(0)
+#undef BN_FWD_EVAL
   }
   THC_HIP_CHECK(hipGetLastError());
   THNN_LEAVE
@@ -919,20 +949,21 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
     THC_HIP_CHECK(hipGetLastError());
     return;
   }
-  if (int RS = needSums ? smallR(v) : 0) {
+  if (const SmallChoice sc = needSums ? smallR(v) : SmallChoice{0, 0}; sc.rs) {
     float *gxp = gradInput_ ? data(gradInput_) : nullptr;
-#define BN_BWD_SMALL(RR)                                                                                          \
-  if (RS == RR) {                                                                                                 \
+#define BN_BWD_SMALL(RR, BS)                                                                                      \
+  if (sc.rs == RR && sc.bs == BS) {                                                                               \
     if (train)                                                                                                    \
-      bnBwdSmall<RR, true><<<g.C, kSmallBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),          \
-                                                       dataOrNull(gradBias_), dataOrNull(weight_), meanSrc, stdSrc, \
-                                                       g.N, g.C, g.L, dev::magicOf(g.L), (float)scale, (float)eps); \
+      bnBwdSmall<RR, true, BS><<<g.C, BS, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),               \
+                                                  dataOrNull(gradBias_), dataOrNull(weight_), meanSrc, stdSrc,    \
+                                                  g.N, g.C, g.L, dev::magicOf(g.L), (float)scale, (float)eps);    \
     else                                                                                                          \
-      bnBwdSmall<RR, false><<<g.C, kSmallBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),         \
-                                                        dataOrNull(gradBias_), dataOrNull(weight_), meanSrc, stdSrc, \
-                                                        g.N, g.C, g.L, dev::magicOf(g.L), (float)scale, (float)eps); \
+      bnBwdSmall<RR, false, BS><<<g.C, BS, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),              \
+                                                   dataOrNull(gradBias_), dataOrNull(weight_), meanSrc, stdSrc,   \
+                                                   g.N, g.C, g.L, dev::magicOf(g.L), (float)scale, (float)eps);   \
   }
-    BN_BWD_SMALL(4) BN_BWD_SMALL(8) BN_BWD_SMALL(16) BN_BWD_SMALL(32)
+    BN_BWD_SMALL(4, kSmallBlock) BN_BWD_SMALL(8, kSmallBlock) BN_BWD_SMALL(16, kSmallBlock) BN_BWD_SMALL(32, kSmallBlock)
+    BN_BWD_SMALL(16, kResBlock) BN_BWD_SMALL(32, kResBlock)
 #undef BN_BWD_SMALL
     THC_HIP_CHECK(hipGetLastError());
     return;
@@ -942,10 +973,12 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
   if (needSums) {
     partial = Temp(s, (size_t)g.C * g.chunks * 2 * sizeof(float));
     p = (float *)partial.get();
-    if (v.vec)
-      bnGradSumsKernel<true><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g);
+    if (v.mode == 1)
+      bnGradSumsKernel<1><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g);
+    else if (v.mode == 2)
+      bnGradSumsKernel<2><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g);
     else
-      bnGradSumsKernel<false><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g);
+      bnGradSumsKernel<0><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g);
     THC_HIP_CHECK(hipGetLastError());
   }
   BnGeom ga = g;
@@ -957,15 +990,19 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
   bnBackwardKernel<TRAIN, VEC><<<gridApply, block, 0, s>>>(in.ptr(), go.ptr(), gx, p, gw, gb, w, meanSrc, stdSrc, ga, \
                                                            (float)scale, (float)eps)
   if (train) {
-    if (v.vec)
-      BN_BWD(true, true);
+    if (v.mode == 1)
+      BN_BWD(true, 1);
+    else if (v.mode == 2)
+      BN_BWD(true, 2);
     else
-      BN_BWD(true, false);
+      BN_BWD(true, 0);
   } else {
-    if (v.vec)
-      BN_BWD(false, true);
+    if (v.mode == 1)
+      BN_BWD(false, 1);
+    else if (v.mode == 2)
+      BN_BWD(false, 2);
     else
-      BN_BWD(false, false);
+      BN_BWD(false, 0);
   }
 #undef BN_BWD
   THC_HIP_CHECK(hipGetLastError());

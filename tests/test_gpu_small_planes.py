@@ -135,3 +135,21 @@ def test_batchnorm_small_random(T, seed):
     H, W = (int(v) for v in rng.integers(1, 12, 2))
     N, C = int(rng.integers(1, 80)), int(rng.integers(96, 140))
     _bn_run(T, (N, C, H, W), bool(seed % 2), seed=5100 + seed)
+
+
+# plane sizes that are not multiples of 4 beyond the 256-lane resident kernels: 1024-lane resident kernels
+# (channels of up to 32768 elements, >= 96 channels) and the chunked kernels with 16-byte accesses around
+# unaligned plane starts (whole planes per chunk, and planes cut into segments)
+BN_ODD_SHAPES = [(32, 100, 17, 17), (64, 96, 13, 13), (30, 97, 27, 27), (32, 96, 31, 31), (17, 101, 35, 35),
+                 (4, 8, 35, 35), (3, 5, 147, 147), (2, 3, 99, 101), (5, 7, 3, 3), (6, 4, 1, 9), (2, 130, 75, 75)]
+
+
+@pytest.mark.parametrize("shape", BN_ODD_SHAPES, ids=lambda c: "x".join(map(str, c)))
+def test_batchnorm_odd_planes(T, shape):
+    _bn_run(T, shape, True, seed=5200)
+
+
+@pytest.mark.parametrize("shape", BN_ODD_SHAPES[:4] + BN_ODD_SHAPES[6:7], ids=lambda c: "x".join(map(str, c)))
+def test_batchnorm_odd_planes_chunked(T, shape):
+    with force_direct("THCUNN_BN_FORCE_CHUNKED", "1"):
+        _bn_run(T, shape, False, seed=5201)

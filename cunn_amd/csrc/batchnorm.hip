@@ -182,7 +182,10 @@ bnApplyKernel(const float *__restrict__ x, float *__restrict__ y, const float *_
               float *__restrict__ runningVar, float *__restrict__ saveMean, float *__restrict__ saveStd, BnGeom g,
               float momentum, float eps) {
   __shared__ float bc[2];
-  const int ch = blockIdx.x / g.chunks, chunk = blockIdx.x - ch * g.chunks;
+  // the statistics pass went through the tensor front to back: going back to front meets what it read last
+  // while that is still in the last-level cache
+  const int bid = gridDim.x - 1 - blockIdx.x;
+  const int ch = bid / g.chunks, chunk = bid - ch * g.chunks;
   float mean, invStd;
   if (TRAIN) {
     if (threadIdx.x < dev::kWave) {
@@ -282,7 +285,8 @@ bnBackwardKernel(const float *__restrict__ x, const float *__restrict__ gy, floa
                  const float *__restrict__ weight, const float *__restrict__ meanSrc,
                  const float *__restrict__ stdSrc, BnGeom g, float scale, float eps) {
   __shared__ float bc[2];
-  const int ch = blockIdx.x / g.chunks, chunk = blockIdx.x - ch * g.chunks;
+  const int bid = gridDim.x - 1 - blockIdx.x;  // back to front, see bnApplyKernel
+  const int ch = bid / g.chunks, chunk = bid - ch * g.chunks;
   const float mean = meanSrc[ch];
   const float stdVal = TRAIN ? stdSrc[ch] : 1.f / sqrtf(stdSrc[ch] + eps);
   const float weightVal = weight ? weight[ch] : 1.f;

@@ -153,3 +153,45 @@ def test_batchnorm_odd_planes(T, shape):
 def test_batchnorm_odd_planes_chunked(T, shape):
     with force_direct("THCUNN_BN_FORCE_CHUNKED", "1"):
         _bn_run(T, shape, False, seed=5201)
+
+
+def _at_offset(T, a, off):
+    """A contiguous tensor whose first element sits `off` floats behind a 16-byte boundary of its storage."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    big = T.CudaTensor.with_size(a.size + 8)
+    big.fill(float("nan"))
+    strides = [1] * a.ndim
+    for d in range(a.ndim - 2, -1, -1):
+        strides[d] = strides[d + 1] * a.shape[d + 1]
+    v = big.view(off, a.shape, strides)
+    v.copy_(a)
+    return v
+
+
+@pytest.mark.parametrize("off", [1, 2, 3])
+def test_run_kernels_decline_unaligned_tensors(T, off):
+    """The run-of-memory kernels fetch from the 16-byte boundary below a run and so need 16-byte aligned
+    tensors; an input that starts elsewhere in its storage takes the other kernels, with the same results."""
+    THNN, CT, LT = T.THNN, T.CudaTensor, T.CudaLongTensor
+    rng = np.random.default_rng(6000 + off)
+    # depthwise convolution, small planes
+    case = (2, 9, 1, 14, 14, 3, 3, 1, 1, 1, 1)
+    _, x, w, b = _dw_inputs(case, 6100 + off)
+    _dw_run(T, case, x, w, b, xt=_at_offset(T, x, off))
+    # pooling, odd width
+    x = _tied_input((2, 5, 27, 27), 6200 + off, q=8)
+    _maxpool_run(T, (2, 5, 27, 27, 3, 3, 2, 2, 0, 0, False), x, xt=_at_offset(T, x, off))
+    tx, out = _at_offset(T, x, off), CT()
+    THNN.SpatialAveragePooling_updateOutput(tx, out, 3, 3, 2, 2, 0, 0, False, True)
+    close(out.numpy(), O.avgpool_updateOutput(x, 3, 3, 2, 2, 0, 0, False, True))
+    # batch normalization, plane size not a multiple of 4
+    shape = (6, 5, 9, 9)
+    x = rng.standard_normal(shape).astype(np.float32)
+    C = shape[1]
+    v = lambda a: CT.from_numpy(np.asarray(a, np.float32))
+    rm, rv, sm, ss = v(np.zeros(C)), v(np.ones(C)), v(np.zeros(C)), v(np.zeros(C))
+    out = CT()
+    THNN.BatchNormalization_updateOutput(_at_offset(T, x, off), out, None, None, rm, rv, sm, ss, True, 0.1, 1e-5)
+    mean = x.mean(axis=(0, 2, 3), keepdims=True, dtype=np.float64)
+    var = x.var(axis=(0, 2, 3), keepdims=True, dtype=np.float64)
+    close(out.numpy(), ((x - mean) / np.sqrt(var + 1e-5)).astype(np.float32), 1e-4, 2e-4)

@@ -354,6 +354,9 @@ struct FwdArgs {
   // tail launch: tiles tile0 .. are each reduced by nSplit workgroups over ktPerSplit k-tiles;
   // their 128x128 partial tiles go to `partial` and fwdTailFixupKernel folds them
   int tile0, nSplit, ktPerSplit;
+  // padded kernel, one launch for both: workgroups 0 .. full - 1 reduce tiles 0 .. full - 1 over all of K,
+  // workgroup full + split * tail + i reduces split `split` of tile tile0 + i (tile0 = full)
+  int full, tail;
   float *partial;
   const int *taps;    // padded kernel: byte offset of tap (c, kh, kw) inside a (zero-padded) image, per k
 };
@@ -365,9 +368,9 @@ struct FwdArgs {
 template <int TBN = BN>
 __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g, const float16v (&acc)[2][2], int bx,
                                             int by, int m0, int j0, int wm, int wn, int grp, int idx,
-                                            const float *biasLds = nullptr) {
+                                            const float *biasLds = nullptr, int toPartial = -1) {
   const int rowHalf = grp * 4;
-  if (p.nSplit > 1) {
+  if (toPartial < 0 ? p.nSplit > 1 : toPartial != 0) {
     float *dst = p.partial + ((long)bx * p.nSplit + by) * (BM * BN);  // both tile shapes hold BM * BN elements
 #pragma unroll
     for (int tj = 0; tj < 2; ++tj)
@@ -697,8 +700,10 @@ __device__ __forceinline__ void mfmaHalf(const float4 *aSrc, const float4 *bSrc,
 // Rows past M and columns past the batch are clamped to valid ones and dropped in the epilogue.
 // WM = 2: 128 x 128 tiles, the four waves as 2 x 2; WM = 1: 64 x 256 tiles, the four waves side by side,
 // for row counts whose last 128-row tile would be at most half full. A wave multiplies 64 x 64 either way.
+// (bx, by): position among the tiles that start at tile0 and split; whole: the workgroup reduces all of K
+// of tile bx and writes the output itself
 template <int WM>
-__device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &g) {
+__device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &g, int bx, int by, bool whole) {
   constexpr int TBM = 64 * WM, TBN = 256 / WM;
   constexpr int AP = TBM + 8, BP = TBN + 8;  // float4 per k-group row
   constexpr int NB = WM == 2 ? 8 : 16;        // image elements a lane gathers per k-tile
@@ -707,7 +712,7 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   __shared__ __attribute__((aligned(16))) float biasS[TBM];  // the tile's bias values: the epilogue reads them from here
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm = WM == 2 ? wave >> 1 : 0, wn = WM == 2 ? wave & 1 : wave;
-  const int tileIdx = p.tile0 + blockIdx.x;
+  const int tileIdx = whole ? bx : p.tile0 + bx;
   const int mTile = tileIdx % p.mTiles, nTile = tileIdx / p.mTiles;
   const int m0 = mTile * TBM, j0 = nTile * TBN;
   if (t < TBM) biasS[t] = p.bias && m0 + t < p.M ? p.bias[m0 + t] : 0.f;  // visible after the first barrier
@@ -738,8 +743,8 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
     const int oh = l / g.oW, ow = l - oh * g.oW;
     posOff = ((n * g.Cin * g.H + oh * g.dH) * g.W + ow * g.dW) * 4;
   }
-  const int ktBegin = blockIdx.y * p.ktPerSplit;
-  const int nkt = min(g.K / BK, ktBegin + p.ktPerSplit);  // this workgroup reduces k-tiles [ktBegin, nkt)
+  const int ktBegin = by * p.ktPerSplit;  // by == 0 for whole tiles
+  const int nkt = whole ? g.K / BK : min(g.K / BK, ktBegin + p.ktPerSplit);  // this workgroup reduces k-tiles [ktBegin, nkt)
 
   u32x4 ra[WM];
   unsigned rb[NB];
@@ -818,13 +823,20 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   step(Buf0{}, Buf1{}, kt, kt + 1 < nkt, kt + 2 < nkt);
   if (kt + 1 < nkt) step(Buf1{}, Buf0{}, kt + 1, kt + 2 < nkt, false);
   if (kt + 2 < nkt) step(Buf0{}, Buf1{}, kt + 2, false, false);
-  fwdEpilogue<TBN>(p, g, acc, blockIdx.x, blockIdx.y, m0, j0, wm, wn, grp, idx, biasS);
+  fwdEpilogue<TBN>(p, g, acc, bx, by, m0, j0, wm, wn, grp, idx, biasS, whole ? 0 : 1);
 }
 
 template <int WM>
 __global__ void __launch_bounds__(dev::kBlock, 3)
 convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
-  fwdPaddedBody<WM>(p, g);
+  int bx = blockIdx.x, by = 0;
+  const bool whole = bx < p.full;
+  if (!whole) {
+    const int u = bx - p.full;
+    by = u / p.tail;
+    bx = u - by * p.tail;
+  }
+  fwdPaddedBody<WM>(p, g, bx, by, whole);
 }
 
 // Several independent GEMMs of the same tile shape in one launch (the phases of a strided gradInput):
@@ -844,7 +856,7 @@ __global__ void __launch_bounds__(dev::kBlock, 3)
 convFwdPaddedBatchKernel(FwdBatch b) {
   const FwdBatchItem &it = b.item[blockIdx.z];
   if ((int)blockIdx.x >= it.tiles || (int)blockIdx.y >= it.p.nSplit) return;
-  fwdPaddedBody<WM>(it.p, it.g);
+  fwdPaddedBody<WM>(it.p, it.g, blockIdx.x, blockIdx.y, it.p.nSplit <= 1);
 }
 
 // out tile = bias + sum over the nSplit partial tiles (ascending split order).
@@ -1370,6 +1382,8 @@ bool forceGeneric() {
 // CUs in rounds; a last partial round would leave most CUs idle while a few
 // finish one more tile, so the tiles of that round are instead split along K
 // over all CUs (partials in scratch, folded by fwdTailFixupKernel in a fixed order).
+// Whole tiles and splits are workgroups of one launch: the splits take the slots
+// that the last whole tiles free.
 struct FwdPlan {
   int bm, bn;          // tile shape: 128 x 128, or 64 x 256 when that wastes fewer rows (padded kernel only)
   int mTiles, total, full, tail, nSplit, ktPerSplit;
@@ -1389,7 +1403,9 @@ void planTiles(FwdPlan &pl, int M, long Ncols, int nkt, bool wideOk) {
   pl.tail = 0;
   if (pl.total > cus) {
     pl.tail = pl.total % cus;
-    if (pl.tail > 0) nSplit = std::min(nkt / 4, cus / pl.tail);  // >= 4 k-tiles per split
+    // at most one split per CU, >= 4 k-tiles each (finer splits - ceil(cus / tail) - measured slower: the
+    // partial tiles cost more than the balance gains)
+    if (pl.tail > 0) nSplit = std::min(nkt / 4, cus / pl.tail);
   } else {
     // fewer tiles than CUs: every tile is split along K so that the grid fills the resident slots
     pl.tail = pl.total;
@@ -1427,16 +1443,31 @@ FwdPlan planFwdImplicit(int M, int nImages, const ConvGeom &g, bool wAligned = t
 void launchFwdKernels(hipStream_t s, const FwdPlan &pl, FwdArgs p, float *partial, const ConvGeom &gk, bool fast) {
   p.mTiles = pl.mTiles;
   p.bm = pl.bm, p.bn = pl.bn;
+  p.full = pl.full, p.tail = pl.tail;
+  if (fast) {
+    // one launch: the tiles reduced by one workgroup first, then the splits of the tail tiles, which fill
+    // the slots that the last whole tiles leave
+    p.tile0 = pl.full;
+    p.nSplit = pl.tail > 0 ? pl.nSplit : 1;
+    p.ktPerSplit = pl.tail > 0 ? pl.ktPerSplit : launch::ceilDiv(gk.K, BK);
+    p.partial = partial;
+    const dim3 grid(pl.full + pl.tail * p.nSplit);
+    if (pl.bm == 64)
+      convFwdPaddedKernel<1><<<grid, dev::kBlock, 0, s>>>(p, gk);
+    else
+      convFwdPaddedKernel<2><<<grid, dev::kBlock, 0, s>>>(p, gk);
+    THC_HIP_CHECK(hipGetLastError());
+    if (pl.tail > 0) {
+      fwdTailFixupKernel<<<dim3(pl.tail, BM * BN / (4 * dev::kBlock)), dev::kBlock, 0, s>>>(p, gk);
+      THC_HIP_CHECK(hipGetLastError());
+    }
+    return;
+  }
   p.tile0 = 0;
   p.nSplit = 1;
   p.ktPerSplit = launch::ceilDiv(gk.K, BK);
   if (pl.full > 0) {
-    if (fast && pl.bm == 64)
-      convFwdPaddedKernel<1><<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
-    else if (fast)
-      convFwdPaddedKernel<2><<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
-    else
-      convFwdImplicitKernel<<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
+    convFwdImplicitKernel<<<dim3(pl.full), dev::kBlock, 0, s>>>(p, gk);
     THC_HIP_CHECK(hipGetLastError());
   }
   if (pl.tail > 0) {
@@ -1444,12 +1475,7 @@ void launchFwdKernels(hipStream_t s, const FwdPlan &pl, FwdArgs p, float *partia
     p.ktPerSplit = pl.ktPerSplit;
     p.nSplit = pl.nSplit;
     p.partial = partial;
-    if (fast && pl.bm == 64)
-      convFwdPaddedKernel<1><<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, gk);
-    else if (fast)
-      convFwdPaddedKernel<2><<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, gk);
-    else
-      convFwdImplicitKernel<<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, gk);
+    convFwdImplicitKernel<<<dim3(pl.tail, pl.nSplit), dev::kBlock, 0, s>>>(p, gk);
     THC_HIP_CHECK(hipGetLastError());
     fwdTailFixupKernel<<<dim3(pl.tail, BM * BN / (4 * dev::kBlock)), dev::kBlock, 0, s>>>(p, gk);
     THC_HIP_CHECK(hipGetLastError());

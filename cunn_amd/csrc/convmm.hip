@@ -359,6 +359,7 @@ struct FwdArgs {
   int full, tail;
   float *partial;
   const int *taps;    // padded kernel: byte offset of tap (c, kh, kw) inside a (zero-padded) image, per k
+  int tapStride;      // > 0 (1x1 windows): tap k sits at byte offset k * tapStride, no table is read
 };
 
 // Epilogue shared by the forward kernels: a lane holds column (lane & 31) and rows
@@ -702,7 +703,9 @@ __device__ __forceinline__ void mfmaHalf(const float4 *aSrc, const float4 *bSrc,
 // for row counts whose last 128-row tile would be at most half full. A wave multiplies 64 x 64 either way.
 // (bx, by): position among the tiles that start at tile0 and split; whole: the workgroup reduces all of K
 // of tile bx and writes the output itself
-template <int WM>
+// LINEAR: 1x1 windows - the tap offsets are an arithmetic sequence, computed by the scalar unit instead of
+// read from the table
+template <int WM, bool LINEAR = false>
 __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &g, int bx, int by, bool whole) {
   constexpr int TBM = 64 * WM, TBN = 256 / WM;
   constexpr int AP = TBM + 8, BP = TBN + 8;  // float4 per k-group row
@@ -754,7 +757,14 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   int4 e[NB / 4];
   auto loadTaps = [&](int kt) {
 #pragma unroll
-    for (int i = 0; i < NB / 4; ++i) e[i] = tapBase[kt * (BK / 4) + i];
+    for (int i = 0; i < NB / 4; ++i) {
+      if (LINEAR) {
+        const int b = __builtin_amdgcn_readfirstlane((int)((unsigned)(kt * BK + kB + 4 * i) * (unsigned)p.tapStride));
+        e[i] = make_int4(b, b + p.tapStride, b + 2 * p.tapStride, b + 3 * p.tapStride);
+      } else {
+        e[i] = tapBase[kt * (BK / 4) + i];
+      }
+    }
   };
   auto loadTiles = [&](int kt) {
     const int k0 = __builtin_amdgcn_readfirstlane(kt * BK);
@@ -826,7 +836,7 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   fwdEpilogue<TBN>(p, g, acc, bx, by, m0, j0, wm, wn, grp, idx, biasS, whole ? 0 : 1);
 }
 
-template <int WM>
+template <int WM, bool LINEAR = false>
 __global__ void __launch_bounds__(dev::kBlock, 3)
 convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
   int bx = blockIdx.x, by = 0;
@@ -836,7 +846,7 @@ convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
     by = u / p.tail;
     bx = u - by * p.tail;
   }
-  fwdPaddedBody<WM>(p, g, bx, by, whole);
+  fwdPaddedBody<WM, LINEAR>(p, g, bx, by, whole);
 }
 
 // Several independent GEMMs of the same tile shape in one launch (the phases of a strided gradInput):
@@ -1452,10 +1462,16 @@ void launchFwdKernels(hipStream_t s, const FwdPlan &pl, FwdArgs p, float *partia
     p.ktPerSplit = pl.tail > 0 ? pl.ktPerSplit : launch::ceilDiv(gk.K, BK);
     p.partial = partial;
     const dim3 grid(pl.full + pl.tail * p.nSplit);
-    if (pl.bm == 64)
+    if (p.tapStride > 0) {
+      if (pl.bm == 64)
+        convFwdPaddedKernel<1, true><<<grid, dev::kBlock, 0, s>>>(p, gk);
+      else
+        convFwdPaddedKernel<2, true><<<grid, dev::kBlock, 0, s>>>(p, gk);
+    } else if (pl.bm == 64) {
       convFwdPaddedKernel<1><<<grid, dev::kBlock, 0, s>>>(p, gk);
-    else
+    } else {
       convFwdPaddedKernel<2><<<grid, dev::kBlock, 0, s>>>(p, gk);
+    }
     THC_HIP_CHECK(hipGetLastError());
     if (pl.tail > 0) {
       fwdTailFixupKernel<<<dim3(pl.tail, BM * BN / (4 * dev::kBlock)), dev::kBlock, 0, s>>>(p, gk);
@@ -1499,9 +1515,14 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
       launchPadPlanes(s, x, xp, (long)nImages * g.Cin, g.H, g.W, g.padH, g.padW);
       p.x = xp;
     }
-    buildTapTableKernel<<<launch::directGrid(pl.tapEntries, dev::kBlock), dev::kBlock, 0, s>>>(
-        reinterpret_cast<int *>(scratch), pl.tapEntries, gk);
-    THC_HIP_CHECK(hipGetLastError());
+    // 1x1 windows over a whole number of k-tiles: tap k is plane k of the image, no table needed
+    if (g.kH == 1 && g.kW == 1 && g.K % BK == 0) {
+      p.tapStride = gk.H * gk.W * (int)sizeof(float);
+    } else {
+      buildTapTableKernel<<<launch::directGrid(pl.tapEntries, dev::kBlock), dev::kBlock, 0, s>>>(
+          reinterpret_cast<int *>(scratch), pl.tapEntries, gk);
+      THC_HIP_CHECK(hipGetLastError());
+    }
     if (pl.weightFloats > 0) {
       float *wp = xp + (pl.paddedFloats + 3) / 4 * 4;
       gk.K = (int)(pl.weightFloats / M);

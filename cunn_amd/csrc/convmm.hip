@@ -430,14 +430,17 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
 // taps[k] = ((c*H + kh*dilH)*W + kw*dilW) * 4 for k = (c*kH + kh)*kW + kw; g is the geometry of the padded images.
 // Entries beyond Cin*kH*kW (rows padded to a multiple of BK, spare entries) point at the position's own
 // first element: valid memory, and their weights are zero or they are never used.
+// byte offset of tap k = (c, kh, kw) inside a (zero-bordered) image of g.H x g.W; 0 beyond the last tap
+__device__ __forceinline__ int tapOffset(int k, const ConvGeom &g) {
+  const int KK = g.kH * g.kW;
+  const int c = k / KK, rem = k - c * KK;
+  const int kh = rem / g.kW, kw = rem - kh * g.kW;
+  return c < g.Cin ? ((c * g.H + kh * g.dilH) * g.W + kw * g.dilW) * 4 : 0;
+}
+
 __global__ void __launch_bounds__(dev::kBlock)
 buildTapTableKernel(int *taps, int entries, ConvGeom g) {
-  const int KK = g.kH * g.kW;
-  for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < entries; k += gridDim.x * blockDim.x) {
-    const int c = k / KK, rem = k - c * KK;
-    const int kh = rem / g.kW, kw = rem - kh * g.kW;
-    taps[k] = c < g.Cin ? ((c * g.H + kh * g.dilH) * g.W + kw * g.dilW) * 4 : 0;
-  }
+  for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < entries; k += gridDim.x * blockDim.x) taps[k] = tapOffset(k, g);
 }
 
 // wp(rows x Kp) = w(rows x K) with zeros in columns K .. Kp-1
@@ -456,7 +459,12 @@ padRowsKernel(const float *__restrict__ w, float *__restrict__ wp, int rows, int
 // (plane size a multiple of 4 floats, 16-byte aligned destination).
 template <bool VEC>
 __global__ void __launch_bounds__(dev::kBlock)
-padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int padTop, int padLeft, int Hp, int Wp) {
+padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int padTop, int padLeft, int Hp, int Wp,
+                int planes, int *taps, int tapEntries, ConvGeom tg) {
+  if ((int)blockIdx.x == planes) {  // one more column of workgroups builds the tap table of the convolution that follows
+    for (int k = blockIdx.y * dev::kBlock + threadIdx.x; k < tapEntries; k += gridDim.y * dev::kBlock) taps[k] = tapOffset(k, tg);
+    return;
+  }
   const unsigned magic = dev::magicOf(Wp);
   const float *src = x + (long)blockIdx.x * H * W;
   float *dst = xp + (long)blockIdx.x * Hp * Wp;
@@ -474,20 +482,24 @@ padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int 
   }
 }
 
+// taps != nullptr: the same launch also builds the tap table (tapEntries entries) of geometry tg
 void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int H, int W, int padTop, int padLeft, int Hp,
-                     int Wp) {
+                     int Wp, int *taps = nullptr, int tapEntries = 0, const ConvGeom *tg = nullptr) {
   const int plane = Hp * Wp;
   if (launch::ceilDiv(plane, dev::kBlock) > 65535) error("SpatialConvolutionMM: image plane too large");
+  const unsigned gx = (unsigned)planes + (taps ? 1 : 0);
+  const ConvGeom g = tg ? *tg : ConvGeom{};
   if (plane % 4 == 0 && launch::aligned16(xp))
-    padPlanesKernel<true><<<dim3((unsigned)planes, launch::ceilDiv(plane / 4, dev::kBlock)), dev::kBlock, 0, s>>>(
-        x, xp, H, W, padTop, padLeft, Hp, Wp);
+    padPlanesKernel<true><<<dim3(gx, launch::ceilDiv(plane / 4, dev::kBlock)), dev::kBlock, 0, s>>>(
+        x, xp, H, W, padTop, padLeft, Hp, Wp, (int)planes, taps, tapEntries, g);
   else
-    padPlanesKernel<false><<<dim3((unsigned)planes, launch::ceilDiv(plane, dev::kBlock)), dev::kBlock, 0, s>>>(
-        x, xp, H, W, padTop, padLeft, Hp, Wp);
+    padPlanesKernel<false><<<dim3(gx, launch::ceilDiv(plane, dev::kBlock)), dev::kBlock, 0, s>>>(
+        x, xp, H, W, padTop, padLeft, Hp, Wp, (int)planes, taps, tapEntries, g);
   THC_HIP_CHECK(hipGetLastError());
 }
-inline void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int H, int W, int padH, int padW) {
-  launchPadPlanes(s, x, xp, planes, H, W, padH, padW, H + 2 * padH, W + 2 * padW);
+inline void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int H, int W, int padH, int padW,
+                            int *taps = nullptr, int tapEntries = 0, const ConvGeom *tg = nullptr) {
+  launchPadPlanes(s, x, xp, planes, H, W, padH, padW, H + 2 * padH, W + 2 * padW, taps, tapEntries, tg);
 }
 
 // ---- gradInput by output phase ------------------------------------------------------------------
@@ -1511,14 +1523,16 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
   if (fast) {
     gk.H = g.H + 2 * g.padH, gk.W = g.W + 2 * g.padW, gk.padH = gk.padW = 0;
     float *xp = partial + partialFloats(pl);
-    if (pl.paddedFloats > 0) {
-      launchPadPlanes(s, x, xp, (long)nImages * g.Cin, g.H, g.W, g.padH, g.padW);
+    // 1x1 windows over a whole number of k-tiles: tap k is plane k of the image, no table needed
+    const bool linear = g.kH == 1 && g.kW == 1 && g.K % BK == 0;
+    if (pl.paddedFloats > 0) {  // the copy into the bordered layout builds the tap table on the side
+      launchPadPlanes(s, x, xp, (long)nImages * g.Cin, g.H, g.W, g.padH, g.padW, linear ? nullptr : reinterpret_cast<int *>(scratch),
+                      pl.tapEntries, &gk);
       p.x = xp;
     }
-    // 1x1 windows over a whole number of k-tiles: tap k is plane k of the image, no table needed
-    if (g.kH == 1 && g.kW == 1 && g.K % BK == 0) {
+    if (linear) {
       p.tapStride = gk.H * gk.W * (int)sizeof(float);
-    } else {
+    } else if (pl.paddedFloats <= 0) {
       buildTapTableKernel<<<launch::directGrid(pl.tapEntries, dev::kBlock), dev::kBlock, 0, s>>>(
           reinterpret_cast<int *>(scratch), pl.tapEntries, gk);
       THC_HIP_CHECK(hipGetLastError());

@@ -947,17 +947,34 @@ struct GradWeightArgs {
 };
 
 // WM = 2: 128 x 128 tiles of gradWeight (Cout x K), WM = 1: 64 x 256 tiles (as in the forward kernel).
-template <bool L16, int WM>
+// WM = 0: 64 x 64 tiles for small gradWeights (first layers, narrow 1x1 convolutions), where the large tiles
+// would spend most of their multiplications on padding: the four waves all own the whole tile and take one
+// position group (4 of the 16 positions) of every k-tile each, i.e. a wave is a split of its own - it stores
+// its partial under split index 4 * split + wave and the fold adds them like any other splits.
+template <int OA, int OB>
+__device__ __forceinline__ void mfmaGroupPair(const float *aSrc, const float *bSrc, float16v (&acc)[2][2]) {
+  // lanes 0-31 hold position OA / OB of the group, lanes 32-63 the next one (aSrc / bSrc already point there)
+  const float a0 = aSrc[OA], a1 = aSrc[OA + 32 * 4];
+  const float b0 = bSrc[OB], b1 = bSrc[OB + 32 * 4];
+  acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+  acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+  acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+  acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+}
+
+template <bool L16, int WMODE>
 __global__ void __launch_bounds__(dev::kBlock, 3)
 convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
-  constexpr int TBM = 64 * WM, TBN = 256 / WM;
+  constexpr bool TINY = WMODE == 0;
+  constexpr int WM = TINY ? 1 : WMODE;  // loader layout: 64 rows as in the 64 x 256 shape
+  constexpr int TBM = 64 * WM, TBN = TINY ? 64 : 256 / WM;
   constexpr int AP = TBM + 8;   // float4 per position-group row of As
   constexpr int GP = TBN + 4;   // of Bs: the 4 groups of a wave's scalar stores hit disjoint banks
   constexpr int NB = TBN / 16;  // columns a lane gathers per k-tile
   __shared__ float4 As[2][BK / 4][AP];
   __shared__ float4 Bs[2][BK / 4][GP];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int wm = WM == 2 ? wave >> 1 : 0, wn = WM == 2 ? wave & 1 : wave;
+  const int wm = WM == 2 ? wave >> 1 : 0, wn = TINY ? 0 : (WM == 2 ? wave & 1 : wave);
   // workgroups that reduce the same positions (one split) are neighbours in the remapped order: same XCD, same L2
   const int tilesPerSplit = p.mTiles * p.nTiles;
   const int bid = dev::xcdRemap(blockIdx.x, gridDim.x);
@@ -1072,18 +1089,27 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   const int grp = lane >> 5, idx = lane & 31;
   const float4 *aSrc = &As[0][grp][wm * 64 + idx];
   const float4 *bSrc = &Bs[0][grp][wn * 64 + idx];
+  // small tiles: this wave's position group, element grp (then grp + 2) of its float4
+  const float *aTiny = reinterpret_cast<const float *>(&As[0][wave][idx]) + grp;
+  const float *bTiny = reinterpret_cast<const float *>(&Bs[0][wave][idx]) + grp;
   using Buf0 = std::integral_constant<int, 0>;
   using Buf1 = std::integral_constant<int, 1>;
 
   // same software pipeline as the forward kernel: tile kt in LDS, kt + 1 in registers, kt + 2 requested
   auto step = [&](auto cur, auto nxt, bool store, bool load) {
     constexpr int C = decltype(cur)::value;
-    mfmaHalf<C * BUFA, C * BUFB>(aSrc, bSrc, acc);
+    if constexpr (TINY)
+      mfmaGroupPair<C * BUFA * 4, C * BUFB * 4>(aTiny, bTiny, acc);
+    else
+      mfmaHalf<C * BUFA, C * BUFB>(aSrc, bSrc, acc);
     __builtin_amdgcn_sched_barrier(0);
     if (store) storeTiles(nxt);
     if (load) loadTiles();
     __builtin_amdgcn_sched_barrier(0);
-    mfmaHalf<C * BUFA + 2 * AP, C * BUFB + 2 * GP>(aSrc, bSrc, acc);
+    if constexpr (TINY)
+      mfmaGroupPair<C * BUFA * 4 + 2, C * BUFB * 4 + 2>(aTiny, bTiny, acc);
+    else
+      mfmaHalf<C * BUFA + 2 * AP, C * BUFB + 2 * GP>(aSrc, bSrc, acc);
     __syncthreads();
   };
   if (ktBegin < ktEnd) {
@@ -1103,7 +1129,7 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   }
 
   // lane holds column (lane & 31), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
-  float *dst = p.partial + (long)split * p.M * p.Ncols;
+  float *dst = p.partial + (long)(TINY ? split * 4 + wave : split) * p.M * p.Ncols;
 #pragma unroll
   for (int tj = 0; tj < 2; ++tj) {
     const int col = j0 + wn * 64 + tj * 32 + idx;
@@ -1120,7 +1146,14 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
     // the 2 (WM = 2) or 4 (WM = 1) lanes that loaded parts of a row are neighbours inside a quad
     rowSum = dev::dppAdd<0xB1>(rowSum);
     if (WM == 1) rowSum = dev::dppAdd<0x4E>(rowSum);
-    if ((t & (WM == 2 ? 1 : 3)) == 0 && m0 + rowA < p.M) p.biasPartial[(long)split * p.M + m0 + rowA] = rowSum;
+    if ((t & (WM == 2 ? 1 : 3)) == 0 && m0 + rowA < p.M) {
+      if (TINY) {  // four partial slots per workgroup: the row sums go to the first, the others add nothing
+        float *bp = p.biasPartial + (long)split * 4 * p.M + m0 + rowA;
+        bp[0] = rowSum, bp[p.M] = 0.f, bp[2 * (long)p.M] = 0.f, bp[3 * (long)p.M] = 0.f;
+      } else {
+        p.biasPartial[(long)split * p.M + m0 + rowA] = rowSum;
+      }
+    }
   }
 }
 
@@ -1130,28 +1163,32 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
 // LDS. With few elements and hundreds of splits (1x1 convolutions) a one-lane-per-element loop is
 // latency bound; this form keeps enough bytes in flight to run at memory speed.
 // Blocks past the last float4 of gW do the same for the bias partials (biasPartial(splits, M), M % 4 == 0), when given.
+// E: float4 of gW a workgroup owns (64, 16 or 4); its 256 / E lane groups share the splits. Small
+// gradWeights with thousands of splits take small E: more workgroups, more loads in flight.
+template <int E>
 __global__ void __launch_bounds__(dev::kBlock)
 foldPartials4Kernel(const float *__restrict__ partial, float *__restrict__ dst, long count4, int splits, float scale,
                     const float *__restrict__ biasPartial, float *__restrict__ gradBias, int M, int gwBlocks) {
-  __shared__ float4 part[4][64];
+  constexpr int G = dev::kBlock / E;
+  __shared__ float4 part[G][E];
   int blk = blockIdx.x;
   if (blk >= gwBlocks) blk -= gwBlocks, partial = biasPartial, dst = gradBias, count4 = M >> 2;
-  const int e = threadIdx.x & 63, grp = threadIdx.x >> 6;
-  const long i = (long)blk * 64 + e;
+  const int e = threadIdx.x % E, grp = threadIdx.x / E;
+  const long i = (long)blk * E + e;
   float4 a[4];
 #pragma unroll
   for (int u = 0; u < 4; ++u) a[u] = make_float4(0.f, 0.f, 0.f, 0.f);
   if (i < count4) {
     const float4 *p = reinterpret_cast<const float4 *>(partial) + i;
     int s = grp;
-    for (; s + 12 < splits; s += 16) {
+    for (; s + 3 * G < splits; s += 4 * G) {
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const float4 v = p[(long)(s + 4 * u) * count4];
+        const float4 v = p[(long)(s + G * u) * count4];
         a[u].x += v.x, a[u].y += v.y, a[u].z += v.z, a[u].w += v.w;
       }
     }
-    for (; s < splits; s += 4) {
+    for (; s < splits; s += G) {
       const float4 v = p[(long)s * count4];
       a[0].x += v.x, a[0].y += v.y, a[0].z += v.z, a[0].w += v.w;
     }
@@ -1160,10 +1197,15 @@ foldPartials4Kernel(const float *__restrict__ partial, float *__restrict__ dst, 
                              (a[0].z + a[1].z) + (a[2].z + a[3].z), (a[0].w + a[1].w) + (a[2].w + a[3].w));
   __syncthreads();
   if (grp == 0 && i < count4) {
-    const float4 p0 = part[0][e], p1 = part[1][e], p2 = part[2][e], p3 = part[3][e];
+    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
+    for (int q = 0; q < G; q += 4) {
+      const float4 p0 = part[q][e], p1 = part[q + 1][e], p2 = part[q + 2][e], p3 = part[q + 3][e];
+      t.x += (p0.x + p1.x) + (p2.x + p3.x), t.y += (p0.y + p1.y) + (p2.y + p3.y);
+      t.z += (p0.z + p1.z) + (p2.z + p3.z), t.w += (p0.w + p1.w) + (p2.w + p3.w);
+    }
     float4 d = reinterpret_cast<float4 *>(dst)[i];
-    d.x += scale * ((p0.x + p1.x) + (p2.x + p3.x)), d.y += scale * ((p0.y + p1.y) + (p2.y + p3.y));
-    d.z += scale * ((p0.z + p1.z) + (p2.z + p3.z)), d.w += scale * ((p0.w + p1.w) + (p2.w + p3.w));
+    d.x += scale * t.x, d.y += scale * t.y, d.z += scale * t.z, d.w += scale * t.w;
     reinterpret_cast<float4 *>(dst)[i] = d;
   }
 }
@@ -1912,18 +1954,27 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   const bool l16 = g.L % BK == 0;
   // tile shape: 64 x 256 where it covers gradWeight (Cout x K) with less padding than 128 x 128
   const bool wide = fast && tiles(g.Cout, 64) * 64 * tiles(g.K, 256) * 256 < tiles(g.Cout, BM) * BM * tiles(g.K, BN) * BN;
-  const int mT = (int)tiles(g.Cout, wide ? 64 : BM), nT = (int)tiles(g.K, wide ? 256 : BN);
-  const void *kern = !fast ? (const void *)convGemmKernel<kGradWeight>
-                     : l16 ? (wide ? (const void *)convGradWeightKernel<true, 1> : (const void *)convGradWeightKernel<true, 2>)
-                           : (wide ? (const void *)convGradWeightKernel<false, 1> : (const void *)convGradWeightKernel<false, 2>);
+  // 64 x 64 tiles (the waves of a workgroup split the positions instead of the tile) where the large shapes
+  // would multiply at least four times as much padding: small gradWeights are bound by memory, not by the matrix pipe
+  const long bigArea = std::min(tiles(g.Cout, 64) * 64 * tiles(g.K, 256) * 256, tiles(g.Cout, BM) * BM * tiles(g.K, BN) * BN);
+  const bool tiny = fast && tiles(g.Cout, 64) * 64 * tiles(g.K, 64) * 64 * 4 <= bigArea;
+  const int mT = (int)tiles(g.Cout, tiny || wide ? 64 : BM), nT = (int)tiles(g.K, tiny ? 64 : wide ? 256 : BN);
+  const void *kern =
+      !fast  ? (const void *)convGemmKernel<kGradWeight>
+      : tiny ? (l16 ? (const void *)convGradWeightKernel<true, 0> : (const void *)convGradWeightKernel<false, 0>)
+      : l16  ? (wide ? (const void *)convGradWeightKernel<true, 1> : (const void *)convGradWeightKernel<true, 2>)
+             : (wide ? (const void *)convGradWeightKernel<false, 1> : (const void *)convGradWeightKernel<false, 2>);
   // Every split leaves a partial copy of gradWeight (64 KB per tile) for the fold: three workgroups per CU
   // measured better than the four that fit (less partial traffic for the same matrix-pipe load), two when
-  // gradWeight is one or two tiles and the partials are most of the traffic.
-  const int perCu = mT * nT <= 2 ? 2 : 3;
+  // gradWeight is one or two tiles and the partials are most of the traffic. The small tiles stream: as many
+  // workgroups as fit, to have enough loads in flight.
+  const int perCu = tiny ? 4 : mT * nT <= 2 ? 2 : 3;
   const int slots = std::min(residentSlots(kern), residentSlots(nullptr) * perCu);
   int splits = std::max(1, std::min(totalKt, slots / (mT * nT)));
   const int perSplit = launch::ceilDiv(totalKt, splits);
   splits = launch::ceilDiv(totalKt, perSplit);
+  const int wgSplits = splits;       // splits of the positions over workgroups
+  if (tiny) splits *= 4;             // partial copies of gradWeight: one per wave
   const long count = (long)g.Cout * g.K;
   // scratch: the splits' partial products, then (second-generation kernel) the images with their zero border
   const long partialFloats = (splits * count + 3) / 4 * 4;
@@ -1958,8 +2009,12 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     q.gyBytes = (int)gyBytes;
     q.xBytes = (int)(xpFloats * 4);
     q.magicOW = dev::magicOf(g.oW);
-    const dim3 grid(mT * nT * splits);
-    if (l16 && wide)
+    const dim3 grid(mT * nT * wgSplits);
+    if (tiny && l16)
+      convGradWeightKernel<true, 0><<<grid, dev::kBlock, 0, s>>>(q, gk);
+    else if (tiny)
+      convGradWeightKernel<false, 0><<<grid, dev::kBlock, 0, s>>>(q, gk);
+    else if (l16 && wide)
       convGradWeightKernel<true, 1><<<grid, dev::kBlock, 0, s>>>(q, gk);
     else if (l16)
       convGradWeightKernel<true, 2><<<grid, dev::kBlock, 0, s>>>(q, gk);
@@ -1984,10 +2039,19 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   }
   THC_HIP_CHECK(hipGetLastError());
   if (fold4) {  // (the scratch starts on a 16-byte boundary)
-    const int gwBlocks = (int)((count / 4 + 63) / 64);
-    const int biasBlocks = fusedBias ? launch::ceilDiv(g.Cout / 4, 64) : 0;
-    foldPartials4Kernel<<<gwBlocks + biasBlocks, dev::kBlock, 0, s>>>(partial, gW, count / 4, splits, scale, biasPartial,
-                                                                       gB, g.Cout, gwBlocks);
+    // elements per workgroup: the fewest (most lane groups over the splits) that still give 128 workgroups
+    const int E = count / 4 >= 128 * 64 ? 64 : count / 4 >= 128 * 16 ? 16 : 4;
+    const int gwBlocks = (int)((count / 4 + E - 1) / E);
+    const int biasBlocks = fusedBias ? launch::ceilDiv(g.Cout / 4, E) : 0;
+    if (E == 64)
+      foldPartials4Kernel<64><<<gwBlocks + biasBlocks, dev::kBlock, 0, s>>>(partial, gW, count / 4, splits, scale, biasPartial,
+                                                                           gB, g.Cout, gwBlocks);
+    else if (E == 16)
+      foldPartials4Kernel<16><<<gwBlocks + biasBlocks, dev::kBlock, 0, s>>>(partial, gW, count / 4, splits, scale, biasPartial,
+                                                                           gB, g.Cout, gwBlocks);
+    else
+      foldPartials4Kernel<4><<<gwBlocks + biasBlocks, dev::kBlock, 0, s>>>(partial, gW, count / 4, splits, scale, biasPartial,
+                                                                          gB, g.Cout, gwBlocks);
   } else {
     foldPartialsKernel<<<launch::directGrid(count, dev::kBlock), dev::kBlock, 0, s>>>(partial, gW, count, splits, scale);
   }

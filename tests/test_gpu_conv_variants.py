@@ -197,6 +197,13 @@ TILE_CASES = [
     (32, 16, 64, 48, 48, 3, 3, 1, 1, 1, 1, 1, 1),    # 64 rows, more tiles than CUs: full rounds + K-split tail
     (3, 3, 64, 40, 40, 7, 7, 2, 2, 3, 3, 1, 1),      # K = 147 padded to 160, stride 2
     (2, 24, 48, 18, 22, 3, 3, 1, 1, 1, 1, 1, 1),     # 64 x 256 weight-gradient tiles with L % 16 != 0
+    # 64 x 64 weight-gradient tiles (the waves split the positions): narrow 1x1, first layers, L % 16 != 0,
+    # Cout not a multiple of 4 (bias gradient in a pass of its own), 1x1 forward without a tap table
+    (6, 32, 64, 28, 28, 1, 1, 1, 1, 0, 0, 1, 1),
+    (4, 3, 32, 64, 64, 3, 3, 2, 2, 1, 1, 1, 1),
+    (3, 5, 20, 18, 18, 3, 3, 1, 1, 1, 1, 1, 1),
+    (2, 16, 27, 20, 24, 1, 1, 1, 1, 0, 0, 1, 1),
+    (2, 48, 96, 12, 12, 1, 1, 1, 1, 0, 0, 1, 1),     # 1x1, K = 48: three k-tiles, computed tap offsets
 ]
 
 

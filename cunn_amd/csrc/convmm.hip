@@ -482,6 +482,32 @@ padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int 
   }
 }
 
+// The same for small planes (7x7 ... 28x28 stages: a workgroup per plane would leave most lanes idle): a lane per
+// 16-byte group of the whole destination. Workgroups past copyBlocks build the tap table.
+__global__ void __launch_bounds__(dev::kBlock)
+padPlanesFlatKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int padTop, int padLeft, int Hp, int Wp,
+                    long total4, int copyBlocks, int *taps, int tapEntries, ConvGeom tg) {
+  if ((int)blockIdx.x >= copyBlocks) {
+    for (int k = (blockIdx.x - copyBlocks) * dev::kBlock + threadIdx.x; k < tapEntries; k += (gridDim.x - copyBlocks) * dev::kBlock)
+      taps[k] = tapOffset(k, tg);
+    return;
+  }
+  const int plane4 = (Hp * Wp) >> 2;
+  const unsigned magicPlane = dev::magicOf(plane4), magicW = dev::magicOf(Wp);
+  for (long i = (long)blockIdx.x * dev::kBlock + threadIdx.x; i < total4; i += (long)copyBlocks * dev::kBlock) {
+    const int pl = dev::fastDiv((int)i, magicPlane), j = ((int)i - pl * plane4) * 4;
+    const float *src = x + (long)pl * H * W;
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int hp = dev::fastDiv(j + k, magicW), wp = j + k - hp * Wp;
+      const int h = hp - padTop, w = wp - padLeft;
+      v[k] = (((unsigned)h < (unsigned)H) & ((unsigned)w < (unsigned)W)) ? src[h * W + w] : 0.f;
+    }
+    reinterpret_cast<float4 *>(xp)[i] = make_float4(v[0], v[1], v[2], v[3]);
+  }
+}
+
 // taps != nullptr: the same launch also builds the tap table (tapEntries entries) of geometry tg
 void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int H, int W, int padTop, int padLeft, int Hp,
                      int Wp, int *taps = nullptr, int tapEntries = 0, const ConvGeom *tg = nullptr) {
@@ -489,7 +515,14 @@ void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int 
   if (launch::ceilDiv(plane, dev::kBlock) > 65535) error("SpatialConvolutionMM: image plane too large");
   const unsigned gx = (unsigned)planes + (taps ? 1 : 0);
   const ConvGeom g = tg ? *tg : ConvGeom{};
-  if (plane % 4 == 0 && launch::aligned16(xp))
+  const long total4 = planes * (plane / 4);
+  // (the reciprocal division of a group index by the groups per plane is exact while index * divisor < 2^32)
+  if (plane % 4 == 0 && plane < 4096 && launch::aligned16(xp) && total4 * (plane / 4) < 0xffffffffL) {
+    const int copyBlocks = (int)std::min<long>((total4 + dev::kBlock - 1) / dev::kBlock, 16384);
+    const int tapBlocks = taps ? std::max(1, std::min(16, launch::ceilDiv(tapEntries, dev::kBlock))) : 0;
+    padPlanesFlatKernel<<<copyBlocks + tapBlocks, dev::kBlock, 0, s>>>(x, xp, H, W, padTop, padLeft, Hp, Wp, total4, copyBlocks,
+                                                                      taps, tapEntries, g);
+  } else if (plane % 4 == 0 && launch::aligned16(xp))
     padPlanesKernel<true><<<dim3(gx, launch::ceilDiv(plane / 4, dev::kBlock)), dev::kBlock, 0, s>>>(
         x, xp, H, W, padTop, padLeft, Hp, Wp, (int)planes, taps, tapEntries, g);
   else
@@ -1943,15 +1976,26 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   // resident workgroup slots of the chip exactly once: with fewer, fatter
   // splits some CUs would carry one workgroup more than others for the whole
   // kernel.
-  if ((long)g.N * g.L >= 0x7fffffffL) error("spatial convolution: batch too large");
-  const int totalKt = launch::ceilDiv(g.N * g.L, BK);
+  // The second-generation kernel loads 4 consecutive positions of a gradOutput row as one 16-byte group. Rows
+  // whose length is not a multiple of 4 (7x7, 13x13, 27x27 ... planes) or that start off a 16-byte boundary are
+  // first copied into rows padded with zeros to a multiple of 4: the added positions contribute nothing, and the
+  // image rows they stand for are zero rows appended to the bordered copy of the images.
+  const int Lp = launch::roundUp(g.L, 4);
+  const bool padGy = !forceGeneric() && (g.L % 4 != 0 || !launch::aligned16(gy)) && Lp >= BK;
+  const int Lk = padGy ? Lp : g.L;  // positions per image as the kernel sees them
+  if ((long)g.N * Lk >= 0x7fffffffL) error("spatial convolution: batch too large");
+  const int totalKt = launch::ceilDiv(g.N * Lk, BK);
+  // output rows the added positions spill into, and the image rows their windows reach
+  const int extraRows = Lk > g.L ? (Lk - g.L - 1) / g.oW + 1 : 0;
+  const int HpX = std::max(g.H + 2 * g.padH, (g.oH - 1 + extraRows) * g.dH + (g.kH - 1) * g.dilH + 1);
   // second-generation kernel: gradOutput rows loadable as float4 groups, 32-bit byte offsets into both operands
-  const bool bordered = g.padH > 0 || g.padW > 0;
-  const long gyBytes = (long)g.N * g.Cout * g.L * 4;
-  const long xpFloats = (long)g.N * g.Cin * (g.H + 2 * g.padH) * (g.W + 2 * g.padW);
-  const bool fast = !forceGeneric() && g.L % 4 == 0 && g.L >= BK && launch::aligned16(gy) &&
-                    gyBytes < 0x7fffffffL && xpFloats * 4 < 0x7fffffffL - 65536 && (long)g.L * g.oW < 0x7fffffffL;
-  const bool l16 = g.L % BK == 0;
+  const bool bordered = g.padH > 0 || g.padW > 0 || extraRows > 0;
+  const long gyBytes = (long)g.N * g.Cout * Lk * 4;
+  const long xpFloats = (long)g.N * g.Cin * HpX * (g.W + 2 * g.padW);
+  const long gypFloats = padGy ? (long)g.N * g.Cout * Lp : 0;
+  const bool fast = !forceGeneric() && Lk % 4 == 0 && Lk >= BK && (padGy || launch::aligned16(gy)) &&
+                    gyBytes < 0x7fffffffL && xpFloats * 4 < 0x7fffffffL - 65536 && (long)Lk * g.oW < 0x7fffffffL;
+  const bool l16 = Lk % BK == 0;
   // tile shape: 64 x 256 where it covers gradWeight (Cout x K) with less padding than 128 x 128
   const bool wide = fast && tiles(g.Cout, 64) * 64 * tiles(g.K, 256) * 256 < tiles(g.Cout, BM) * BM * tiles(g.K, BN) * BN;
   // 64 x 64 tiles (the waves of a workgroup split the positions instead of the tile) where the large shapes
@@ -1983,20 +2027,26 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   const bool fusedBias = gB && fast && fold4 && g.Cout % 4 == 0 && launch::aligned16(gB);
   const long biasFloats = fusedBias ? ((long)splits * g.Cout + 3) / 4 * 4 : 0;
   Temp tmp;
-  float *partial =
-      scratchFloats(state, scratchBuf, partialFloats + biasFloats + (fast && bordered ? xpFloats : 0), tmp, "columns");
+  const long xpScratch = fast && bordered ? (xpFloats + 3) / 4 * 4 : 0;
+  float *partial = scratchFloats(state, scratchBuf, partialFloats + biasFloats + xpScratch + (fast ? gypFloats : 0), tmp, "columns");
   float *biasPartial = fusedBias ? partial + partialFloats : nullptr;
   if (fast) {
     ConvGeom gk = g;
-    const float *xk = x;
+    const float *xk = x, *gyk = gy;
     if (bordered) {
       float *xp = partial + partialFloats + biasFloats;
-      launchPadPlanes(s, x, xp, (long)g.N * g.Cin, g.H, g.W, g.padH, g.padW);
-      gk.H = g.H + 2 * g.padH, gk.W = g.W + 2 * g.padW, gk.padH = gk.padW = 0;
+      launchPadPlanes(s, x, xp, (long)g.N * g.Cin, g.H, g.W, g.padH, g.padW, HpX, g.W + 2 * g.padW);
+      gk.H = HpX, gk.W = g.W + 2 * g.padW, gk.padH = gk.padW = 0;
       xk = xp;
     }
+    if (padGy) {  // rows of L floats -> rows of Lp floats, zeros behind
+      float *gyp = partial + partialFloats + biasFloats + xpScratch;
+      launchPadPlanes(s, gy, gyp, (long)g.N * g.Cout, 1, g.L, 0, 0, 1, Lp);
+      gk.L = Lp;
+      gyk = gyp;
+    }
     GradWeightArgs q{};
-    q.gy = gy;
+    q.gy = gyk;
     q.x = xk;
     q.partial = partial;
     q.biasPartial = biasPartial;

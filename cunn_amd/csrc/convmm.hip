@@ -977,6 +977,7 @@ struct GradWeightArgs {
   int totalKt, ktPerSplit;  // k-tiles of BK positions over the N*L positions; per split
   int gyBytes, xBytes;      // < 2^31
   unsigned magicOW;
+  int Lvalid;               // positions of an image (g.L may count the padding of the gradOutput rows)
 };
 
 // WM = 2: 128 x 128 tiles of gradWeight (Cout x K), WM = 1: 64 x 256 tiles (as in the forward kernel).
@@ -1087,7 +1088,10 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
       if (lA >= g.L) lA -= g.L, ++nA;
     }
     {
-      const int oh = dev::fastDiv(lB, p.magicOW), ow = lB - oh * g.oW;
+      // (positions behind the image's last one exist when the gradOutput rows were padded to a multiple of 4:
+      // their gradOutput is zero, they read the image at position 0)
+      const int lq = lB < p.Lvalid ? lB : 0;
+      const int oh = dev::fastDiv(lq, p.magicOW), ow = lq - oh * g.oW;
       const int posOff = nOffB + oh * rowStepB + ow * colStepB;
 #pragma unroll
       for (int i = 0; i < NB; ++i)
@@ -1981,18 +1985,16 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   // kernel.
   // The second-generation kernel loads 4 consecutive positions of a gradOutput row as one 16-byte group. Rows
   // whose length is not a multiple of 4 (7x7, 13x13, 27x27 ... planes) or that start off a 16-byte boundary are
-  // first copied into rows padded with zeros to a multiple of 4: the added positions contribute nothing, and the
-  // image rows they stand for are zero rows appended to the bordered copy of the images.
+  // first copied into rows padded with zeros to a multiple of 4: the added positions contribute nothing (the
+  // kernel lets them read position 0 of the image).
   const int Lp = launch::roundUp(g.L, 4);
   const bool padGy = !forceGeneric() && (g.L % 4 != 0 || !launch::aligned16(gy)) && Lp >= BK;
   const int Lk = padGy ? Lp : g.L;  // positions per image as the kernel sees them
   if ((long)g.N * Lk >= 0x7fffffffL) error("spatial convolution: batch too large");
   const int totalKt = launch::ceilDiv(g.N * Lk, BK);
-  // output rows the added positions spill into, and the image rows their windows reach
-  const int extraRows = Lk > g.L ? (Lk - g.L - 1) / g.oW + 1 : 0;
-  const int HpX = std::max(g.H + 2 * g.padH, (g.oH - 1 + extraRows) * g.dH + (g.kH - 1) * g.dilH + 1);
+  const int HpX = g.H + 2 * g.padH;
   // second-generation kernel: gradOutput rows loadable as float4 groups, 32-bit byte offsets into both operands
-  const bool bordered = g.padH > 0 || g.padW > 0 || extraRows > 0;
+  const bool bordered = g.padH > 0 || g.padW > 0;
   const long gyBytes = (long)g.N * g.Cout * Lk * 4;
   const long xpFloats = (long)g.N * g.Cin * HpX * (g.W + 2 * g.padW);
   const long gypFloats = padGy ? (long)g.N * g.Cout * Lp : 0;
@@ -2004,7 +2006,8 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   // 64 x 64 tiles (the waves of a workgroup split the positions instead of the tile) where the large shapes
   // would multiply at least four times as much padding: small gradWeights are bound by memory, not by the matrix pipe
   const long bigArea = std::min(tiles(g.Cout, 64) * 64 * tiles(g.K, 256) * 256, tiles(g.Cout, BM) * BM * tiles(g.K, BN) * BN);
-  const bool tiny = fast && tiles(g.Cout, 64) * 64 * tiles(g.K, 64) * 64 * 4 <= bigArea;
+  const int tinyPct = 120;  // 64 x 64 tiles whenever they cut the padded area by a fifth: measured faster down to that
+  const bool tiny = fast && tiles(g.Cout, 64) * 64 * tiles(g.K, 64) * 64 * tinyPct <= bigArea * 100;
   const int mT = (int)tiles(g.Cout, tiny || wide ? 64 : BM), nT = (int)tiles(g.K, tiny ? 64 : wide ? 256 : BN);
   const void *kern =
       !fast  ? (const void *)convGemmKernel<kGradWeight>
@@ -2015,7 +2018,7 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   // measured better than the four that fit (less partial traffic for the same matrix-pipe load), two when
   // gradWeight is one or two tiles and the partials are most of the traffic. The small tiles stream: as many
   // workgroups as fit, to have enough loads in flight.
-  const int perCu = tiny ? 4 : mT * nT <= 2 ? 2 : 3;
+  const int perCu = mT * nT <= 2 ? 2 : tiny ? 4 : 3;
   const int slots = std::min(residentSlots(kern), residentSlots(nullptr) * perCu);
   int splits = std::max(1, std::min(totalKt, slots / (mT * nT)));
   const int perSplit = launch::ceilDiv(totalKt, splits);
@@ -2062,6 +2065,7 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     q.gyBytes = (int)gyBytes;
     q.xBytes = (int)(xpFloats * 4);
     q.magicOW = dev::magicOf(g.oW);
+    q.Lvalid = g.L;
     const dim3 grid(mT * nT * wgSplits);
     if (tiny && l16)
       convGradWeightKernel<true, 0><<<grid, dev::kBlock, 0, s>>>(q, gk);

@@ -1508,9 +1508,11 @@ void planTiles(FwdPlan &pl, int M, long Ncols, int nkt, bool wideOk) {
     // partial tiles cost more than the balance gains)
     if (pl.tail > 0) nSplit = std::min(nkt / 4, cus / pl.tail);
   } else {
-    // fewer tiles than CUs: every tile is split along K so that the grid fills the resident slots
+    // fewer tiles than CUs: every tile is split along K so that the grid occupies the chip
     pl.tail = pl.total;
-    nSplit = std::min(nkt / 4, residentSlots((const void *)convFwdPaddedKernel<2>) / pl.total);
+    // (two workgroups per CU measured best on 7x7 and 14x14 layers: each further split is another partial tile
+    // to write and fold)
+    nSplit = std::min(nkt / 4, std::min(residentSlots((const void *)convFwdPaddedKernel<2>), 2 * cus) / pl.total);
   }
   if (nSplit < 2) {
     pl.tail = 0;

@@ -60,6 +60,45 @@ def _dil_run(T, case, bias=True, xt=None, scale=1.0, seed=80, single=False):
         close(tgb.numpy(), rgb, WG_RTOL, WG_ATOL * max(1.0, abs(scale)) * 4)
 
 
+def _offset_tensor(T, a, off):
+    """A contiguous tensor whose first element sits `off` floats behind a 16-byte boundary of its storage."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    big = T.CudaTensor.with_size(a.size + 8)
+    big.fill(float("nan"))
+    strides = [1] * a.ndim
+    for d in range(a.ndim - 2, -1, -1):
+        strides[d] = strides[d + 1] * a.shape[d + 1]
+    v = big.view(off, a.shape, strides)
+    v.copy_(a)
+    return v
+
+
+@pytest.mark.parametrize("case,off", [
+    ((3, 8, 20, 9, 9, 3, 3, 1, 1, 1, 1), 0),      # 81 positions per image: rows padded to 84
+    ((2, 16, 24, 7, 7, 1, 1, 1, 1, 0, 0), 0),     # 1x1 at 7x7: padded rows, images read in place
+    ((2, 8, 20, 8, 8, 3, 3, 1, 1, 1, 1), 1),      # rows of 64 floats that start off a 16-byte boundary
+    ((2, 5, 12, 13, 11, 3, 3, 2, 2, 1, 1), 3),    # stride 2, 42 positions, odd offset
+])
+def test_weight_gradient_with_unaligned_gradoutput_rows(T, case, off):
+    """gradOutput rows that are not whole 16-byte groups (length not a multiple of 4, or the tensor starts off a
+    16-byte boundary) are copied into zero-padded rows first; the padding must not reach any sum."""
+    N, Cin, Cout, H, W, kW, kH, dW, dH, pW, pH = case
+    THNN, CT = T.THNN, T.CudaTensor
+    rng = np.random.default_rng(90 + off)
+    K = Cin * kH * kW
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    oH, oW = (H + 2 * pH - kH) // dH + 1, (W + 2 * pW - kW) // dW + 1
+    gy = rng.standard_normal((N, Cout, oH, oW)).astype(np.float32)
+    gw0 = rng.standard_normal((Cout, K)).astype(np.float32)
+    gb0 = rng.standard_normal(Cout).astype(np.float32)
+    tgw, tgb = CT.from_numpy(gw0), CT.from_numpy(gb0)
+    tgy = _offset_tensor(T, gy, off) if off else CT.from_numpy(gy)
+    THNN.SpatialConvolutionMM_accGradParameters(CT.from_numpy(x), tgy, tgw, tgb, CT(), CT(), kW, kH, dW, dH, pW, pH, 0.5)
+    rgw, rgb = O.dilconv_accGradParameters(x, gy, gw0.copy(), gb0.copy(), kW, kH, dW, dH, pW, pH, 1, 1, scale=0.5)
+    close(tgw.numpy(), rgw, WG_RTOL, WG_ATOL * 4)
+    close(tgb.numpy(), rgb, WG_RTOL, WG_ATOL * 4)
+
+
 @pytest.mark.parametrize("case", DIL_CASES)
 def test_dilated_convolution(T, case):
     _dil_run(T, case)

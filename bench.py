@@ -96,6 +96,10 @@ def wl_dw(cfg, nsets):
     from oracle import oracle as O
     if cfg == "cfg1":
         N, Cc, H, k, s, p, seed, full = 32, 32, 112, 3, 1, 1, 0, False
+    elif cfg == "dw147":  # a plane width that is not a multiple of 4 (Xception entry flow): bands of rows per workgroup
+        N, Cc, H, k, s, p, seed, full = 32, 128, 147, 3, 1, 1, 5, True
+    elif cfg == "dw14":   # small planes (MobileNet 14x14 stage): several planes per workgroup
+        N, Cc, H, k, s, p, seed, full = 64, 512, 14, 3, 1, 1, 6, True
     else:
         N, Cc, H, k, s, p, seed, full = 64, 128, 56, 3, 2, 1, 1, True
     oH = (H + 2 * p - k) // s + 1
@@ -203,49 +207,57 @@ def wl_bn(nsets):
                 desc=f"SpatialBatchNormalization train fwd+bwd fp32 N={N} C={Cc} {H}x{H} affine eps=1e-5 momentum=0.1")
 
 
-def wl_pool(nsets):
+def wl_pool(nsets, odd=False):
     from cunn_amd import CudaLongTensor as LT, CudaTensor as CT, THNN
     from oracle import oracle as O
-    N, Cc, H = 64, 64, 112
-    rng = np.random.default_rng(3)
+    # odd: 71x71 planes (Inception-style 3x3 stride-2 max pooling without padding, 3x3 stride-1 average pooling)
+    N, Cc, H = (32, 192, 71) if odd else (64, 64, 112)
+    mk, ms, mp = (3, 2, 0) if odd else (3, 2, 1)
+    ak, as_, ap_ = (3, 1, 1) if odd else (2, 2, 0)
+    oM, oA = (H + 2 * mp - mk) // ms + 1, (H + 2 * ap_ - ak) // as_ + 1
+    rng = np.random.default_rng(7 if odd else 3)
     x = (np.round(rng.uniform(-1, 1, (N, Cc, H, H)) * 64) / 64).astype(np.float32)
-    gy = rng.standard_normal((N, Cc, 56, 56)).astype(np.float32)
+    gy = rng.standard_normal((N, Cc, oM, oM)).astype(np.float32)
+    gya = gy if oA == oM else rng.standard_normal((N, Cc, oA, oA)).astype(np.float32)
     sets = []
     for _ in range(nsets):
-        sets.append(dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), idx=LT(), gx=CT(), ya=CT(), gxa=CT()))
+        sets.append(dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), gya=CT.from_numpy(gya), y=CT(), idx=LT(), gx=CT(), ya=CT(),
+                         gxa=CT()))
+    M, A = (mk, mk, ms, ms, mp, mp, False), (ak, ak, as_, as_, ap_, ap_, False, True)
 
     def calls(i):
         t = sets[i]
-        return [("maxpool_updateOutput", lambda: THNN.SpatialMaxPooling_updateOutput(t["x"], t["y"], t["idx"], 3, 3, 2, 2, 1, 1, False)),
-                ("maxpool_updateGradInput", lambda: THNN.SpatialMaxPooling_updateGradInput(t["x"], t["gy"], t["gx"], t["idx"], 3, 3, 2, 2, 1, 1, False)),
-                ("avgpool_updateOutput", lambda: THNN.SpatialAveragePooling_updateOutput(t["x"], t["ya"], 2, 2, 2, 2, 0, 0, False, True)),
-                ("avgpool_updateGradInput", lambda: THNN.SpatialAveragePooling_updateGradInput(t["x"], t["gy"], t["gxa"], 2, 2, 2, 2, 0, 0, False, True))]
+        return [("maxpool_updateOutput", lambda: THNN.SpatialMaxPooling_updateOutput(t["x"], t["y"], t["idx"], *M)),
+                ("maxpool_updateGradInput", lambda: THNN.SpatialMaxPooling_updateGradInput(t["x"], t["gy"], t["gx"], t["idx"], *M)),
+                ("avgpool_updateOutput", lambda: THNN.SpatialAveragePooling_updateOutput(t["x"], t["ya"], *A)),
+                ("avgpool_updateGradInput", lambda: THNN.SpatialAveragePooling_updateGradInput(t["x"], t["gya"], t["gxa"], *A))]
 
-    xb, yb = x.nbytes, gy.nbytes
+    xb, yb, yab = x.nbytes, gy.nbytes, gya.nbytes
     work = {"maxpool_updateOutput": (xb + yb + 2 * yb, "bytes"), "maxpool_updateGradInput": (yb + 2 * yb + xb, "bytes"),
-            "avgpool_updateOutput": (xb + yb, "bytes"), "avgpool_updateGradInput": (yb + xb, "bytes")}
+            "avgpool_updateOutput": (xb + yab, "bytes"), "avgpool_updateGradInput": (yab + xb, "bytes")}
 
     def cpu(reps):
         t0 = time.perf_counter()
         for _ in range(reps):
-            _, idx = O.maxpool_updateOutput(x, 3, 3, 2, 2, 1, 1, False)
-            O.maxpool_updateGradInput(x.shape, gy, idx, 3, 3, 2, 2, 1, 1, False)
-            O.avgpool_updateOutput(x, 2, 2, 2, 2, 0, 0, False, True)
-            O.avgpool_updateGradInput(x.shape, gy, 2, 2, 2, 2, 0, 0, False, True)
-        return time.perf_counter() - t0, reps * N, f"{reps} full passes of cfg4 ({N} images each)"
+            _, idx = O.maxpool_updateOutput(x, *M)
+            O.maxpool_updateGradInput(x.shape, gy, idx, *M)
+            O.avgpool_updateOutput(x, *A)
+            O.avgpool_updateGradInput(x.shape, gya, *A)
+        return time.perf_counter() - t0, reps * N, f"{reps} full passes of {'pool71' if odd else 'cfg4'} ({N} images each)"
 
     def verify():
         t = sets[0]
         for _, fn in calls(0):
             fn()
-        ry, ridx = O.maxpool_updateOutput(x, 3, 3, 2, 2, 1, 1, False)
+        ry, ridx = O.maxpool_updateOutput(x, *M)
         assert np.array_equal(t["y"].numpy(), ry) and np.array_equal(t["idx"].numpy(), ridx)
-        np.testing.assert_allclose(t["gx"].numpy(), O.maxpool_updateGradInput(x.shape, gy, ridx, 3, 3, 2, 2, 1, 1, False), rtol=1e-5, atol=1e-4)
-        np.testing.assert_allclose(t["ya"].numpy(), O.avgpool_updateOutput(x, 2, 2, 2, 2, 0, 0, False, True), rtol=1e-5, atol=1e-4)
-        np.testing.assert_allclose(t["gxa"].numpy(), O.avgpool_updateGradInput(x.shape, gy, 2, 2, 2, 2, 0, 0, False, True), rtol=1e-5, atol=1e-4)
+        np.testing.assert_allclose(t["gx"].numpy(), O.maxpool_updateGradInput(x.shape, gy, ridx, *M), rtol=1e-5, atol=1e-4)
+        np.testing.assert_allclose(t["ya"].numpy(), O.avgpool_updateOutput(x, *A), rtol=1e-5, atol=1e-4)
+        np.testing.assert_allclose(t["gxa"].numpy(), O.avgpool_updateGradInput(x.shape, gya, *A), rtol=1e-5, atol=1e-4)
 
     return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="hbm",
-                desc=f"SpatialMaxPooling 3x3 s2 p1 (+indices) and SpatialAveragePooling 2x2 s2, fwd+bwd fp32 N={N} C={Cc} 112x112->56x56")
+                desc=f"SpatialMaxPooling {mk}x{mk} s{ms} p{mp} (+indices) and SpatialAveragePooling {ak}x{ak} s{as_} p{ap_}, fwd+bwd fp32 "
+                     f"N={N} C={Cc} {H}x{H}->{oM}x{oM} / {oA}x{oA}")
 
 
 def wl_conv(nsets):
@@ -445,6 +457,7 @@ def wl_copy(nsets):
 
 
 WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda n: wl_dw("cfg2", n), "cfg3": wl_bn, "cfg4": wl_pool,
+             "dw147": lambda n: wl_dw("dw147", n), "dw14": lambda n: wl_dw("dw14", n), "pool71": lambda n: wl_pool(n, odd=True),
              "cfg5": wl_conv, "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu}
 
 

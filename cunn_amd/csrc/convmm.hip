@@ -2020,9 +2020,15 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   // measured better than the four that fit (less partial traffic for the same matrix-pipe load), two when
   // gradWeight is one or two tiles and the partials are most of the traffic. The small tiles stream: as many
   // workgroups as fit, to have enough loads in flight.
-  const int perCu = mT * nT <= 2 ? 2 : tiny ? 4 : 3;
-  const int slots = std::min(residentSlots(kern), residentSlots(nullptr) * perCu);
-  int splits = std::max(1, std::min(totalKt, slots / (mT * nT)));
+  // A split should keep at least about 20 k-tiles (short reductions at 14x14 and 7x7: with 8 k-tiles per split the
+  // partial copies and the pipeline fill cost more than the third workgroup per CU gains).
+  int perCu = mT * nT <= 2 ? 2 : tiny ? 4 : 3;
+  auto splitsAt = [&](int wgPerCu) {
+    const int slots = std::min(residentSlots(kern), residentSlots(nullptr) * wgPerCu);
+    return std::max(1, std::min(totalKt, slots / (mT * nT)));
+  };
+  while (perCu > 1 && totalKt / splitsAt(perCu) < 20) --perCu;
+  int splits = splitsAt(perCu);
   const int perSplit = launch::ceilDiv(totalKt, splits);
   splits = launch::ceilDiv(totalKt, perSplit);
   const int wgSplits = splits;       // splits of the positions over workgroups

@@ -856,7 +856,7 @@ bool smallPlan(const DwGeom &g, SmallPass pass, SmallGeom *out, int *rw, size_t 
   const int base = g.W + 2 * PAD;
   const int room = (int)((launch::kLdsMax / sizeof(float) - secondFloats - kSlack - 4) / ((size_t)sg.P * sg.LH));  // widest pitch that fits
   const launch::ItemChoice ch = launch::pickItem(pass, sg.oW, sg.rowsPerBand, sg.lp, sg.lpShift, sg.LH, CS, base,
-                                                 std::max(room, sg.LW), pass == kSmallAccGrad);
+                                                 std::max(room, sg.LW), pass == kSmallAccGrad, KS);
   *rw = ch.rw;
   sg.LW = ch.LW;
   sg.xsFloats = roundUp(sg.P * sg.LH * sg.LW + kSlack, 4);

@@ -59,24 +59,24 @@ bool pickBand(int produced, long planes, BytesFn bytes, int *tileRows, int *tile
 // Work items of the kernels that convolve or pool staged planes from LDS: an item produces `rw` consecutive
 // outputs of a row (7 or 4), `lp` lanes share a plane of LH rows, the window rows of output row r start at
 // staged row r * CS. Chooses rw and the LDS row pitch (base .. base + 8, at most maxPitch): the pair with
-// the fewest LDS read cycles = lane-steps (rounds over the lanes that share a plane x (outputs + the
-// window's extra columns)) x the most lanes of the first wave that read the same of the 64 banks at one
+// the fewest LDS read cycles = lane-steps (rounds over the lanes that share a plane x the columns of an
+// item's window, (rw - 1) * CS + KS) x the most lanes of the first wave that read the same of the 64 banks at one
 // window column. splitRagged: the items that end past the row run in a pass of their own. The last choice
 // is kept per slot (0..7) and thread: the search costs a few microseconds.
 struct ItemChoice {
   int rw, LW;
 };
 inline ItemChoice pickItem(int slot, int oW, int rows, int lp, int lpShift, int LH, int CS, int base, int maxPitch,
-                           bool splitRagged) {
+                           bool splitRagged, int KS = 3) {
   struct Key {
-    int oW, rows, lp, LH, CS, base, maxPitch, split, rw, LW;
+    int oW, rows, lp, LH, CS, base, maxPitch, split, KS, rw, LW;
   };
   static thread_local Key last[8] = {};
   Key &ch = last[slot & 7];
   if (ch.rw != 0 && ch.oW == oW && ch.rows == rows && ch.lp == lp && ch.LH == LH && ch.CS == CS && ch.base == base &&
-      ch.maxPitch == maxPitch && ch.split == (int)splitRagged)
+      ch.maxPitch == maxPitch && ch.split == (int)splitRagged && ch.KS == KS)
     return ItemChoice{ch.rw, ch.LW};
-  ch = Key{oW, rows, lp, LH, CS, base, maxPitch, (int)splitRagged, 0, 0};
+  ch = Key{oW, rows, lp, LH, CS, base, maxPitch, (int)splitRagged, KS, 0, 0};
   long best = 0;
   for (int LW = base; LW <= std::min(base + 8, std::max(maxPitch, base)); ++LW)
     for (int r : {7, 4}) {
@@ -90,7 +90,7 @@ inline ItemChoice pickItem(int slot, int oW, int rows, int lp, int lpShift, int 
         const int row = it / nseg, c0 = (it - row * nseg) * r;
         worst = std::max(worst, (int)++lanes[(pl * LH * LW + row * CS * LW + c0 * CS) & 63]);
       }
-      const long cost = (long)(ceilDiv(items, lp) + (split ? ceilDiv(rows, lp) : 0)) * (r + 2) * worst;
+      const long cost = (long)(ceilDiv(items, lp) + (split ? ceilDiv(rows, lp) : 0)) * ((r - 1) * CS + KS) * worst;  // window columns
       if (ch.rw == 0 || cost < best) best = cost, ch.rw = r, ch.LW = LW;
     }
   return ItemChoice{ch.rw, ch.LW};

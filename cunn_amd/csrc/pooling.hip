@@ -869,7 +869,7 @@ bool poolRunPlanFor(const PoolGeom &g, long planes, bool backward, bool max, Poo
   if (!backward) {
     const int room = (int)((launch::kLdsMax / sizeof(float) - nIdx * second - kSlack - 4) / ((size_t)sg.P * sg.LH));
     const launch::ItemChoice ch = launch::pickItem(3 + (max ? 1 : 0), sg.oW, sg.rowsPerBand, sg.lp, sg.lpShift, sg.LH, ST,
-                                                   LW0 & ~1, std::max(room, LW0), false);
+                                                   LW0 & ~1, std::max(room, LW0), false, KS);
     rw = ch.rw, sg.LW = std::max(ch.LW, std::max(PAD + g.W, (g.oW - 1) * ST + KS));
   }
   sg.xsFloats = roundUp(sg.P * sg.LH * sg.LW + kSlack, 4);

@@ -886,14 +886,15 @@ int runSwitch() {
   return e ? atoi(e) : -1;
 }
 // Where both families apply (widths that are multiples of 4), measured on 8x8 ... 224x224 planes: the run
-// kernels' max forward is never slower (16x16: 44 -> 12 us, 112x112: 64 -> 62 us); the average forward wins
-// up to 28x28 and the backward passes up to about 36x36 (a plane per workgroup leaves the strip kernels'
-// lanes idle there), beyond that the strip kernels' backward is 10-20 % faster.
+// kernels' max forward wins up to 112x112 (16x16: 44 -> 12 us, 112x112: 64 -> 62 us; at 224x224 the strip
+// kernels are 5-15 % faster); the average forward wins up to 28x28 and the backward passes up to about 36x36
+// (a plane per workgroup leaves the strip kernels' lanes idle there), beyond that the strip kernels'
+// backward is 10-20 % faster.
 bool runsFirst(const PoolGeom &g, bool backward, bool max) {
   if (runSwitch() >= 0) return runSwitch() == 1;
   const long plane = std::max((long)g.H * g.W, (long)g.oH * g.oW);
   if (backward) return plane <= 2048;
-  return max || plane <= 1024;
+  return plane <= (max ? 112 * 112 : 1024);
 }
 
 bool poolRunPlan(const PoolGeom &g, long planes, bool backward, bool max, PoolRunPlan *out) {

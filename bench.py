@@ -461,58 +461,75 @@ WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda
              "cfg5": wl_conv, "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu}
 
 
+PREROLL_SAMPLES = 12   # event samples per entry point collected before the timed region, whatever --warmup is
+
+
 def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds):
     wl = WORKLOADS[name](nsets)
     wl["verify"]()                       # parity against the oracle in this very run
     names = [n for n, _ in wl["calls"](0)]
+    cursor = [0]                         # buffer sets keep rotating across the phases below
 
-    def timed(nsteps, bracket):
+    def run(nsteps, bracket):
         """nsteps steps back to back; HIP events around the entry points named in `bracket`."""
         ev = {n: [(hip.event(), hip.event()) for _ in range(nsteps)] for n in bracket}
         hip.sync()
         t0 = time.perf_counter()
         for i in range(nsteps):
-            for n, fn in wl["calls"](i % nsets):
+            for n, fn in wl["calls"](cursor[0] % nsets):
                 if n in ev:
                     hip.record(ev[n][i][0], stream)
                     fn()
                     hip.record(ev[n][i][1], stream)
                 else:
                     fn()
+            cursor[0] += 1
         hip.sync()
         wall = time.perf_counter() - t0
         return wall, {n: [hip.elapsed_ms(a, b) for a, b in ev[n]] for n in bracket}
 
-    # warm-up: a few plain steps, then the rest instrumented one entry point at a time (events around
-    # neighbouring launches would add their own few microseconds to each other's bracket) - that finds
-    # the dominant kernel and times the others
-    plain = max(1, warmup // 4)
-    timed(plain, [])
+    # pre-roll (untimed, reported as preroll_steps): one plain step on every buffer set, so that every
+    # output / gradInput / scratch storage has its final size before anything is measured (a first call at
+    # a new size allocates), then PREROLL_SAMPLES steps per entry point with HIP events around that entry
+    # point alone (events around neighbouring launches would add their own few microseconds to each
+    # other's bracket) - that finds the dominant kernel and times the others
+    run(nsets, [])
+    preroll = nsets
     per_kernel = {}
     for n in names:
-        per_kernel.update(timed(max((warmup - plain) // len(names), 1), [n])[1])
-    dominant = max(names, key=lambda n: float(np.mean(per_kernel[n])))
+        per_kernel.update(run(PREROLL_SAMPLES, [n])[1])
+        preroll += PREROLL_SAMPLES
+    dominant = max(names, key=lambda n: float(np.median(per_kernel[n])))
+    run(warmup, [])                      # the W warm-up steps asked for
     # the timed region: exactly `steps` steps; only the dominant kernel is bracketed by events,
     # so the measurement perturbs the step as little as possible
-    wall, dom = timed(steps, [dominant])
+    wall, dom = run(steps, [dominant])
     per_kernel[dominant] = dom[dominant]
     kern = {}
     for n in names:
-        avg = float(np.mean(per_kernel[n]))
+        med, avg = float(np.median(per_kernel[n])), float(np.mean(per_kernel[n]))
         amount, kind = wl["work"][n]
         if kind == "bytes":
-            ach, peak, unit = amount / (avg * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
+            scale, peak, unit = 1e9, HBM_PEAK_GBS, "GB/s"
         else:
-            ach, peak, unit = amount / (avg * 1e-3) / 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
-        kern[n] = dict(avg_ms=avg, min_ms=float(np.min(per_kernel[n])), samples=len(per_kernel[n]), achieved=ach,
-                       peak=peak, unit=unit, frac=ach / peak, algorithmic=amount, kind=kind)
+            scale, peak, unit = 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
+        kern[n] = dict(avg_ms=avg, median_ms=med, min_ms=float(np.min(per_kernel[n])), samples=len(per_kernel[n]),
+                       achieved=amount / (avg * 1e-3) / scale, achieved_median=amount / (med * 1e-3) / scale,
+                       peak=peak, unit=unit, frac=amount / (avg * 1e-3) / scale / peak,
+                       frac_median=amount / (med * 1e-3) / scale / peak, algorithmic=amount, kind=kind)
     ms_per_step = wall * 1e3 / steps
     d = kern[dominant]
+    step_work = sum(wl["work"][n][0] for n in names)
+    step_scale, step_peak = (1e9, HBM_PEAK_GBS) if wl["bound"] == "hbm" else (1e12, FP32_MFMA_PEAK_TFLOPS)
     roofline = dict(bound=wl["bound"], kernel=dominant, achieved=round(d["achieved"], 3), peak=d["peak"], unit=d["unit"],
                     frac=round(d["frac"], 4), traffic=MEASURED_TRAFFIC_BYTES.get((name, dominant)),
-                    algorithmic_per_launch=d["algorithmic"], avg_launch_ms=round(d["avg_ms"], 5))
+                    algorithmic_per_launch=d["algorithmic"], avg_launch_ms=round(d["avg_ms"], 5),
+                    median_launch_ms=round(d["median_ms"], 5), min_launch_ms=round(d["min_ms"], 5),
+                    frac_median=round(d["frac_median"], 4), samples=d["samples"],
+                    step_frac=round(step_work / (ms_per_step * 1e-3) / step_scale / step_peak, 4),
+                    algorithmic_per_step=step_work)
     res = dict(workload=wl["desc"], images_per_s=wl["images"] / (ms_per_step * 1e-3), ms_per_step=ms_per_step,
-               device_ms_per_step=float(sum(kern[n]["avg_ms"] for n in names)), roofline=roofline,
+               device_ms_per_step=float(sum(kern[n]["median_ms"] for n in names)), roofline=roofline, preroll_steps=preroll,
                kernels={n: {k: (round(v, 5) if isinstance(v, float) else v) for k, v in kern[n].items()} for n in names})
     if cpu_seconds > 0 and name != "copy":
         from oracle import oracle as O
@@ -554,6 +571,7 @@ def main():
         "config": {"workload": f"{args.workload}: {main_res['workload']}", "buffer_sets": args.sets,
                    "entry": "C ABI libTHCUNN.so (THNN_Cuda*) via ctypes"},
         "device_ms_per_step": round(main_res["device_ms_per_step"], 5),
+        "preroll_steps": main_res["preroll_steps"],
         "roofline": main_res["roofline"],
         "cpu_baseline": main_res.get("cpu_baseline"),
         "kernels": main_res["kernels"],
@@ -563,7 +581,7 @@ def main():
         for name in sorted(WORKLOADS):
             if name == args.workload or name == "copy":
                 continue
-            r = run_workload(name, max(20, args.steps // 4), max(5, args.warmup // 2), hip, stream,
+            r = run_workload(name, max(20, args.steps // 4), max(4, args.warmup // 2), hip, stream,
                              args.sets, min(args.cpu_seconds, 8.0))
             others[name] = dict(workload=r["workload"], images_per_s=round(r["images_per_s"], 1),
                                 ms_per_step=round(r["ms_per_step"], 5), roofline=r["roofline"],

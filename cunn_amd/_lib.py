@@ -26,6 +26,8 @@ ENTRY_POINTS = [
     "SpatialFullConvolution_updateOutput", "SpatialFullConvolution_updateGradInput",
     "SpatialFullConvolution_accGradParameters",
     "Threshold_updateOutput", "Threshold_updateGradInput",
+    # no counterpart in the reference: for callers that cannot allocate device memory
+    "SpatialDepthWiseConvolution_accGradParameters_noAlloc",
 ]
 
 _T = C.c_void_p  # THCudaTensor* / THCudaLongTensor* / THCState*
@@ -57,6 +59,7 @@ SIGNATURES = {
     "SpatialFullConvolution_accGradParameters": [_T] * 7 + [_i] * 8 + [_f],
     "Threshold_updateOutput": [_T] * 3 + [_f, _f, _b],
     "Threshold_updateGradInput": [_T] * 4 + [_f, _f, _b],
+    "SpatialDepthWiseConvolution_accGradParameters_noAlloc": [_T] * 5 + [_i] * 6 + [_f],
 }
 
 _LP = C.POINTER(C.c_long)

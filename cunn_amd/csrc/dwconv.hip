@@ -16,6 +16,8 @@
 #include "strip.h"
 #include "thc_internal.h"
 
+#include <mutex>
+
 using namespace thc;
 
 namespace {
@@ -889,6 +891,58 @@ inline unsigned smallGrid(const SmallGeom &sg) {
     if (g.kH == 5 && rw == 7) dwSmallAccGrad<5, ST, 7><<<grid, dev::kBlock, lds, s>>>(__VA_ARGS__);               \
   } while (0)
 
+// ---- fixed scratch of the entry point that allocates nothing ----------------------------------
+// accGradParameters needs device memory beyond its inputs and outputs: the per-workgroup partial sums that
+// its second kernel folds. The regular entry point takes it from the caller's `columns` tensor (growing it)
+// or from a stream-ordered temporary; the no-allocation variant takes it from this array, which each GPU the
+// library runs on holds (4 MiB) until the process ends. In host code the array's name is only a handle for
+// hipGetSymbolAddress, never a device address: the address is looked up once per device and kept.
+constexpr long kNoAllocScratchFloats = 1L << 20;
+static __device__ __align__(256) float scratch[kNoAllocScratchFloats];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratchMutex;
+float *g_scratchPtr[kMaxDevices];  // per device: that GPU's copy of `scratch`
+
+// Address of the current device's copy of the array; `device` must be the current device.
+float *noAllocScratch(int device) {
+  if (device < 0 || device >= kMaxDevices) error("device ordinal %d out of range", device);
+  std::lock_guard<std::mutex> lock(g_scratchMutex);
+  if (!g_scratchPtr[device]) {
+    void *p = nullptr;
+    THC_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    g_scratchPtr[device] = static_cast<float *>(p);
+  }
+  return g_scratchPtr[device];
+}
+
+// Where accGradParameters puts its partial sums.
+struct DwScratch {
+  THCudaTensor *columns = nullptr;  // the caller's buffer tensor (resized), or NULL: a stream-ordered temporary
+  float *fixed = nullptr;           // no-allocation variant: the device's fixed array
+  bool noAlloc = false;
+  Temp tmp;
+
+  // `rows` x `nslots` floats of scratch
+  float *get(THCState *state, long rows, long nslots) {
+    if (noAlloc) {
+      if (rows * nslots > kNoAllocScratchFloats)
+        error("SpatialDepthWiseConvolution_accGradParameters_noAlloc: this shape needs %ld floats of scratch "
+              "(%ld partial sums for each of %ld channel taps), the fixed scratch holds %ld; use "
+              "SpatialDepthWiseConvolution_accGradParameters",
+              rows * nslots, nslots, rows, kNoAllocScratchFloats);
+      return fixed;
+    }
+    if (columns) {
+      resize(state, columns, {rows, nslots});
+      if (!isContiguous(erase(columns))) error("columns tensor has to be contiguous");
+      return data(columns);
+    }
+    tmp = Temp(state->stream, (size_t)(rows * nslots) * sizeof(float));
+    return (float *)tmp.get();
+  }
+};
+
 }  // namespace
 
 extern "C" {
@@ -1047,18 +1101,29 @@ void THNN_CudaSpatialDepthWiseConvolution_updateGradInput(THCState *state, THCud
   THNN_LEAVE
 }
 
-void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THCudaTensor *input,
-                                                            THCudaTensor *gradOutput, THCudaTensor *gradWeight,
-                                                            THCudaTensor *gradBias, THCudaTensor *columns,
-                                                            THCudaTensor *ones, int kW, int kH, int dW, int dH,
-                                                            int padW, int padH, float scale) {
-  THNN_ENTER
-  (void)ones;
+}  // extern "C"
+
+namespace {
+
+// lib/THCUNN/generic/SpatialDepthWiseConvolution.cu:418-650; `sc` says where the partial sums go
+void dwAccGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradWeight,
+                         THCudaTensor *gradBias, DwScratch &sc, int kW, int kH, int dW, int dH, int padW, int padH,
+                         float scale) {
   THC_ARG_CHECK(gradOutput != nullptr, 3, "gradOutput tensor expected");
   THC_ARG_CHECK(gradWeight != nullptr, 4, "gradWeight tensor expected");
+  if (sc.noAlloc) {
+    // everything that would allocate in the regular entry point is refused up front
+    THC_ARG_CHECK(input != nullptr, 2, "input tensor expected");
+    if (gradWeight->nDimension != 4)
+      error("SpatialDepthWiseConvolution_accGradParameters_noAlloc: 4D gradWeight tensor expected, but got: %s",
+            sizeDesc(erase(gradWeight)).c_str());
+    if (!isContiguous(erase(input)) || !isContiguous(erase(gradOutput)))
+      error("SpatialDepthWiseConvolution_accGradParameters_noAlloc: input and gradOutput have to be contiguous "
+            "(packing them would allocate)");
+  }
   DwCall call = dwSetup(state, input, gradOutput, gradWeight, gradBias, kW, kH, dW, dH, padW, padH);
   DwGeom &g = call.g;
-  Contiguous in(state, input);
+  Contiguous in(state, input);  // contiguous tensors are used in place
   Contiguous go(state, gradOutput);
   hipStream_t s = state->stream;
   const long planes = (long)g.N * g.C;
@@ -1072,18 +1137,9 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
     if (aligned16(in.ptr()) && aligned16(go.ptr()) && smallPlan(g, kSmallAccGrad, &sg, &rw, &lds)) {
       const int T = g.kH * g.kW + 1;
       // one partial per (channel, tap, image); scratch as in the general case below
-      Temp tmp;
-      float *partial;
       const long nslots = (long)g.N * sg.bands;
       if (nslots >= 0x7fffffffL) error("SpatialDepthWiseConvolution: batch too large");
-      if (columns) {
-        resize(state, columns, {(long)g.C * T, nslots});
-        if (!isContiguous(erase(columns))) error("columns tensor has to be contiguous");
-        partial = data(columns);
-      } else {
-        tmp = Temp(s, (size_t)g.C * T * nslots * sizeof(float));
-        partial = (float *)tmp.get();
-      }
+      float *partial = sc.get(state, (long)g.C * T, nslots);
       const dim3 grid(smallGrid(sg));
       if (g.dH == 1)
         DW_SMALL_ACC(1, in.ptr(), go.ptr(), partial, sg, g.N);
@@ -1122,17 +1178,7 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
     // per-workgroup partials: the caller's `columns` buffer is the scratch the ABI
     // provides for this call (the reference resizes it as well, :528); fall back to a
     // stream-ordered temporary when none is passed
-    long nPartial = (long)g.C * g.M * T * g.nslots;
-    Temp tmp;
-    float *partial;
-    if (columns) {
-      resize(state, columns, {(long)g.C * g.M * T, g.nslots});
-      if (!isContiguous(erase(columns))) error("columns tensor has to be contiguous");
-      partial = data(columns);
-    } else {
-      tmp = Temp(s, (size_t)nPartial * sizeof(float));
-      partial = (float *)tmp.get();
-    }
+    float *partial = sc.get(state, (long)g.C * g.M * T, g.nslots);
     // a band of gradOutput rows starts at ((plane*M+j)*oH + oh0) * oW
     bool vecg = aligned16(go.ptr()) && (g.oW % 4 == 0 || (g.tilesPerPlane == 1 && ((long)g.oH * g.oW) % 4 == 0));
     if (useStrip) {
@@ -1159,6 +1205,46 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THC
                                                           strides4(gradWeight), gbPtr, strides2(gradBias), g, scale);
   }
   THC_HIP_CHECK(hipGetLastError());
+}
+
+}  // namespace
+
+namespace thc {
+void dwNoAllocInit(int device) { (void)noAllocScratch(device); }
+}  // namespace thc
+
+extern "C" {
+
+void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(THCState *state, THCudaTensor *input,
+                                                            THCudaTensor *gradOutput, THCudaTensor *gradWeight,
+                                                            THCudaTensor *gradBias, THCudaTensor *columns,
+                                                            THCudaTensor *ones, int kW, int kH, int dW, int dH,
+                                                            int padW, int padH, float scale) {
+  THNN_ENTER
+  (void)ones;
+  DwScratch sc;
+  sc.columns = columns;
+  dwAccGradParameters(state, input, gradOutput, gradWeight, gradBias, sc, kW, kH, dW, dH, padW, padH, scale);
+  THNN_LEAVE
+}
+
+// No counterpart in the reference: the same pass for callers that cannot allocate device memory (HIP graph
+// capture, serving loops). Same kernels; the partial sums go to the device's fixed scratch array.
+void THNN_CudaSpatialDepthWiseConvolution_accGradParameters_noAlloc(THCState *state, THCudaTensor *input,
+                                                                    THCudaTensor *gradOutput,
+                                                                    THCudaTensor *gradWeight, THCudaTensor *gradBias,
+                                                                    int kW, int kH, int dW, int dH, int padW,
+                                                                    int padH, float scale) {
+  THNN_ENTER
+  int device = -1;
+  THC_HIP_CHECK(hipGetDevice(&device));
+  if (device != state->device)
+    error("SpatialDepthWiseConvolution_accGradParameters_noAlloc: the state was made on device %d but device %d "
+          "is current", state->device, device);
+  DwScratch sc;
+  sc.noAlloc = true;
+  sc.fixed = noAllocScratch(device);  // looked up when the state was made; a table read here
+  dwAccGradParameters(state, input, gradOutput, gradWeight, gradBias, sc, kW, kH, dW, dH, padW, padH, scale);
   THNN_LEAVE
 }
 

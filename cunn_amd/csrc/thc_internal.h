@@ -141,6 +141,11 @@ class Contiguous {
   Temp tmp_;
 };
 
+// Looks up, for the current device `device`, the address of the fixed scratch array behind
+// THNN_CudaSpatialDepthWiseConvolution_accGradParameters_noAlloc (dwconv.hip). Called when a state is
+// made, so that the entry point itself finds the address in a table.
+void dwNoAllocInit(int device);
+
 // THCUNN_check_dim_size (lib/THCUNN/common.h:69-75)
 void checkDimSize(const Tensor *t, const char *name, int dim, int dimSize, long size);
 

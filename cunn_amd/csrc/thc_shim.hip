@@ -332,6 +332,7 @@ THCState *THCState_alloc(void) {
   s = (THCState *)calloc(1, sizeof(THCState));
   THC_HIP_CHECK(hipGetDevice(&s->device));
   s->stream = nullptr;  // the device's default stream
+  dwNoAllocInit(s->device);
   THNN_LEAVE
   return s;
 }

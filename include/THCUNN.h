@@ -100,6 +100,20 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(
     THCudaTensor *columns, THCudaTensor *ones,
     int kW, int kH, int dW, int dH, int padW, int padH, float scale);
 
+/* No counterpart in the reference. SpatialDepthWiseConvolution_accGradParameters for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): same kernels and results, but the per-workgroup partial sums go to a fixed 4 MiB device array
+ * that the library holds on each GPU it runs on, and nothing is allocated, freed or resized. It therefore
+ * takes no `columns` / `ones`, and refuses (TH error, nothing launched) what the regular entry point would
+ * allocate for: non-contiguous input / gradOutput, a 2-D gradWeight, and shapes whose partial sums exceed
+ * 2^20 floats (C * M * (kH*kW + 1) * N * bands-per-plane). The state must have been made on the current
+ * device. All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two
+ * threads) race. */
+void THNN_CudaSpatialDepthWiseConvolution_accGradParameters_noAlloc(
+    THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradWeight,
+    THCudaTensor *gradBias,     /* [OPTIONAL] */
+    int kW, int kH, int dW, int dH, int padW, int padH, float scale);
+
 /* ---- SpatialDilatedMaxPooling / SpatialMaxPooling ------------------------ */
 
 /* replaces lib/THCUNN/generic/THCUNN.h:808-817, lib/THCUNN/generic/SpatialDilatedMaxPooling.cu:84-158 */

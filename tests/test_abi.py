@@ -20,7 +20,8 @@ def test_library_exports_every_declared_symbol():
     from cunn_amd import _lib
     lib = _lib.load()
     declared = _declared("THCUNN.h") + _declared("THCShim.h")
-    assert len([n for n in declared if n.startswith("THNN_Cuda")]) == 25  # 14 hot-path + 9 dilated / transposed convolution + 2 Threshold
+    # 14 hot-path + 9 dilated / transposed convolution + 2 Threshold + the no-allocation accGradParameters variant
+    assert len([n for n in declared if n.startswith("THNN_Cuda")]) == 26
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/ but not exported"
 

@@ -12,9 +12,10 @@ region; four buffer sets are rotated so that no step finds its inputs in the
 256 MB Infinity Cache from the step before.
 
 Prints ONE JSON line: images/s for the whole job, plus
-  roofline     - the dominant kernel's algorithmic bytes (or flops) per launch
+  roofline     - the dominant entry point's algorithmic bytes (or flops) per launch
                  over its average duration measured with HIP events on the
-                 stream the kernels run on, against MI355X's published peak;
+                 stream the kernels run on, against MI355X's published peak
+                 (median, min and the whole step's fraction beside it);
   cpu_baseline - the CPU oracle (a port of the reference algorithm) timed on
                  this host's cores on a bounded sample of the same workload;
   workloads    - with --all, the same figures for the other four configurations.
@@ -37,14 +38,31 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 FP32_MFMA_PEAK_TFLOPS = 157.3
 METRIC = "DW-conv fwd+bwd images/s + achieved HBM GB/s (% of peak), 1 MI355X"
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/dwconv_cfg2_hbm_traffic.txt gives the runs and the copy-kernel scale
-# factors); workloads without a counter run report null.
+# HBM bytes per entry-point call measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch; the
+# profiles/*_hbm_traffic.txt and profiles/cfg5_mfma_util.txt summaries give the runs and the copy-kernel scale
+# factors: FETCH_SIZE x 2, WRITE_SIZE x 1), summed over the kernels an entry point launches.
 _KIB = 1024
+
+
+def _traffic(*kernels):
+    return int(sum(f * 2.0 + w for f, w in kernels) * _KIB)
+
+
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg2", "dw_updateOutput"): int((50220.6 * 2.0 + 25154.3) * _KIB),
-    ("cfg2", "dw_updateGradInput"): int((12841.8 * 2.0 + 100368.2) * _KIB),
-    ("cfg2", "dw_accGradParameters"): int(((63014.8 + 197.5) * 2.0 + 320.8 + 16.0) * _KIB),
+    ("cfg1", "dw_updateOutput"): _traffic((26658.6, 50207.7)),
+    ("cfg2", "dw_updateOutput"): _traffic((50224.5, 25123.4)),
+    ("cfg2", "dw_updateGradInput"): _traffic((12836.5, 100354.0)),
+    ("cfg2", "dw_accGradParameters"): _traffic((63007.5, 512.0), (541.0, 12.0)),
+    ("cfg3", "bn_updateOutput"): _traffic((25722.0, 51041.0)),
+    ("cfg3", "bn_backward"): _traffic((56377.2, 51211.0)),
+    ("cfg4", "maxpool_updateOutput"): _traffic((103481.2, 150592.2)),
+    ("cfg4", "maxpool_updateGradInput"): _traffic((76828.4, 200725.9)),
+    ("cfg4", "avgpool_updateOutput"): _traffic((101707.4, 50176.0)),
+    ("cfg4", "avgpool_updateGradInput"): _traffic((30467.5, 200744.3)),
+    # bordered copy + GEMM + tail fold (+ flipped weights for gradInput; + partial fold for the weight gradient)
+    ("cfg5", "convmm_updateOutput"): _traffic((25983.0, 57606.1), (109420.3, 68419.4), (8237.0, 1024.0)),
+    ("cfg5", "convmm_updateGradInput"): _traffic((25983.0, 57606.1), (109420.3, 68419.4), (8237.0, 1024.0), (5180.1, 2304.0)),
+    ("cfg5", "convmm_accGradParameters"): _traffic((25983.0, 57606.1), (70844.7, 48405.0), (25371.6, 2305.0)),
 }
 
 

@@ -249,9 +249,13 @@ dwGradInputDirect(const float *__restrict__ gradOut, const float *__restrict__ w
 }
 
 // -------------------------------------------------------- accGradParameters --
+// floats between the partial runs of neighbouring (slot, c, j): the T sums rounded up to whole 64-byte groups
+__host__ __device__ constexpr int partialPitch(int T) { return (T + 15) & ~15; }
+
 // Stage 1: per workgroup, partial sums over its band of one (n,c) plane of
 //   gw[tap] = sum gy[oh,ow] * x[oh*d-p+kh, ow*d-p+kw]   and   gb = sum gy
-// written to partial[((c*M+j) * T + tap) * nslots + slot], T = KS*KS + 1.
+// written to partial[(slot * C*M + c*M+j) * TP + tap], T = KS*KS + 1, TP = T rounded up to 16 (partialPitch):
+// what a workgroup leaves is one aligned run of 64 or 128 bytes.
 template <int KS, int ST, bool VEC, bool VECG>
 __global__ void __launch_bounds__(dev::kBlock)
 dwAccGradStage1(const float *__restrict__ in, const float *__restrict__ gradOut, float *__restrict__ partial,
@@ -302,36 +306,50 @@ dwAccGradStage1(const float *__restrict__ in, const float *__restrict__ gradOut,
       float v = 0.f;
 #pragma unroll
       for (int w = 0; w < nWaves; ++w) v += red[w][threadIdx.x];
-      partial[(((long)c * g.M + j) * T + threadIdx.x) * g.nslots + slot] = v;
+      partial[((long)slot * (g.C * g.M) + c * g.M + j) * partialPitch(T) + threadIdx.x] = v;
     }
   }
 }
 
-// Stage 2: one wave per ((c,j), tap) folds the partials of all slots in a fixed order and
-// accumulates scale * sum into the caller's tensors; the old value is requested before the
-// partials so that the read-modify-write costs no second round trip.
-__global__ void __launch_bounds__(dev::kBlock)
+// Stage 2: one wave per (c, j) folds the partials of all slots in a fixed order and accumulates
+// scale * sum into the caller's tensors. A lane owns one tap (lane % TP) and every PH-th slot
+// (PH = 64 / TP slot phases, lane / TP): a load instruction of the wave reads PH whole runs as the
+// stage-1 workgroups wrote them; the phases are then added in a fixed association. The old value is
+// requested before the partials so that the read-modify-write costs no second round trip.
+template <int TP>
+__global__ void __launch_bounds__(dev::kWave)
 dwAccGradStage2(const float *__restrict__ partial, float *__restrict__ gradWeight, Strides4 gs,
-                float *__restrict__ gradBias, Strides2 bs, int M, int kW, int T, int nslots, float scale, int pairs) {
-  const int lane = threadIdx.x % dev::kWave;
-  const int pair = blockIdx.x * (dev::kBlock / dev::kWave) + threadIdx.x / dev::kWave;  // (c*M + j) * T + t
-  if (pair >= pairs) return;
-  const int cj = pair / T, t = pair - cj * T;
+                float *__restrict__ gradBias, Strides2 bs, int M, int kW, int T, int nslots, float scale, int CJ) {
+  constexpr int PH = dev::kWave / TP;
+  constexpr int U = 8;  // loads in flight per lane
+  const int cj = blockIdx.x;
+  const int t = threadIdx.x % TP, ph = threadIdx.x / TP;
   const int c = cj / M, j = cj - c * M;
-  float *dst;
-  if (t < T - 1) {
+  float *dst = nullptr;
+  if (ph == 0 && t < T - 1) {
     const int kh = t / kW, kw = t - kh * kW;
     dst = gradWeight + j * gs.s0 + c * gs.s1 + kh * gs.s2 + kw * gs.s3;
-  } else {
-    if (!gradBias) return;
+  } else if (ph == 0 && t == T - 1 && gradBias) {
     dst = gradBias + j * bs.s0 + c * bs.s1;
   }
-  const float old = *dst;
-  const float *p = partial + (long)pair * nslots;
+  const float old = dst ? *dst : 0.f;
+  const long step = (long)CJ * TP;  // floats between the runs of consecutive slots
+  const float *p = partial + (long)cj * TP + t;
   float v = 0.f;
-  for (int s = lane; s < nslots; s += dev::kWave) v += p[s];
-  v = dev::waveSum(v);
-  if (lane == 0) *dst = old + scale * v;
+  int sl = ph;
+  if (t < T) {
+    for (; sl + (U - 1) * PH < nslots; sl += U * PH) {
+      float a[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) a[u] = p[(long)(sl + u * PH) * step];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v += a[u];
+    }
+    for (; sl < nslots; sl += PH) v += p[(long)sl * step];
+  }
+  if (PH == 4) v += __shfl_down(v, 32);
+  v += __shfl_down(v, TP);
+  if (dst) *dst = old + scale * v;
 }
 
 // Any geometry: one workgroup per (c, j, tap) - tap == kH*kW is the bias - that
@@ -591,11 +609,13 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
       if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][t] = v;
     }
     __syncthreads();
-    if (threadIdx.x < T) {
+    if (threadIdx.x < partialPitch(T)) {  // the whole run, padding included, leaves in one store instruction
       float v = 0.f;
+      if (threadIdx.x < T) {
 #pragma unroll
-      for (int w = 0; w < nWaves * 4; ++w) v += red[w][threadIdx.x];
-      partial[(((long)c * nMul + j) * T + threadIdx.x) * g.nslots + slot] = v;
+        for (int w = 0; w < nWaves * 4; ++w) v += red[w][threadIdx.x];
+      }
+      partial[((long)slot * (g.C * nMul) + c * nMul + j) * partialPitch(T) + threadIdx.x] = v;
     }
   }
 }
@@ -731,6 +751,14 @@ void launchAcc1(hipStream_t s, size_t lds, bool vec, bool vecg, const float *in,
     dwAccGradStage1<KS, ST, false, true><<<grid, block, lds, s>>>(in, go, partial, g);
   else
     dwAccGradStage1<KS, ST, false, false><<<grid, block, lds, s>>>(in, go, partial, g);
+}
+
+void launchStage2(hipStream_t s, int TP, const float *partial, float *gw, Strides4 gs, float *gb, Strides2 bs, int M, int kW,
+                  int T, int nslots, float scale, int CJ) {
+  if (TP == 16)
+    dwAccGradStage2<16><<<CJ, dev::kWave, 0, s>>>(partial, gw, gs, gb, bs, M, kW, T, nslots, scale, CJ);
+  else
+    dwAccGradStage2<32><<<CJ, dev::kWave, 0, s>>>(partial, gw, gs, gb, bs, M, kW, T, nslots, scale, CJ);
 }
 
 // Environment switch used by the tests to exercise the shape-agnostic kernels on
@@ -928,15 +956,15 @@ struct DwScratch {
     if (noAlloc) {
       if (rows * nslots > kNoAllocScratchFloats)
         error("SpatialDepthWiseConvolution_accGradParameters_noAlloc: this shape needs %ld floats of scratch "
-              "(%ld partial sums for each of %ld channel taps), the fixed scratch holds %ld; use "
+              "(%ld workgroup slots of %ld floats), the fixed scratch holds %ld; use "
               "SpatialDepthWiseConvolution_accGradParameters",
-              rows * nslots, nslots, rows, kNoAllocScratchFloats);
+              rows * nslots, rows, nslots, kNoAllocScratchFloats);
       return fixed;
     }
     if (columns) {
       resize(state, columns, {rows, nslots});
       if (!isContiguous(erase(columns))) error("columns tensor has to be contiguous");
-      return data(columns);
+      if (launch::aligned16(data(columns))) return data(columns);  // the runs are written as 16-byte groups
     }
     tmp = Temp(state->stream, (size_t)(rows * nslots) * sizeof(float));
     return (float *)tmp.get();
@@ -1139,16 +1167,16 @@ void dwAccGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gra
       // one partial per (channel, tap, image); scratch as in the general case below
       const long nslots = (long)g.N * sg.bands;
       if (nslots >= 0x7fffffffL) error("SpatialDepthWiseConvolution: batch too large");
-      float *partial = sc.get(state, (long)g.C * T, nslots);
+      const int TP = partialPitch(T);
+      float *partial = sc.get(state, nslots, (long)g.C * TP);
       const dim3 grid(smallGrid(sg));
       if (g.dH == 1)
-        DW_SMALL_ACC(1, in.ptr(), go.ptr(), partial, sg, g.N);
+        DW_SMALL_ACC(1, in.ptr(), go.ptr(), partial, sg);
       else
-        DW_SMALL_ACC(2, in.ptr(), go.ptr(), partial, sg, g.N);
+        DW_SMALL_ACC(2, in.ptr(), go.ptr(), partial, sg);
       THC_HIP_CHECK(hipGetLastError());
-      const int pairs = g.C * T;
-      dwAccGradStage2<<<ceilDiv(pairs, dev::kBlock / dev::kWave), dev::kBlock, 0, s>>>(
-          partial, data(gradWeight), strides4(gradWeight), gbPtr, strides2(gradBias), 1, g.kW, T, (int)nslots, scale, pairs);
+      launchStage2(s, TP, partial, data(gradWeight), strides4(gradWeight), gbPtr, strides2(gradBias), 1, g.kW, T, (int)nslots,
+                   scale, g.C);
       THC_HIP_CHECK(hipGetLastError());
       return;
     }
@@ -1178,7 +1206,8 @@ void dwAccGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gra
     // per-workgroup partials: the caller's `columns` buffer is the scratch the ABI
     // provides for this call (the reference resizes it as well, :528); fall back to a
     // stream-ordered temporary when none is passed
-    float *partial = sc.get(state, (long)g.C * g.M * T, g.nslots);
+    const int TP = partialPitch(T);
+    float *partial = sc.get(state, g.nslots, (long)g.C * g.M * TP);
     // a band of gradOutput rows starts at ((plane*M+j)*oH + oh0) * oW
     bool vecg = aligned16(go.ptr()) && (g.oW % 4 == 0 || (g.tilesPerPlane == 1 && ((long)g.oH * g.oW) % 4 == 0));
     if (useStrip) {
@@ -1196,9 +1225,8 @@ void dwAccGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gra
       if (ks == 5 && st == 2) launchAcc1<5, 2>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);
     }
     THC_HIP_CHECK(hipGetLastError());
-    const int pairs = g.C * g.M * T;
-    dwAccGradStage2<<<ceilDiv(pairs, dev::kBlock / dev::kWave), dev::kBlock, 0, s>>>(
-        partial, data(gradWeight), strides4(gradWeight), gbPtr, strides2(gradBias), g.M, g.kW, T, g.nslots, scale, pairs);
+    launchStage2(s, TP, partial, data(gradWeight), strides4(gradWeight), gbPtr, strides2(gradBias), g.M, g.kW, T, g.nslots,
+                 scale, g.C * g.M);
   } else {
     int T = g.kH * g.kW + 1;
     dwAccGradDirect<<<g.C * g.M * T, dev::kBlock, 0, s>>>(in.ptr(), go.ptr(), data(gradWeight),

@@ -87,12 +87,12 @@ dwSmallConv(const float *__restrict__ src, const float *__restrict__ weight, Str
   smallStoreRun(dst, outFirst, os, b.np * b.nOut * g.oW);
 }
 
-// partial[(c * T + t) * nslots + n * bands + band] = sum over the band of plane (n, c) of gradOutput * input
-// window element t (t = kh * KS + kw; t = KS * KS: the bias, sum of gradOutput), T = KS * KS + 1, nslots = N * bands.
+// partial[((n * bands + band) * C + c) * TP + t] = sum over the band of plane (n, c) of gradOutput * input
+// window element t (t = kh * KS + kw; t = KS * KS: the bias, sum of gradOutput), T = KS * KS + 1, TP = T rounded
+// up to 16: the sums of one (plane, band) are one aligned run, written as 16-byte groups (padding zero).
 template <int KS, int ST, int RW>
 __global__ void __launch_bounds__(dev::kBlock)
-dwSmallAccGrad(const float *__restrict__ in, const float *__restrict__ gradOut, float *__restrict__ partial, SmallGeom g,
-               int N) {
+dwSmallAccGrad(const float *__restrict__ in, const float *__restrict__ gradOut, float *__restrict__ partial, SmallGeom g) {
   constexpr int PAD = KS / 2, NWIN = (RW - 1) * ST + KS, T = KS * KS + 1;
   extern __shared__ float smem[];
   __shared__ float red[dev::kBlock / dev::kWave][T];
@@ -177,8 +177,11 @@ dwSmallAccGrad(const float *__restrict__ in, const float *__restrict__ gradOut, 
   if (live && it0 == 0) {
     const int q = b.q0 + pl;
     const int n = dev::fastDiv(q, g.magicC), c = q - n * g.C;
-    const long nslots = (long)N * g.bands;
+    constexpr int TP = (T + 15) & ~15;
+    float4 *dst = reinterpret_cast<float4 *>(partial + (((long)n * g.bands + b.band) * g.C + c) * TP);
 #pragma unroll
-    for (int t = 0; t < T; ++t) partial[((long)c * T + t) * nslots + n * g.bands + b.band] = acc[t];
+    for (int t4 = 0; t4 < (T + 3) / 4; ++t4)
+      dst[t4] = make_float4(acc[t4 * 4], t4 * 4 + 1 < T ? acc[t4 * 4 + 1] : 0.f, t4 * 4 + 2 < T ? acc[t4 * 4 + 2] : 0.f,
+                            t4 * 4 + 3 < T ? acc[t4 * 4 + 3] : 0.f);
   }
 }

@@ -106,7 +106,7 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters(
  * that the library holds on each GPU it runs on, and nothing is allocated, freed or resized. It therefore
  * takes no `columns` / `ones`, and refuses (TH error, nothing launched) what the regular entry point would
  * allocate for: non-contiguous input / gradOutput, a 2-D gradWeight, and shapes whose partial sums exceed
- * 2^20 floats (C * M * (kH*kW + 1) * N * bands-per-plane). The state must have been made on the current
+ * 2^20 floats (C * M * P * N * bands-per-plane, P = kH*kW + 1 rounded up to 16). The state must have been made on the current
  * device. All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two
  * threads) race. */
 void THNN_CudaSpatialDepthWiseConvolution_accGradParameters_noAlloc(

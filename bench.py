@@ -215,10 +215,10 @@ def wl_bn(nsets):
             fn()
         rm, rv = np.zeros(Cc, np.float32), np.ones(Cc, np.float32)
         ry, sm, ss = O.bn_updateOutput(x, g, b, rm, rv, True, 0.1, 1e-5)
-        np.testing.assert_allclose(t["y"].numpy(), ry, rtol=1e-5, atol=2e-4)
+        np.testing.assert_allclose(t["y"].numpy(), ry, rtol=1e-5, atol=1e-4)
         np.testing.assert_allclose(t["ss"].numpy(), ss, rtol=1e-3)
         rgi, rgw, _ = O.bn_backward(x, gy, g, rm, rv, sm, ss, True, 1.0, 1e-5, np.zeros(Cc, np.float32), np.zeros(Cc, np.float32))
-        np.testing.assert_allclose(t["gx"].numpy(), rgi, rtol=1e-4, atol=2e-4)
+        np.testing.assert_allclose(t["gx"].numpy(), rgi, rtol=1e-5, atol=1e-4)
         np.testing.assert_allclose(t["gw"].numpy(), rgw, rtol=1e-3, atol=1e-2)
 
     return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="hbm",

@@ -99,7 +99,10 @@ def main():
         "bn_2d": bn_case(rng, (16, 7)),
         "pool_3s2p1": pool_case(rng, 2, 3, 24, 24, 3, 2, 1, False),
         "pool_2s2": pool_case(rng, 2, 3, 24, 24, 2, 2, 0, False),
-        "pool_3s2p1_ceil": pool_case(rng, 1, 2, 15, 18, 3, 2, 1, False),
+        "pool_3s2p1_ceil": pool_case(rng, 1, 2, 15, 18, 3, 2, 1, True),     # ceil mode adds a last, clipped window: 8x10 outputs
+        # ceil mode where the last window would start in the padding and is dropped again
+        # (lib/THCUNN/generic/SpatialDilatedMaxPooling.cu:56-64): 7 -> 4 and 9 -> 5 outputs instead of 5 and 6
+        "pool_2s2p1_ceil_drop": pool_case(rng, 2, 3, 7, 9, 2, 2, 1, True),
     }
     flat = {}
     for cname, d in cases.items():

@@ -74,14 +74,14 @@ def test_cfg3_batchnorm_train(T):
     THNN.BatchNormalization_backward(tx, tgy, gx, gw, gb, tg, rm, rv, sm, ss, True, 1.0, 1e-5)
     orm, orv = np.zeros(C, np.float32), np.ones(C, np.float32)
     ry, osm, oss = O.bn_updateOutput(x, g, b, orm, orv, True, 0.1, 1e-5)
-    np.testing.assert_allclose(y.numpy(), ry, rtol=1e-5, atol=2e-4)
+    np.testing.assert_allclose(y.numpy(), ry, rtol=1e-5, atol=1e-4)
     np.testing.assert_allclose(sm.numpy(), osm, rtol=1e-3, atol=1e-5)
     np.testing.assert_allclose(ss.numpy(), oss, rtol=1e-3)
     np.testing.assert_allclose(rm.numpy(), orm, rtol=1e-3, atol=1e-5)
     np.testing.assert_allclose(rv.numpy(), orv, rtol=1e-3)
     rgx, rgw, rgb = O.bn_backward(x, gy, g, orm, orv, osm, oss, True, 1.0, 1e-5, np.zeros(C, np.float32), np.zeros(C, np.float32))
     gxv = gx.numpy()
-    np.testing.assert_allclose(gxv, rgx, rtol=1e-4, atol=2e-4)
+    np.testing.assert_allclose(gxv, rgx, rtol=1e-5, atol=1e-4)
     np.testing.assert_allclose(gw.numpy(), rgw, rtol=1e-3, atol=5e-2)
     np.testing.assert_allclose(gb.numpy(), rgb, rtol=1e-3, atol=5e-2)
     # per channel: output mean = beta, output variance = gamma^2 var/(var+eps); gradInput sums to zero

@@ -517,7 +517,7 @@ def _bn_run(T, shape, affine, seed=40):
     rm, rv = rm0.copy(), rv0.copy()
     ry, sm, ss = O.bn_updateOutput(x, g, b, rm, rv, True, mom, eps)
     assert out.size() == tuple(shape)
-    close(out.numpy(), ry, 1e-5, 2e-4)
+    close(out.numpy(), ry)
     close(tsm.numpy(), sm, WG_RTOL, 1e-5)
     close(tss.numpy(), ss, WG_RTOL, 1e-6)
     close(trm.numpy(), rm, WG_RTOL, 1e-5)
@@ -526,7 +526,7 @@ def _bn_run(T, shape, affine, seed=40):
     oute = CT()
     THNN.BatchNormalization_updateOutput(tx, oute, tg, tb, trm, trv, tsm, tss, False, mom, eps)
     rye, _, _ = O.bn_updateOutput(x, g, b, rm.copy(), rv.copy(), False, mom, eps)
-    close(oute.numpy(), rye, 1e-5, 2e-4)
+    close(oute.numpy(), rye)
     # backward: fused call, then the split order (updateGradInput, accGradParameters) (test.lua:989-1003)
     gy = rng.standard_normal(shape).astype(np.float32)
     tgy = CT.from_numpy(gy)
@@ -537,7 +537,7 @@ def _bn_run(T, shape, affine, seed=40):
         tgw, tgb = CT.from_numpy(gw0), CT.from_numpy(gb0)
         THNN.BatchNormalization_backward(tx, tgy, gi, tgw, tgb, tg, trm, trv, tsm, tss, train, 0.5, eps)
         rgi, rgw, rgb = O.bn_backward(x, gy, g, rm, rv, sm, ss, train, 0.5, eps, gw0.copy(), gb0.copy())
-        close(gi.numpy(), rgi, 1e-4, 2e-4)
+        close(gi.numpy(), rgi)
         close(tgw.numpy(), rgw, WG_RTOL, 1e-3)
         close(tgb.numpy(), rgb, WG_RTOL, 1e-3)
         gi2 = CT.with_size(*shape)

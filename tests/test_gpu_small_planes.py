@@ -194,4 +194,4 @@ def test_run_kernels_decline_unaligned_tensors(T, off):
     THNN.BatchNormalization_updateOutput(_at_offset(T, x, off), out, None, None, rm, rv, sm, ss, True, 0.1, 1e-5)
     mean = x.mean(axis=(0, 2, 3), keepdims=True, dtype=np.float64)
     var = x.var(axis=(0, 2, 3), keepdims=True, dtype=np.float64)
-    close(out.numpy(), ((x - mean) / np.sqrt(var + 1e-5)).astype(np.float32), 1e-4, 2e-4)
+    close(out.numpy(), ((x - mean) / np.sqrt(var + 1e-5)).astype(np.float32))

@@ -12,7 +12,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def _declared(header):
     text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    names = re.findall(r"\b(THNN_Cuda\w+|THCState_\w+|THCuda(?:Long)?Tensor_\w+|THSet\w+)\s*\(", text)
+    names = re.findall(r"\b(THNN_Cuda\w+|THCState_\w+|THCuda(?:Long)?Tensor_\w+|THSet\w+|THCUNN_\w+)\s*\(", text)
     return sorted(set(names))
 
 
@@ -21,7 +21,9 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     declared = _declared("THCUNN.h") + _declared("THCShim.h")
     # 14 hot-path + 9 dilated / transposed convolution + 2 Threshold + the no-allocation accGradParameters variant
-    assert len([n for n in declared if n.startswith("THNN_Cuda")]) == 26
+    assert len(_declared("THCUNN.h")) == 26
+    # the test hooks: the two column kernels and the kernel-family switch
+    assert {"THNN_Cuda_im2col", "THNN_Cuda_col2im", "THCUNN_setSwitch"} <= set(_declared("THCShim.h"))
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/ but not exported"
 
@@ -70,3 +72,54 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libTHCUNN.so")
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         _lib.load()
+
+
+# ---- the prototypes are what the reference's binder would hand to ffi.cdef ---------------------------------
+REFERENCE_HEADER = "/root/reference/lib/THCUNN/generic/THCUNN.h"
+
+
+def _binder_cdef(text):
+    """THCUNN.lua:22-69 restated: strip preprocessor lines, `TH_API void THNN_(X)` -> `void THNN_TYPEX`, then
+    the plain substring replacements of the 'Cuda' (fp32) instantiation."""
+    text = re.sub(r"\n#[^\n]*", "", text)
+    text = re.sub(r"^#[^\n]*\n", "", text)
+    text = re.sub(r"TH_API void THNN_\(([A-Za-z0-9_]+)\)", r"void THNN_TYPE\1", text)
+    for k, v in (("THCTensor", "THCudaTensor"), ("THCIndexTensor", "THCudaLongTensor"), ("TYPE", "Cuda"), ("accreal", "float")):
+        text = text.replace(k, v)
+    return text
+
+
+def _prototypes(text):
+    """{name: [parameter type, ...]} of every `void THNN_Cuda<name>(...)` in C text (comments dropped,
+    parameter names dropped, whitespace normalised: 'THCudaTensor *', 'int', 'bool', 'float', 'double')."""
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    out = {}
+    for name, args in re.findall(r"void\s+THNN_Cuda(\w+)\s*\(([^)]*)\)\s*;", text):
+        types = []
+        for a in args.split(","):
+            a = " ".join(a.split())
+            m = re.match(r"^(.*?)(\w+)$", a)            # everything before the parameter name
+            t = m.group(1).replace(" *", "*").replace("* ", "*").strip()
+            types.append(re.sub(r"\s*\*", " *", t))
+        out[name] = types
+    return out
+
+
+@pytest.mark.skipif(not os.path.exists(REFERENCE_HEADER), reason="the reference tree is not on this machine")
+def test_prototypes_equal_the_binder_rewrite_of_the_reference_header():
+    """What LuaJIT would cdef from the reference's own header (THCUNN.lua:22-69) is, for every entry point this
+    library declares with a reference counterpart, exactly the prototype in include/THCUNN.h - and the ctypes
+    signatures of the Python harness say the same."""
+    import ctypes as C
+    from cunn_amd import _lib
+    ref = _prototypes(_binder_cdef(open(REFERENCE_HEADER).read()))
+    ours = _prototypes(open(os.path.join(ROOT, "include", "THCUNN.h")).read())
+    extensions = {"SpatialDepthWiseConvolution_accGradParameters_noAlloc"}   # no counterpart in the reference
+    assert set(ours) - set(ref) == extensions
+    assert len(set(ours) & set(ref)) == 25
+    ctype = {"THCState *": C.c_void_p, "THCudaTensor *": C.c_void_p, "THCudaLongTensor *": C.c_void_p, "int": C.c_int,
+             "bool": C.c_bool, "float": C.c_float, "double": C.c_double}
+    for name in sorted(set(ours) - extensions):
+        assert ours[name] == ref[name], f"{name}: {ours[name]} != {ref[name]}"
+        assert _lib.SIGNATURES[name] == [ctype[t] for t in ref[name]], name

@@ -99,6 +99,7 @@ SHIM = {  # name: (restype, argtypes)
     "THCudaLongTensor_nElement": (C.c_ssize_t, [_T, _T]),
     "THCudaLongTensor_copyFromHost": (None, [_T, _T, _T]),
     "THCudaLongTensor_copyToHost": (None, [_T, _T, _T]),
+    "THCUNN_setSwitch": (_i, [C.c_char_p, C.c_char_p]),
     "THNN_Cuda_im2col": (None, [_T, _T] + [_i] * 12 + [_T]),
     "THNN_Cuda_col2im": (None, [_T, _T] + [_i] * 12 + [_T]),
 }

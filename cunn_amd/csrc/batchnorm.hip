@@ -772,8 +772,7 @@ inline int currentDevice() {
 // The resident kernels hold a channel in the registers of one 1024-lane
 // workgroup: at most maxR float4 per lane, and enough channels to occupy the chip.
 int residentR(const BnView &v, int maxR) {
-  const char *e = getenv("THCUNN_BN_FORCE_CHUNKED");
-  if (e && e[0] == '1') return 0;
+  if (g_switches.bnChunked == 1) return 0;
   const BnGeom &g = v.g;
   if (!v.vec || g.C < 96 || g.L / 4 > kResBlock || (long)g.N * g.C * g.L * 4 >= 0x7fffffffL) return 0;
   long total4 = (long)g.N * (g.L / 4);
@@ -791,8 +790,7 @@ struct SmallChoice {
   int rs, bs;
 };
 SmallChoice smallR(const BnView &v) {
-  const char *e = getenv("THCUNN_BN_FORCE_CHUNKED");
-  if (e && e[0] == '1') return {0, 0};
+  if (g_switches.bnChunked == 1) return {0, 0};
   const BnGeom &g = v.g;
   const long NL = (long)g.N * g.L;
   if (g.L % 4 == 0 || g.C < 96 || NL > 32 * kResBlock || (long)g.N * g.C * g.L >= 0x7fffffffL) return {0, 0};

@@ -1474,10 +1474,7 @@ int residentSlots(const void *kernel) {
 
 // Test switch: "1" routes the forward pass (and the stride-1 gradInput that
 // reuses it) through the first-generation kernels.
-bool forceGeneric() {
-  const char *e = getenv("THCUNN_CONV_FORCE_GENERIC");
-  return e && e[0] == '1';
-}
+bool forceGeneric() { return g_switches.convGeneric == 1; }
 
 // Plan of one implicit-GEMM forward launch. The 128x128 tiles are dealt to the
 // CUs in rounds; a last partial round would leave most CUs idle while a few
@@ -1903,9 +1900,9 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
   }
   // With few input planes the phase GEMMs would use a sliver of their 64-row tiles; the column GEMM
   // (K rows) is the better shape then. Test switch THCUNN_CONV_GRADINPUT = "phases" / "columns" overrides.
-  const char *route = getenv("THCUNN_CONV_GRADINPUT");
+  const int route = g_switches.convGradInput;  // 1: phases, 2: columns
   const bool phasesPay = 2L * g.Cin >= (long)tiles(g.Cin, 64) * 64;
-  const bool tryPhases = route && !strcmp(route, "phases") ? true : route && !strcmp(route, "columns") ? false : phasesPay;
+  const bool tryPhases = route == 1 ? true : route == 2 ? false : phasesPay;
   if (!forceGeneric() && tryPhases && gradInputByPhase(state, g, gy, w, gi, scratchBuf, bufName, bias)) return;
   // Gradient columns of a group of images at a time (<= 128 MB so the buffer stays cache resident), then
   // the col2im gather. gradCol[n][k][l] = sum_o W[o][k] * gy[n][o][l] is itself a 1x1 convolution of gy

@@ -761,13 +761,10 @@ void launchStage2(hipStream_t s, int TP, const float *partial, float *gw, Stride
     dwAccGradStage2<32><<<CJ, dev::kWave, 0, s>>>(partial, gw, gs, gb, bs, M, kW, T, nslots, scale, CJ);
 }
 
-// Environment switch used by the tests to exercise the shape-agnostic kernels on
+// Switch used by the tests (THCUNN_setSwitch) to exercise the shape-agnostic kernels on
 // shapes the tiled ones would otherwise take.
 // 1: shape-agnostic direct kernels, 2: generic LDS-tiled kernels (no strip fast path).
-int forcedPath() {
-  const char *e = getenv("THCUNN_DW_FORCE_DIRECT");
-  return e ? atoi(e) : 0;
-}
+int forcedPath() { return g_switches.dwForce; }
 bool forceDirect() { return forcedPath() == 1; }
 
 // Geometry the strip kernels are compiled for.
@@ -814,10 +811,7 @@ enum SmallPass { kSmallFwd, kSmallGradInput, kSmallAccGrad };
 // kernels up to 28x28), and so do larger planes whose width or output width is not a multiple of 4 (which
 // the strip kernels need): two per workgroup up to 2048 elements, a band of rows per workgroup beyond. Test switch THCUNN_DW_SMALL: 0 never, 1 also for
 // the larger planes that the strip kernels could take.
-int smallSwitch() {
-  const char *e = getenv("THCUNN_DW_SMALL");
-  return e ? atoi(e) : -1;
-}
+int smallSwitch() { return g_switches.dwSmall; }
 
 constexpr int kSmallPlane = 1024;
 

@@ -703,10 +703,7 @@ poolBwdStrip(const float *__restrict__ gradOut, const long *__restrict__ indices
 using launch::aligned16;
 
 // 1: shape-agnostic direct kernels, 2: generic LDS-tiled kernels (no strip fast path).
-int forcedPath() {
-  const char *e = getenv("THCUNN_POOL_FORCE_DIRECT");
-  return e ? atoi(e) : 0;
-}
+int forcedPath() { return g_switches.poolForce; }
 bool forceDirect() { return forcedPath() == 1; }
 
 // 1 when no window of the average pooling is clipped, i.e. every divisor is kH*kW:
@@ -881,10 +878,7 @@ bool poolRunPlanFor(const PoolGeom &g, long planes, bool backward, bool max, Poo
   return out->lds <= launch::kLdsMax;
 }
 
-int runSwitch() {
-  const char *e = getenv("THCUNN_POOL_RUNS");
-  return e ? atoi(e) : -1;
-}
+int runSwitch() { return g_switches.poolRuns; }
 // Where both families apply (widths that are multiples of 4), measured on 8x8 ... 224x224 planes: the run
 // kernels' max forward wins up to 112x112 (16x16: 44 -> 12 us, 112x112: 64 -> 62 us; at 224x224 the strip
 // kernels are 5-15 % faster); the average forward wins up to 28x28 and the backward passes up to about 36x36

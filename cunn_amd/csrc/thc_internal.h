@@ -6,6 +6,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <exception>
 #include <string>
 #include <vector>
 
@@ -43,13 +44,20 @@ void dispatchError(const Error &e);  // calls the installed handler
                    #expr, __FILE__, __LINE__);                                      \
   } while (0)
 
-// Wraps the body of every extern "C" entry point.
+// Wraps the body of every extern "C" entry point: nothing may unwind into the C caller (ctypes, LuaJIT), so
+// whatever the standard library throws (bad_alloc of a host container ...) goes to the TH handler as well.
 #define THNN_ENTER try {
-#define THNN_LEAVE                    \
-  }                                   \
-  catch (const ::thc::Error &e__) {   \
-    ::thc::Error copy__ = e__;        \
-    ::thc::dispatchError(copy__);     \
+#define THNN_LEAVE                                                             \
+  }                                                                            \
+  catch (const ::thc::Error &e__) {                                            \
+    ::thc::Error copy__ = e__;                                                 \
+    ::thc::dispatchError(copy__);                                              \
+  }                                                                            \
+  catch (const std::exception &e__) {                                          \
+    ::thc::dispatchError(::thc::Error{std::string("C++ exception: ") + e__.what(), 0}); \
+  }                                                                            \
+  catch (...) {                                                                \
+    ::thc::dispatchError(::thc::Error{"unknown C++ exception", 0});           \
   }
 
 // ---- type-erased tensor view of THCudaTensor / THCudaLongTensor ------------
@@ -140,6 +148,23 @@ class Contiguous {
   const float *ptr_;
   Temp tmp_;
 };
+
+// ---- kernel-family switches ---------------------------------------------------
+// Several kernel families compute the same results; the parity tests force each of them. The switches take
+// their initial values from the environment once, when the library is loaded (THCUNN_DW_FORCE_DIRECT,
+// THCUNN_DW_SMALL, THCUNN_POOL_FORCE_DIRECT, THCUNN_POOL_RUNS, THCUNN_BN_FORCE_CHUNKED,
+// THCUNN_CONV_FORCE_GENERIC, THCUNN_CONV_GRADINPUT), and change afterwards only through THCUNN_setSwitch:
+// an entry point reads a plain int, never the environment.
+struct Switches {
+  int dwForce = 0;        // 1: shape-agnostic direct kernels, 2: generic LDS-tiled kernels
+  int dwSmall = -1;       // 0: never the run-of-memory kernels, 1: also where the strip kernels would be chosen
+  int poolForce = 0;      // as dwForce
+  int poolRuns = -1;      // as dwSmall
+  int bnChunked = 0;      // 1: the chunked two-pass kernels also where a channel fits one workgroup
+  int convGeneric = 0;    // 1: first-generation convolution kernels
+  int convGradInput = 0;  // 1: phase route, 2: gradient-column route, 0: by shape
+};
+extern Switches g_switches;
 
 // Looks up, for the current device `device`, the address of the fixed scratch array behind
 // THNN_CudaSpatialDepthWiseConvolution_accGradParameters_noAlloc (dwconv.hip). Called when a state is

@@ -51,6 +51,38 @@ void dispatchError(const Error &e) {
     g_errHandler(e.msg.c_str(), g_errData);
 }
 
+// -------------------------------------------------------------- switches ----
+static int switchValue(const char *name, const char *v, bool *known) {
+  *known = true;
+  if (!strcmp(name, "THCUNN_CONV_GRADINPUT")) return !v ? 0 : !strcmp(v, "phases") ? 1 : !strcmp(v, "columns") ? 2 : 0;
+  if (!strcmp(name, "THCUNN_DW_SMALL") || !strcmp(name, "THCUNN_POOL_RUNS")) return v ? atoi(v) : -1;
+  if (!strcmp(name, "THCUNN_DW_FORCE_DIRECT") || !strcmp(name, "THCUNN_POOL_FORCE_DIRECT") ||
+      !strcmp(name, "THCUNN_BN_FORCE_CHUNKED") || !strcmp(name, "THCUNN_CONV_FORCE_GENERIC"))
+    return v ? atoi(v) : 0;
+  *known = false;
+  return 0;
+}
+static int *switchSlot(Switches &s, const char *name) {
+  if (!strcmp(name, "THCUNN_DW_FORCE_DIRECT")) return &s.dwForce;
+  if (!strcmp(name, "THCUNN_DW_SMALL")) return &s.dwSmall;
+  if (!strcmp(name, "THCUNN_POOL_FORCE_DIRECT")) return &s.poolForce;
+  if (!strcmp(name, "THCUNN_POOL_RUNS")) return &s.poolRuns;
+  if (!strcmp(name, "THCUNN_BN_FORCE_CHUNKED")) return &s.bnChunked;
+  if (!strcmp(name, "THCUNN_CONV_FORCE_GENERIC")) return &s.convGeneric;
+  if (!strcmp(name, "THCUNN_CONV_GRADINPUT")) return &s.convGradInput;
+  return nullptr;
+}
+static Switches switchesFromEnvironment() {
+  Switches s;
+  for (const char *name : {"THCUNN_DW_FORCE_DIRECT", "THCUNN_DW_SMALL", "THCUNN_POOL_FORCE_DIRECT", "THCUNN_POOL_RUNS",
+                           "THCUNN_BN_FORCE_CHUNKED", "THCUNN_CONV_FORCE_GENERIC", "THCUNN_CONV_GRADINPUT"}) {
+    bool known;
+    *switchSlot(s, name) = switchValue(name, getenv(name), &known);
+  }
+  return s;
+}
+Switches g_switches = switchesFromEnvironment();  // read once, when the library is loaded
+
 // --------------------------------------------------------------- storage ----
 static Storage *storageNew(int device) {
   Storage *s = (Storage *)calloc(1, sizeof(Storage));
@@ -65,9 +97,16 @@ static void storageFree(Storage *s) {
   if ((s->flag & TH_STORAGE_FREEMEM) && s->data) (void)hipFree(s->data);
   free(s);
 }
+// Growth allocates with hipMalloc (which may wait for the device) and, when the storage already holds
+// data, copies it over and waits for the stream before the old block is freed: a first call at a new size
+// is not asynchronous. Steady-state calls (sizes unchanged) never get here.
 static void storageGrow(THCState *state, Storage *s, ptrdiff_t elems, size_t elemSize) {
   if (elems <= s->size) return;
   if (!(s->flag & TH_STORAGE_RESIZABLE)) error("Trying to resize storage that is not resizable");
+  // a storage that names an allocator of its own was not made by this library: its memory is that
+  // allocator's to move, so the caller has to size the tensor before the call
+  if (s->allocator)
+    error("Trying to resize a storage that carries its own allocator: give the tensor its final size before the call");
   void *p = nullptr;
   THC_HIP_CHECK(hipMalloc(&p, (size_t)elems * elemSize));
   if (s->data && s->size > 0) {
@@ -343,6 +382,15 @@ void THCState_synchronize(THCState *state) {
   THNN_ENTER
   THC_HIP_CHECK(hipStreamSynchronize(state->stream));
   THNN_LEAVE
+}
+
+int THCUNN_setSwitch(const char *name, const char *value) {
+  bool known = false;
+  if (!name) return 0;
+  const int v = switchValue(name, value, &known);
+  if (!known) return 0;
+  *switchSlot(g_switches, name) = v;
+  return 1;
 }
 
 void THSetErrorHandler(THErrorHandlerFunction handler, void *data) {

@@ -13,11 +13,11 @@ using namespace thc;
 
 namespace {
 
-// GRAD: out = x > thr ? other : 0 (other = gradOutput); else out = x > thr ? x : val
+// GRAD: out = x > thr ? other : 0 (other = gradOutput); else out = x > thr ? x : val.
+// The in-place entry points pass out == x (forward) or out == other (backward): no __restrict__ here.
 template <bool GRAD>
 __global__ void __launch_bounds__(dev::kBlock)
-thresholdKernel4(const float *__restrict__ x, const float *__restrict__ other, float *__restrict__ out, long n4,
-                 float thr, float val) {
+thresholdKernel4(const float *x, const float *other, float *out, long n4, float thr, float val) {
   const long i = (long)blockIdx.x * dev::kBlock + threadIdx.x;
   if (i >= n4) return;
   const float4 a = reinterpret_cast<const float4 *>(x)[i];
@@ -33,8 +33,7 @@ thresholdKernel4(const float *__restrict__ x, const float *__restrict__ other, f
 
 template <bool GRAD>
 __global__ void __launch_bounds__(dev::kBlock)
-thresholdKernel1(const float *__restrict__ x, const float *__restrict__ other, float *__restrict__ out, long begin,
-                 long n, float thr, float val) {
+thresholdKernel1(const float *x, const float *other, float *out, long begin, long n, float thr, float val) {
   const long i = begin + (long)blockIdx.x * dev::kBlock + threadIdx.x;
   if (i >= n) return;
   const float a = x[i];

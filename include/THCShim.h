@@ -139,6 +139,21 @@ ptrdiff_t THCudaLongTensor_nElement(THCState *state, const THCudaLongTensor *sel
 void THCudaLongTensor_copyFromHost(THCState *state, THCudaLongTensor *self, const long *src);
 void THCudaLongTensor_copyToHost(THCState *state, THCudaLongTensor *self, long *dst);
 
+/* ---- hooks for parity tests (no counterpart in the reference's C ABI) ---------- */
+/* The column kernels of lib/THCUNN/im2col.h:9-61 and :63-121 (C++ templates inside the reference library),
+ * on raw device pointers: `im` is nImages x channels x height x width, `col` is
+ * nImages x (channels*kH*kW) x (oH*oW); col2im overwrites `im` with the gathered sums. */
+void THNN_Cuda_im2col(THCState *state, const float *im, int nImages, int channels, int height, int width,
+                      int kH, int kW, int padH, int padW, int dH, int dW, int dilH, int dilW, float *col);
+void THNN_Cuda_col2im(THCState *state, const float *col, int nImages, int channels, int height, int width,
+                      int kH, int kW, int padH, int padW, int dH, int dW, int dilH, int dilW, float *im);
+/* Several kernel families compute the same results; this forces one. `name` is one of THCUNN_DW_FORCE_DIRECT,
+ * THCUNN_DW_SMALL, THCUNN_POOL_FORCE_DIRECT, THCUNN_POOL_RUNS, THCUNN_BN_FORCE_CHUNKED, THCUNN_CONV_FORCE_GENERIC,
+ * THCUNN_CONV_GRADINPUT; `value` is what the environment variable of that name would hold (read once, when the
+ * library is loaded), NULL restores the choice by shape. Returns 0 for an unknown name. Not thread-safe
+ * against concurrent calls of the entry points. */
+int THCUNN_setSwitch(const char *name, const char *value);
+
 #ifdef __cplusplus
 }
 #endif

@@ -8,6 +8,8 @@ import os
 import numpy as np
 import pytest
 
+import cunn_amd
+
 pytestmark = pytest.mark.gpu
 
 from oracle import oracle as O  # noqa: E402
@@ -109,12 +111,12 @@ def test_dilated_convolution_variants(T):
     _dil_run(T, DIL_CASES[0], bias=False, scale=0.5)
     _dil_run(T, DIL_CASES[3], xt=lambda a: T.CudaTensor.noncontiguous_from_numpy(a, rng), scale=2.0)
     _dil_run(T, (1,) + DIL_CASES[1][1:], single=True)
-    os.environ["THCUNN_CONV_FORCE_GENERIC"] = "1"
+    cunn_amd.set_switch("THCUNN_CONV_FORCE_GENERIC", "1")
     try:
         _dil_run(T, DIL_CASES[0])
         _dil_run(T, DIL_CASES[2])
     finally:
-        os.environ.pop("THCUNN_CONV_FORCE_GENERIC", None)
+        cunn_amd.set_switch("THCUNN_CONV_FORCE_GENERIC", None)
 
 
 def test_dilated_convolution_dilation_one_is_convmm(T):
@@ -208,12 +210,12 @@ def test_full_convolution_variants(T):
     _full_run(T, FULL_CASES[0], bias=False, scale=0.5, dilated_entry=False)
     _full_run(T, FULL_CASES[1], dilated_entry=False, xt=lambda a: T.CudaTensor.noncontiguous_from_numpy(a, rng), scale=2.0)
     _full_run(T, (1,) + FULL_CASES[2][1:], single=True, dilated_entry=False)
-    os.environ["THCUNN_CONV_FORCE_GENERIC"] = "1"
+    cunn_amd.set_switch("THCUNN_CONV_FORCE_GENERIC", "1")
     try:
         _full_run(T, FULL_CASES[0])
         _full_run(T, FULL_CASES[2])
     finally:
-        os.environ.pop("THCUNN_CONV_FORCE_GENERIC", None)
+        cunn_amd.set_switch("THCUNN_CONV_FORCE_GENERIC", None)
 
 
 def test_full_convolution_errors(T):
@@ -267,21 +269,21 @@ PHASE_DIL_CASES = [c for c in DIL_CASES if c[7] != 1 or c[8] != 1 or c[9] > c[11
 @pytest.mark.parametrize("route", ["phases", "columns"])
 @pytest.mark.parametrize("case", PHASE_DIL_CASES)
 def test_gradinput_routes(T, case, route):
-    os.environ["THCUNN_CONV_GRADINPUT"] = route
+    cunn_amd.set_switch("THCUNN_CONV_GRADINPUT", route)
     try:
         _dil_run(T, case, seed=83)
     finally:
-        os.environ.pop("THCUNN_CONV_GRADINPUT", None)
+        cunn_amd.set_switch("THCUNN_CONV_GRADINPUT", None)
 
 
 @pytest.mark.parametrize("route", ["phases", "columns"])
 @pytest.mark.parametrize("case", FULL_CASES + [(2, 24, 64, 9, 11, 4, 4, 2, 2, 1, 1, 1, 1, 0, 1)])
 def test_full_convolution_routes(T, case, route):
-    os.environ["THCUNN_CONV_GRADINPUT"] = route
+    cunn_amd.set_switch("THCUNN_CONV_GRADINPUT", route)
     try:
         _full_run(T, case, seed=92)
     finally:
-        os.environ.pop("THCUNN_CONV_GRADINPUT", None)
+        cunn_amd.set_switch("THCUNN_CONV_GRADINPUT", None)
 
 
 def _random_geometry(rng):
@@ -306,8 +308,8 @@ def test_convolution_random_geometries(T, seed):
     case = _random_geometry(rng)
     route = [None, "phases", "columns"][seed % 3]
     if route:
-        os.environ["THCUNN_CONV_GRADINPUT"] = route
+        cunn_amd.set_switch("THCUNN_CONV_GRADINPUT", route)
     try:
         _dil_run(T, case, seed=2000 + seed, scale=float(rng.choice([1.0, 0.5])))
     finally:
-        os.environ.pop("THCUNN_CONV_GRADINPUT", None)
+        cunn_amd.set_switch("THCUNN_CONV_GRADINPUT", None)

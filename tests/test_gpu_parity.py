@@ -13,6 +13,8 @@ import os
 import numpy as np
 import pytest
 
+import cunn_amd
+
 pytestmark = pytest.mark.gpu
 
 from oracle import oracle as O  # noqa: E402
@@ -39,10 +41,10 @@ class force_direct:
         self.var, self.mode = var, mode
 
     def __enter__(self):
-        os.environ[self.var] = self.mode
+        cunn_amd.set_switch(self.var, self.mode)
 
     def __exit__(self, *a):
-        os.environ.pop(self.var, None)
+        cunn_amd.set_switch(self.var, None)
 
 
 # ------------------------------------------------------------------ depthwise --
@@ -555,11 +557,11 @@ def test_batchnorm(T, shape, affine):
 
 
 def test_batchnorm_chunked_path_on_resident_shape(T):
-    os.environ["THCUNN_BN_FORCE_CHUNKED"] = "1"
+    cunn_amd.set_switch("THCUNN_BN_FORCE_CHUNKED", "1")
     try:
         _bn_run(T, (40, 96, 20, 20), True)
     finally:
-        os.environ.pop("THCUNN_BN_FORCE_CHUNKED", None)
+        cunn_amd.set_switch("THCUNN_BN_FORCE_CHUNKED", None)
 
 
 def test_batchnorm_large_mean_and_zero_variance(T):
@@ -635,12 +637,12 @@ def test_convmm(T, case):
 
 
 def test_convmm_first_generation_kernels(T):
-    os.environ["THCUNN_CONV_FORCE_GENERIC"] = "1"
+    cunn_amd.set_switch("THCUNN_CONV_FORCE_GENERIC", "1")
     try:
         _conv_run(T, CONV_CASES[0])
         _conv_run(T, CONV_CASES[3])
     finally:
-        os.environ.pop("THCUNN_CONV_FORCE_GENERIC", None)
+        cunn_amd.set_switch("THCUNN_CONV_FORCE_GENERIC", None)
 
 
 def test_convmm_variants(T):

@@ -455,6 +455,66 @@ def wl_relu(nsets):
                 desc="Threshold (ReLU) fwd+bwd fp32 N=64 C=128 56x56")
 
 
+def wl_bnrelu(nsets, fused=True):
+    """Beyond the five configurations: BatchNormalization (train) + ReLU forward and backward on the cfg3 tensor, as the
+    fused entry points (include/THCUNN_fused.h) or as the four separate calls they replace."""
+    from cunn_amd import CudaTensor as CT, THNN
+    from oracle import oracle as O
+    N, Cc, H = 64, 256, 28
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((N, Cc, H, H)) * 2 + 0.5).astype(np.float32)
+    gy = rng.standard_normal((N, Cc, H, H)).astype(np.float32)
+    g = (rng.random(Cc) + 0.25).astype(np.float32)
+    b = rng.standard_normal(Cc).astype(np.float32)
+    z = lambda: CT.from_numpy(np.zeros(Cc, np.float32))
+    sets = [dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), a=CT(), ga=CT(), gx=CT.with_size(N, Cc, H, H), g=CT.from_numpy(g),
+                 b=CT.from_numpy(b), rm=z(), rv=CT.from_numpy(np.ones(Cc, np.float32)), sm=CT.with_size(Cc), ss=CT.with_size(Cc),
+                 gw=z(), gb=z()) for _ in range(nsets)]
+
+    def calls(i):
+        t = sets[i]
+        if fused:
+            return [("bnrelu_updateOutput", lambda: THNN.BatchNormalizationReLU_updateOutput(
+                        t["x"], t["a"], t["g"], t["b"], t["rm"], t["rv"], t["sm"], t["ss"], True, 0.1, 1e-5)),
+                    ("bnrelu_backward", lambda: THNN.BatchNormalizationReLU_backward(
+                        t["x"], t["gy"], t["gx"], t["gw"], t["gb"], t["g"], t["b"], t["rm"], t["rv"], t["sm"], t["ss"], True, 1.0, 1e-5))]
+        return [("bn_updateOutput", lambda: THNN.BatchNormalization_updateOutput(
+                    t["x"], t["y"], t["g"], t["b"], t["rm"], t["rv"], t["sm"], t["ss"], True, 0.1, 1e-5)),
+                ("threshold_updateOutput", lambda: THNN.Threshold_updateOutput(t["y"], t["a"], 0.0, 0.0, False)),
+                ("threshold_updateGradInput", lambda: THNN.Threshold_updateGradInput(t["y"], t["gy"], t["ga"], 0.0, 0.0, False)),
+                ("bn_backward", lambda: THNN.BatchNormalization_backward(
+                    t["x"], t["ga"], t["gx"], t["gw"], t["gb"], t["g"], t["rm"], t["rv"], t["sm"], t["ss"], True, 1.0, 1e-5))]
+
+    xb = x.nbytes
+    # algorithmic bytes of the pair: x in, activation out; x and gradOutput in, gradInput out - whichever way it is computed
+    work = ({"bnrelu_updateOutput": (2 * xb, "bytes"), "bnrelu_backward": (3 * xb, "bytes")} if fused else
+            {"bn_updateOutput": (2 * xb, "bytes"), "threshold_updateOutput": (0, "bytes"), "threshold_updateGradInput": (0, "bytes"),
+             "bn_backward": (3 * xb, "bytes")})
+
+    def cpu(reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            rm, rv = np.zeros(Cc, np.float32), np.ones(Cc, np.float32)
+            y, sm, ss = O.bn_updateOutput(x, g, b, rm, rv, True, 0.1, 1e-5)
+            O.threshold_updateOutput(y, 0.0, 0.0)
+            O.bn_backward(x, O.threshold_updateGradInput(y, gy, 0.0), g, rm, rv, sm, ss, True, 1.0, 1e-5,
+                          np.zeros(Cc, np.float32), np.zeros(Cc, np.float32))
+        return time.perf_counter() - t0, reps * N, f"{reps} full passes ({N} images each)"
+
+    def verify():
+        t = sets[0]
+        for _, fn in calls(0):
+            fn()
+        rm, rv = np.zeros(Cc, np.float32), np.ones(Cc, np.float32)
+        y, sm, ss = O.bn_updateOutput(x, g, b, rm, rv, True, 0.1, 1e-5)
+        np.testing.assert_allclose(t["a"].numpy(), O.threshold_updateOutput(y, 0.0, 0.0), rtol=1e-5, atol=1e-4)
+        t["gw"].fill(0.0), t["gb"].fill(0.0)
+
+    return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="hbm",
+                desc=f"BatchNormalization (train) + ReLU fwd+bwd fp32 N={N} C={Cc} {H}x{H}, "
+                     + ("fused entry points" if fused else "four separate calls"))
+
+
 def wl_copy(nsets):
     """Calibration: plain device-to-device copy of 128 MB (2 x 128 MB of HBM traffic per launch)."""
     from cunn_amd import CudaTensor as CT
@@ -476,7 +536,8 @@ def wl_copy(nsets):
 
 WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda n: wl_dw("cfg2", n), "cfg3": wl_bn, "cfg4": wl_pool,
              "dw147": lambda n: wl_dw("dw147", n), "dw14": lambda n: wl_dw("dw14", n), "pool71": lambda n: wl_pool(n, odd=True),
-             "cfg5": wl_conv, "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu}
+             "cfg5": wl_conv, "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu,
+             "bnrelu": wl_bnrelu, "bnrelu_unfused": lambda n: wl_bnrelu(n, fused=False)}
 
 
 PREROLL_SAMPLES = 12   # event samples per entry point collected before the timed region, whatever --warmup is
@@ -531,6 +592,7 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds):
             scale, peak, unit = 1e9, HBM_PEAK_GBS, "GB/s"
         else:
             scale, peak, unit = 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
+        amount = max(amount, 1)           # entry points with no algorithmic traffic of their own (the unfused ReLU steps)
         kern[n] = dict(avg_ms=avg, median_ms=med, min_ms=float(np.min(per_kernel[n])), samples=len(per_kernel[n]),
                        achieved=amount / (avg * 1e-3) / scale, achieved_median=amount / (med * 1e-3) / scale,
                        peak=peak, unit=unit, frac=amount / (avg * 1e-3) / scale / peak,

@@ -28,6 +28,8 @@ ENTRY_POINTS = [
     "Threshold_updateOutput", "Threshold_updateGradInput",
     # no counterpart in the reference: for callers that cannot allocate device memory
     "SpatialDepthWiseConvolution_accGradParameters_noAlloc",
+    # no counterpart in the reference: BatchNormalization + Threshold(0, 0) in one pass (include/THCUNN_fused.h)
+    "BatchNormalizationReLU_updateOutput", "BatchNormalizationReLU_backward",
 ]
 
 _T = C.c_void_p  # THCudaTensor* / THCudaLongTensor* / THCState*
@@ -60,6 +62,8 @@ SIGNATURES = {
     "Threshold_updateOutput": [_T] * 3 + [_f, _f, _b],
     "Threshold_updateGradInput": [_T] * 4 + [_f, _f, _b],
     "SpatialDepthWiseConvolution_accGradParameters_noAlloc": [_T] * 5 + [_i] * 6 + [_f],
+    "BatchNormalizationReLU_updateOutput": [_T] * 9 + [_b, _d, _d],
+    "BatchNormalizationReLU_backward": [_T] * 12 + [_b, _d, _d],
 }
 
 _LP = C.POINTER(C.c_long)

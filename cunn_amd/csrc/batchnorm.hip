@@ -110,6 +110,14 @@ __device__ __forceinline__ void blockSum(float (&v)[NV], float (*red)[NV]) {
   }
 }
 
+// One normalised element, y = gamma * (x - mean) * invStd + beta, in a fixed sequence of fp32 operations: the
+// forward kernels store it and the fused ReLU backward re-derives its sign from x, so both must round alike.
+__device__ __forceinline__ float bnAffine(float x, float mean, float invStd, float gamma, float beta) {
+  return __builtin_fmaf(gamma * (x - mean), invStd, beta);
+}
+// Threshold(0, 0) of lib/THCUNN/Threshold.cu:6-20 on top of it when `relu` is set: v > 0 ? v : 0 (NaN -> 0)
+__device__ __forceinline__ float bnAct(float v, int relu) { return (relu && !(v > 0.f)) ? 0.f : v; }
+
 // ------------------------------------------------------ forward statistics ----
 // partial[(ch * chunks + chunk) * 3 + {0,1,2}] = count, mean, M2 of the chunk
 template <int VEC>
@@ -180,7 +188,7 @@ __global__ void __launch_bounds__(dev::kBlock)
 bnApplyKernel(const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ partial,
               const float *__restrict__ weight, const float *__restrict__ bias, float *__restrict__ runningMean,
               float *__restrict__ runningVar, float *__restrict__ saveMean, float *__restrict__ saveStd, BnGeom g,
-              float momentum, float eps) {
+              float momentum, float eps, int relu) {
   __shared__ float bc[2];
   // the statistics pass went through the tensor front to back: going back to front meets what it read last
   // while that is still in the last-level cache
@@ -219,36 +227,68 @@ bnApplyKernel(const float *__restrict__ x, float *__restrict__ y, const float *_
   forChunk<VEC>(g, ch, c, [&](long off, auto width) {
     if constexpr (decltype(width)::value == 4) {
       float4 q = *reinterpret_cast<const float4 *>(x + off), r;
-      r.x = gamma * (q.x - mean) * invStd + beta;
-      r.y = gamma * (q.y - mean) * invStd + beta;
-      r.z = gamma * (q.z - mean) * invStd + beta;
-      r.w = gamma * (q.w - mean) * invStd + beta;
+      r.x = bnAct(bnAffine(q.x, mean, invStd, gamma, beta), relu);
+      r.y = bnAct(bnAffine(q.y, mean, invStd, gamma, beta), relu);
+      r.z = bnAct(bnAffine(q.z, mean, invStd, gamma, beta), relu);
+      r.w = bnAct(bnAffine(q.w, mean, invStd, gamma, beta), relu);
       dev::storeStream4(y + off, r);  // written once, read by another kernel: keeps x in the caches for the two-pass re-read
     } else {
-      y[off] = gamma * (x[off] - mean) * invStd + beta;
+      y[off] = bnAct(bnAffine(x[off], mean, invStd, gamma, beta), relu);
     }
   });
 }
+
+// ------------------------------------------------- fused ReLU in the backward ----
+// With the fused activation the gradient that reaches the normalisation is gradOutput where the forward
+// output was positive and 0 elsewhere (lib/THCUNN/Threshold.cu:42-56). The output is not an operand of
+// the backward pass: its sign is re-derived from x with the forward's own arithmetic (bnAffine).
+struct ReluMask {
+  int relu;             // 0: plain batch normalisation, nothing is masked
+  int train;            // which statistics stdSrc holds: 1/sigma of the batch, or the running variance
+  const float *weight;  // gamma (NULL: 1)
+  const float *bias;    // beta (NULL: 0)
+  const float *stdSrc;
+  float eps;
+};
+struct ChannelMask {
+  int relu;
+  float mean, invStd, gamma, beta;
+  __device__ ChannelMask(const ReluMask &rm, int ch, float mean_) : relu(rm.relu), mean(mean_), invStd(0.f), gamma(1.f), beta(0.f) {
+    if (relu) {
+      invStd = rm.train ? rm.stdSrc[ch] : 1.f / sqrtf(rm.stdSrc[ch] + rm.eps);
+      gamma = rm.weight ? rm.weight[ch] : 1.f;
+      beta = rm.bias ? rm.bias[ch] : 0.f;
+    }
+  }
+  __device__ __forceinline__ float apply(float d, float x) const {
+    return (relu && !(bnAffine(x, mean, invStd, gamma, beta) > 0.f)) ? 0.f : d;
+  }
+  __device__ __forceinline__ void apply(float4 &d, const float4 &q) const {
+    d.x = apply(d.x, q.x), d.y = apply(d.y, q.y), d.z = apply(d.z, q.z), d.w = apply(d.w, q.w);
+  }
+};
 
 // ----------------------------------------------------------- backward sums ----
 // partial[(ch * chunks + chunk) * 2 + {0,1}] = sum gy, sum gy * (x - mean)
 template <int VEC>
 __global__ void __launch_bounds__(dev::kBlock)
 bnGradSumsKernel(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ partial,
-                 const float *__restrict__ meanSrc, BnGeom g) {
+                 const float *__restrict__ meanSrc, BnGeom g, ReluMask rm) {
   __shared__ float red[dev::kBlock / dev::kWave][2];
   const int ch = blockIdx.x / g.chunks, chunk = blockIdx.x - ch * g.chunks;
   const Chunk c = chunkOf(g, chunk);
   const float mean = meanSrc[ch];
+  const ChannelMask m(rm, ch, mean);
   float v[2] = {0.f, 0.f};
   forChunk<VEC>(g, ch, c, [&](long off, auto width) {
     if constexpr (decltype(width)::value == 4) {
       float4 q = *reinterpret_cast<const float4 *>(x + off);
       float4 d = *reinterpret_cast<const float4 *>(gy + off);
+      m.apply(d, q);
       v[0] += (d.x + d.y) + (d.z + d.w);
       v[1] += (d.x * (q.x - mean) + d.y * (q.y - mean)) + (d.z * (q.z - mean) + d.w * (q.w - mean));
     } else {
-      float d = gy[off];
+      float d = m.apply(gy[off], x[off]);
       v[0] += d;
       v[1] += d * (x[off] - mean);
     }
@@ -283,11 +323,12 @@ __global__ void __launch_bounds__(dev::kBlock)
 bnBackwardKernel(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
                  const float *__restrict__ partial, float *__restrict__ gradWeight, float *__restrict__ gradBias,
                  const float *__restrict__ weight, const float *__restrict__ meanSrc,
-                 const float *__restrict__ stdSrc, BnGeom g, float scale, float eps) {
+                 const float *__restrict__ stdSrc, BnGeom g, float scale, float eps, ReluMask rm) {
   __shared__ float bc[2];
   const int bid = gridDim.x - 1 - blockIdx.x;  // back to front, see bnApplyKernel
   const int ch = bid / g.chunks, chunk = bid - ch * g.chunks;
   const float mean = meanSrc[ch];
+  const ChannelMask m(rm, ch, mean);
   const float stdVal = TRAIN ? stdSrc[ch] : 1.f / sqrtf(stdSrc[ch] + eps);
   const float weightVal = weight ? weight[ch] : 1.f;
   float gradOutputSum = 0.f, dotP = 0.f;
@@ -315,19 +356,21 @@ bnBackwardKernel(const float *__restrict__ x, const float *__restrict__ gy, floa
         float4 d = *reinterpret_cast<const float4 *>(gy + off), r;
         if (TRAIN) {
           float4 q = *reinterpret_cast<const float4 *>(x + off);
+          m.apply(d, q);
           r.x = (d.x - (q.x - mean) * projScale - gradMean) * gradScale;
           r.y = (d.y - (q.y - mean) * projScale - gradMean) * gradScale;
           r.z = (d.z - (q.z - mean) * projScale - gradMean) * gradScale;
           r.w = (d.w - (q.w - mean) * projScale - gradMean) * gradScale;
         } else {
+          if (m.relu) m.apply(d, *reinterpret_cast<const float4 *>(x + off));
           r.x = d.x * gradScale, r.y = d.y * gradScale, r.z = d.z * gradScale, r.w = d.w * gradScale;
         }
         dev::storeStream4(gx + off, r);
       } else {
         if (TRAIN)
-          gx[off] = (gy[off] - (x[off] - mean) * projScale - gradMean) * gradScale;
+          gx[off] = (m.apply(gy[off], x[off]) - (x[off] - mean) * projScale - gradMean) * gradScale;
         else
-          gx[off] = gy[off] * gradScale;
+          gx[off] = (m.relu ? m.apply(gy[off], x[off]) : gy[off]) * gradScale;
       }
     });
   }
@@ -390,7 +433,7 @@ __global__ void __launch_bounds__(kResBlock)
 bnFwdResident(const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ weight,
               const float *__restrict__ bias, float *__restrict__ runningMean, float *__restrict__ runningVar,
               float *__restrict__ saveMean, float *__restrict__ saveStd, int N, int C, int L, float momentum,
-              float eps) {
+              float eps, int relu) {
   __shared__ float red[kResWaves];
   const int ch = blockIdx.x;
   const int total4 = N * (L >> 2);
@@ -434,10 +477,10 @@ bnFwdResident(const float *__restrict__ x, float *__restrict__ y, const float *_
   for (int u = 0; u < R; ++u) {
     if (u * kResBlock + (int)threadIdx.x < total4) {
       float4 r;
-      r.x = gamma * (v[u].x - mean) * invStd + beta;
-      r.y = gamma * (v[u].y - mean) * invStd + beta;
-      r.z = gamma * (v[u].z - mean) * invStd + beta;
-      r.w = gamma * (v[u].w - mean) * invStd + beta;
+      r.x = bnAct(bnAffine(v[u].x, mean, invStd, gamma, beta), relu);
+      r.y = bnAct(bnAffine(v[u].y, mean, invStd, gamma, beta), relu);
+      r.z = bnAct(bnAffine(v[u].z, mean, invStd, gamma, beta), relu);
+      r.w = bnAct(bnAffine(v[u].w, mean, invStd, gamma, beta), relu);
       dev::bufStoreStream4(yr, wk.offset(), r);
     }
     wk.next();
@@ -453,7 +496,7 @@ __global__ void __launch_bounds__(kResBlock)
 bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
               float *__restrict__ gradWeight, float *__restrict__ gradBias, const float *__restrict__ weight,
               const float *__restrict__ meanSrc, const float *__restrict__ stdSrc, int N, int C, int L, float scale,
-              float eps, int xlds) {
+              float eps, int xlds, ReluMask rm) {
   __shared__ float red[kResWaves];
   extern __shared__ float4 xpark[];  // !KEEPX: the first xlds (a multiple of 4) float4 of x per lane wait here for the apply phase
   const int ch = blockIdx.x;
@@ -461,6 +504,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
   const float mean = meanSrc[ch];
   const float stdVal = TRAIN ? stdSrc[ch] : 1.f / sqrtf(stdSrc[ch] + eps);
   const float weightVal = weight ? weight[ch] : 1.f;
+  const ChannelMask m(rm, ch, mean);
   const long span = ((long)(N - 1) * C * L + L) * 4;
   const __amdgpu_buffer_rsrc_t xr = dev::makeRsrc(x + (long)ch * L, span), gr = dev::makeRsrc(gy + (long)ch * L, span);
   const __amdgpu_buffer_rsrc_t or_ = dev::makeRsrc(gx ? gx + (long)ch * L : x, gx ? span : 0);
@@ -484,6 +528,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
 #pragma unroll
       for (int u = 0; u < R; ++u) {
         float4 &q = xc[KEEPX ? u : 0];
+        m.apply(d[u], q);
         q.x -= mean, q.y -= mean, q.z -= mean, q.w -= mean;
         s0 += (d[u].x + d[u].y) + (d[u].z + d[u].w);
         s1 += (d[u].x * q.x + d[u].y * q.y) + (d[u].z * q.z + d[u].w * q.w);
@@ -516,6 +561,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
 #pragma unroll
         for (int k = 0; k < XB; ++k)
           if (u0 + k < R) {
+            m.apply(d[u0 + k], q[k]);
             const float4 &g4 = d[u0 + k];
             s0 += (g4.x + g4.y) + (g4.z + g4.w);
             s1 += (g4.x * (q[k].x - mean) + g4.y * (q[k].y - mean)) + (g4.z * (q[k].z - mean) + g4.w * (q[k].w - mean));
@@ -625,7 +671,7 @@ __global__ void __launch_bounds__(BS)
 bnFwdSmall(const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ weight,
            const float *__restrict__ bias, float *__restrict__ runningMean, float *__restrict__ runningVar,
            float *__restrict__ saveMean, float *__restrict__ saveStd, int N, int C, int L, unsigned magicL,
-           float momentum, float eps) {
+           float momentum, float eps, int relu) {
   __shared__ float red[BS / dev::kWave];
   const int ch = blockIdx.x;
   const float *xc = x + (long)ch * L;
@@ -657,7 +703,7 @@ bnFwdSmall(const float *__restrict__ x, float *__restrict__ y, const float *__re
   const float gamma = weight ? weight[ch] : 1.f, beta = bias ? bias[ch] : 0.f;
 #pragma unroll
   for (int u = 0; u < RS; ++u)
-    if (off[u] >= 0) yc[off[u]] = gamma * (v[u] - mean) * invStd + beta;
+    if (off[u] >= 0) yc[off[u]] = bnAct(bnAffine(v[u], mean, invStd, gamma, beta), relu);
 }
 
 template <int RS, bool TRAIN, int BS>
@@ -665,11 +711,12 @@ __global__ void __launch_bounds__(BS)
 bnBwdSmall(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
            float *__restrict__ gradWeight, float *__restrict__ gradBias, const float *__restrict__ weight,
            const float *__restrict__ meanSrc, const float *__restrict__ stdSrc, int N, int C, int L, unsigned magicL,
-           float scale, float eps) {
+           float scale, float eps, ReluMask rm) {
   __shared__ float red[BS / dev::kWave];
   const int ch = blockIdx.x;
   const float *xc = x + (long)ch * L, *gc = gy + (long)ch * L;
   const float mean = meanSrc[ch];
+  const ChannelMask m(rm, ch, mean);
   const float stdVal = TRAIN ? stdSrc[ch] : 1.f / sqrtf(stdSrc[ch] + eps);
   const float weightVal = weight ? weight[ch] : 1.f;
   int off[RS];
@@ -683,6 +730,7 @@ bnBwdSmall(const float *__restrict__ x, const float *__restrict__ gy, float *__r
   float s0 = 0.f, s1 = 0.f;
 #pragma unroll
   for (int u = 0; u < RS; ++u) {
+    d[u] = m.apply(d[u], xm[u]);
     xm[u] -= mean;
     s0 += d[u];
     s1 += d[u] * xm[u];
@@ -802,16 +850,11 @@ SmallChoice smallR(const BnView &v) {
   return {0, 0};
 }
 
-}  // namespace
-
-extern "C" {
-
-void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *input_, THCudaTensor *output_,
-                                              THCudaTensor *weight_, THCudaTensor *bias_,
-                                              THCudaTensor *runningMean_, THCudaTensor *runningVar_,
-                                              THCudaTensor *saveMean_, THCudaTensor *saveStd_, bool train,
-                                              double momentum, double eps) {
-  THNN_ENTER
+// lib/THCUNN/generic/BatchNormalization.cu:34-66; relu: Threshold(0, 0) applied to every element before it is stored
+void bnUpdateOutput(THCState *state, THCudaTensor *input_, THCudaTensor *output_, THCudaTensor *weight_,
+                    THCudaTensor *bias_, THCudaTensor *runningMean_, THCudaTensor *runningVar_,
+                    THCudaTensor *saveMean_, THCudaTensor *saveStd_, bool train, double momentum, double eps,
+                    int relu) {
   THC_ARG_CHECK(input_ != nullptr, 2, "input tensor expected");
   THC_ARG_CHECK(output_ != nullptr, 3, "output tensor expected");
   tensorResize(state, erase(output_), input_->nDimension, input_->size, sizeof(float));  // resizeAs (:40)
@@ -836,7 +879,7 @@ void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *inp
   if (R == RR)                                                                                                      \
     bnFwdResident<RR><<<g.C, kResBlock, 0, s>>>(in.ptr(), data(output_), dataOrNull(weight_), dataOrNull(bias_),    \
                                                 data(runningMean_), data(runningVar_), data(saveMean_),             \
-                                                data(saveStd_), g.N, g.C, g.L, (float)momentum, (float)eps);
+                                                data(saveStd_), g.N, g.C, g.L, (float)momentum, (float)eps, relu);
     BN_FWD_RES(2) BN_FWD_RES(4) BN_FWD_RES(8) BN_FWD_RES(12) BN_FWD_RES(13) BN_FWD_RES(14)
 #undef BN_FWD_RES
     THC_HIP_CHECK(hipGetLastError());
@@ -847,7 +890,7 @@ void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *inp
   if (sc.rs == RR && sc.bs == BS)                                                                                   \
     bnFwdSmall<RR, BS><<<g.C, BS, 0, s>>>(in.ptr(), data(output_), dataOrNull(weight_), dataOrNull(bias_),          \
                                           data(runningMean_), data(runningVar_), data(saveMean_), data(saveStd_),   \
-                                          g.N, g.C, g.L, dev::magicOf(g.L), (float)momentum, (float)eps);
+                                          g.N, g.C, g.L, dev::magicOf(g.L), (float)momentum, (float)eps, relu);
     BN_FWD_SMALL(4, kSmallBlock) BN_FWD_SMALL(8, kSmallBlock) BN_FWD_SMALL(16, kSmallBlock) BN_FWD_SMALL(32, kSmallBlock)
     BN_FWD_SMALL(16, kResBlock) BN_FWD_SMALL(32, kResBlock)
 #undef BN_FWD_SMALL
@@ -863,7 +906,7 @@ void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *inp
     bnApplyKernel<true, MODE><<<grid, block, 0, s>>>(in.ptr(), data(output_), p, dataOrNull(weight_),             \
                                                      dataOrNull(bias_), data(runningMean_), data(runningVar_),    \
                                                      data(saveMean_), data(saveStd_), g, (float)momentum,         \
-                                                     (float)eps);                                                 \
+                                                     (float)eps, relu);                                           \
   }
     if (v.mode == 1) BN_FWD_TRAIN(1) else if (v.mode == 2) BN_FWD_TRAIN(2) else BN_FWD_TRAIN(0)
 #undef BN_FWD_TRAIN
@@ -871,21 +914,19 @@ void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *inp
 #define BN_FWD_EVAL(MODE)                                                                                         \
   bnApplyKernel<false, MODE><<<grid, block, 0, s>>>(in.ptr(), data(output_), nullptr, dataOrNull(weight_),        \
                                                     dataOrNull(bias_), data(runningMean_), data(runningVar_),     \
-                                                    nullptr, nullptr, g, (float)momentum, (float)eps);
+                                                    nullptr, nullptr, g, (float)momentum, (float)eps, relu);
     if (v.mode == 1) BN_FWD_EVAL(1) else if (v.mode == 2) BN_FWD_EVAL(2) else BN_FWD_EVAL(0)
 #undef BN_FWD_EVAL
   }
   THC_HIP_CHECK(hipGetLastError());
-  THNN_LEAVE
 }
 
-void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_, THCudaTensor *gradOutput_,
-                                          THCudaTensor *gradInput_, THCudaTensor *gradWeight_,
-                                          THCudaTensor *gradBias_, THCudaTensor *weight_,
-                                          THCudaTensor *runningMean_, THCudaTensor *runningVar_,
-                                          THCudaTensor *saveMean_, THCudaTensor *saveStd_, bool train, double scale,
-                                          double eps) {
-  THNN_ENTER
+// lib/THCUNN/generic/BatchNormalization.cu:68-94; relu: gradOutput counts only where the fused forward output was
+// positive (bias_ is needed to re-derive that sign from the input)
+void bnBackward(THCState *state, THCudaTensor *input_, THCudaTensor *gradOutput_, THCudaTensor *gradInput_,
+                THCudaTensor *gradWeight_, THCudaTensor *gradBias_, THCudaTensor *weight_, THCudaTensor *bias_,
+                THCudaTensor *runningMean_, THCudaTensor *runningVar_, THCudaTensor *saveMean_,
+                THCudaTensor *saveStd_, bool train, double scale, double eps, int relu) {
   THC_ARG_CHECK(input_ != nullptr, 2, "input tensor expected");
   THC_ARG_CHECK(gradOutput_ != nullptr, 3, "gradOutput tensor expected");
   if (!sameSize(erase(input_), erase(gradOutput_)))  // THCUNN_check_shape (:74)
@@ -906,6 +947,7 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
   checkVector(gradWeight_, "gradWeight", g.C, false);
   checkVector(gradBias_, "gradBias", g.C, false);
   checkVector(weight_, "weight", g.C, false);
+  if (relu) checkVector(bias_, "bias", g.C, false);
   if (train) {
     checkVector(saveMean_, "saveMean", g.C, true);
     checkVector(saveStd_, "saveStd", g.C, true);
@@ -920,6 +962,7 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
   dim3 grid((unsigned)(g.C * g.chunks)), block(dev::kBlock);
   const float *meanSrc = train ? data(saveMean_) : data(runningMean_);
   const float *stdSrc = train ? data(saveStd_) : data(runningVar_);
+  const ReluMask rm{relu, train ? 1 : 0, dataOrNull(weight_), relu ? dataOrNull(bias_) : nullptr, stdSrc, (float)eps};
   const bool needSums = (train && gradInput_) || gradWeight_ || gradBias_;
   if (int R = needSums ? residentR(v, 13) : 0) {
     float *gxp = gradInput_ ? data(gradInput_) : nullptr;
@@ -939,11 +982,11 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
       }                                                                                                            \
       bnBwdResident<RR, true, (RR <= 8)><<<g.C, kResBlock, lds, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_), \
                                                         dataOrNull(gradBias_), dataOrNull(weight_), meanSrc,       \
-                                                        stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, xlds);    \
+                                                        stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, xlds, rm); \
     } else {                                                                                                       \
       bnBwdResident<RR, false, (RR <= 8)><<<g.C, kResBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_), \
                                                          dataOrNull(gradBias_), dataOrNull(weight_), meanSrc,      \
-                                                         stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, 0);      \
+                                                         stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, 0, rm);  \
     }                                                                                                              \
   }
     BN_BWD_RES(2) BN_BWD_RES(4) BN_BWD_RES(8) BN_BWD_RES(12) BN_BWD_RES(13)
@@ -958,11 +1001,11 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
     if (train)                                                                                                    \
       bnBwdSmall<RR, true, BS><<<g.C, BS, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),               \
                                                   dataOrNull(gradBias_), dataOrNull(weight_), meanSrc, stdSrc,    \
-                                                  g.N, g.C, g.L, dev::magicOf(g.L), (float)scale, (float)eps);    \
+                                                  g.N, g.C, g.L, dev::magicOf(g.L), (float)scale, (float)eps, rm); \
     else                                                                                                          \
       bnBwdSmall<RR, false, BS><<<g.C, BS, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_),              \
                                                    dataOrNull(gradBias_), dataOrNull(weight_), meanSrc, stdSrc,   \
-                                                   g.N, g.C, g.L, dev::magicOf(g.L), (float)scale, (float)eps);   \
+                                                   g.N, g.C, g.L, dev::magicOf(g.L), (float)scale, (float)eps, rm); \
   }
     BN_BWD_SMALL(4, kSmallBlock) BN_BWD_SMALL(8, kSmallBlock) BN_BWD_SMALL(16, kSmallBlock) BN_BWD_SMALL(32, kSmallBlock)
     BN_BWD_SMALL(16, kResBlock) BN_BWD_SMALL(32, kResBlock)
@@ -976,11 +1019,11 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
     partial = Temp(s, (size_t)g.C * g.chunks * 2 * sizeof(float));
     p = (float *)partial.get();
     if (v.mode == 1)
-      bnGradSumsKernel<1><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g);
+      bnGradSumsKernel<1><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g, rm);
     else if (v.mode == 2)
-      bnGradSumsKernel<2><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g);
+      bnGradSumsKernel<2><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g, rm);
     else
-      bnGradSumsKernel<0><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g);
+      bnGradSumsKernel<0><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g, rm);
     THC_HIP_CHECK(hipGetLastError());
   }
   BnGeom ga = g;
@@ -990,7 +1033,7 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
   const float *w = dataOrNull(weight_);
 #define BN_BWD(TRAIN, VEC)                                                                                   \
   bnBackwardKernel<TRAIN, VEC><<<gridApply, block, 0, s>>>(in.ptr(), go.ptr(), gx, p, gw, gb, w, meanSrc, stdSrc, ga, \
-                                                           (float)scale, (float)eps)
+                                                           (float)scale, (float)eps, rm)
   if (train) {
     if (v.mode == 1)
       BN_BWD(true, 1);
@@ -1008,6 +1051,57 @@ void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_,
   }
 #undef BN_BWD
   THC_HIP_CHECK(hipGetLastError());
+}
+
+}  // namespace
+
+extern "C" {
+
+void THNN_CudaBatchNormalization_updateOutput(THCState *state, THCudaTensor *input_, THCudaTensor *output_,
+                                              THCudaTensor *weight_, THCudaTensor *bias_,
+                                              THCudaTensor *runningMean_, THCudaTensor *runningVar_,
+                                              THCudaTensor *saveMean_, THCudaTensor *saveStd_, bool train,
+                                              double momentum, double eps) {
+  THNN_ENTER
+  bnUpdateOutput(state, input_, output_, weight_, bias_, runningMean_, runningVar_, saveMean_, saveStd_, train, momentum,
+                 eps, 0);
+  THNN_LEAVE
+}
+
+void THNN_CudaBatchNormalization_backward(THCState *state, THCudaTensor *input_, THCudaTensor *gradOutput_,
+                                          THCudaTensor *gradInput_, THCudaTensor *gradWeight_,
+                                          THCudaTensor *gradBias_, THCudaTensor *weight_,
+                                          THCudaTensor *runningMean_, THCudaTensor *runningVar_,
+                                          THCudaTensor *saveMean_, THCudaTensor *saveStd_, bool train, double scale,
+                                          double eps) {
+  THNN_ENTER
+  bnBackward(state, input_, gradOutput_, gradInput_, gradWeight_, gradBias_, weight_, nullptr, runningMean_, runningVar_,
+             saveMean_, saveStd_, train, scale, eps, 0);
+  THNN_LEAVE
+}
+
+// No counterpart in the reference's C ABI: BatchNormalization followed by Threshold(0, 0) - the conv -> BN -> ReLU
+// step of a residual or depthwise block - in one pass over the tensor (include/THCUNN_fused.h).
+void THNN_CudaBatchNormalizationReLU_updateOutput(THCState *state, THCudaTensor *input_, THCudaTensor *output_,
+                                                  THCudaTensor *weight_, THCudaTensor *bias_,
+                                                  THCudaTensor *runningMean_, THCudaTensor *runningVar_,
+                                                  THCudaTensor *saveMean_, THCudaTensor *saveStd_, bool train,
+                                                  double momentum, double eps) {
+  THNN_ENTER
+  bnUpdateOutput(state, input_, output_, weight_, bias_, runningMean_, runningVar_, saveMean_, saveStd_, train, momentum,
+                 eps, 1);
+  THNN_LEAVE
+}
+
+void THNN_CudaBatchNormalizationReLU_backward(THCState *state, THCudaTensor *input_, THCudaTensor *gradOutput_,
+                                              THCudaTensor *gradInput_, THCudaTensor *gradWeight_,
+                                              THCudaTensor *gradBias_, THCudaTensor *weight_, THCudaTensor *bias_,
+                                              THCudaTensor *runningMean_, THCudaTensor *runningVar_,
+                                              THCudaTensor *saveMean_, THCudaTensor *saveStd_, bool train,
+                                              double scale, double eps) {
+  THNN_ENTER
+  bnBackward(state, input_, gradOutput_, gradInput_, gradWeight_, gradBias_, weight_, bias_, runningMean_, runningVar_,
+             saveMean_, saveStd_, train, scale, eps, 1);
   THNN_LEAVE
 }
 

@@ -19,7 +19,8 @@ def _declared(header):
 def test_library_exports_every_declared_symbol():
     from cunn_amd import _lib
     lib = _lib.load()
-    declared = _declared("THCUNN.h") + _declared("THCShim.h")
+    declared = _declared("THCUNN.h") + _declared("THCShim.h") + _declared("THCUNN_fused.h")
+    assert len(_declared("THCUNN_fused.h")) == 2   # BatchNormalization + ReLU, forward and backward
     # 14 hot-path + 9 dilated / transposed convolution + 2 Threshold + the no-allocation accGradParameters variant
     assert len(_declared("THCUNN.h")) == 26
     # the test hooks: the two column kernels and the kernel-family switch
@@ -33,7 +34,7 @@ def test_entry_point_names_follow_the_reference_binder():
     from cunn_amd import _lib
     assert sorted(_lib.ENTRY_POINTS) == sorted(_lib.SIGNATURES)
     assert sorted("THNN_Cuda" + n for n in _lib.ENTRY_POINTS) == \
-        [n for n in _declared("THCUNN.h") if n.startswith("THNN_Cuda")]
+        sorted(n for n in _declared("THCUNN.h") + _declared("THCUNN_fused.h") if n.startswith("THNN_Cuda"))
 
 
 def test_struct_layout_matches_cutorch_field_order(tmp_path):

@@ -153,7 +153,7 @@ class Contiguous {
 // Several kernel families compute the same results; the parity tests force each of them. The switches take
 // their initial values from the environment once, when the library is loaded (THCUNN_DW_FORCE_DIRECT,
 // THCUNN_DW_SMALL, THCUNN_POOL_FORCE_DIRECT, THCUNN_POOL_RUNS, THCUNN_BN_FORCE_CHUNKED,
-// THCUNN_CONV_FORCE_GENERIC, THCUNN_CONV_GRADINPUT), and change afterwards only through THCUNN_setSwitch:
+// THCUNN_CONV_FORCE_GENERIC, THCUNN_CONV_GRADINPUT, THCUNN_CONV_POINTWISE), and change afterwards only through THCUNN_setSwitch:
 // an entry point reads a plain int, never the environment.
 struct Switches {
   int dwForce = 0;        // 1: shape-agnostic direct kernels, 2: generic LDS-tiled kernels
@@ -163,6 +163,7 @@ struct Switches {
   int bnChunked = 0;      // 1: the chunked two-pass kernels also where a channel fits one workgroup
   int convGeneric = 0;    // 1: first-generation convolution kernels
   int convGradInput = 0;  // 1: phase route, 2: gradient-column route, 0: by shape
+  int convPointwise = 1;  // 0: never the weight-stationary 1x1 kernel; n > 1: at most n workgroups per row block
 };
 extern Switches g_switches;
 

@@ -56,6 +56,7 @@ static int switchValue(const char *name, const char *v, bool *known) {
   *known = true;
   if (!strcmp(name, "THCUNN_CONV_GRADINPUT")) return !v ? 0 : !strcmp(v, "phases") ? 1 : !strcmp(v, "columns") ? 2 : 0;
   if (!strcmp(name, "THCUNN_DW_SMALL") || !strcmp(name, "THCUNN_POOL_RUNS")) return v ? atoi(v) : -1;
+  if (!strcmp(name, "THCUNN_CONV_POINTWISE")) return v ? atoi(v) : 1;
   if (!strcmp(name, "THCUNN_DW_FORCE_DIRECT") || !strcmp(name, "THCUNN_POOL_FORCE_DIRECT") ||
       !strcmp(name, "THCUNN_BN_FORCE_CHUNKED") || !strcmp(name, "THCUNN_CONV_FORCE_GENERIC"))
     return v ? atoi(v) : 0;
@@ -70,12 +71,14 @@ static int *switchSlot(Switches &s, const char *name) {
   if (!strcmp(name, "THCUNN_BN_FORCE_CHUNKED")) return &s.bnChunked;
   if (!strcmp(name, "THCUNN_CONV_FORCE_GENERIC")) return &s.convGeneric;
   if (!strcmp(name, "THCUNN_CONV_GRADINPUT")) return &s.convGradInput;
+  if (!strcmp(name, "THCUNN_CONV_POINTWISE")) return &s.convPointwise;
   return nullptr;
 }
 static Switches switchesFromEnvironment() {
   Switches s;
   for (const char *name : {"THCUNN_DW_FORCE_DIRECT", "THCUNN_DW_SMALL", "THCUNN_POOL_FORCE_DIRECT", "THCUNN_POOL_RUNS",
-                           "THCUNN_BN_FORCE_CHUNKED", "THCUNN_CONV_FORCE_GENERIC", "THCUNN_CONV_GRADINPUT"}) {
+                           "THCUNN_BN_FORCE_CHUNKED", "THCUNN_CONV_FORCE_GENERIC", "THCUNN_CONV_GRADINPUT",
+                           "THCUNN_CONV_POINTWISE"}) {
     bool known;
     *switchSlot(s, name) = switchValue(name, getenv(name), &known);
   }

@@ -278,10 +278,11 @@ def wl_pool(nsets, odd=False):
                      f"N={N} C={Cc} {H}x{H}->{oM}x{oM} / {oA}x{oA}")
 
 
-def wl_conv(nsets):
+def wl_conv(nsets, pointwise=False):
     from cunn_amd import CudaTensor as CT, THNN
     from oracle import oracle as O
-    N, Ci, Co, H, k = 64, 256, 256, 28, 3
+    # pointwise: the 1x1 convolution behind the metric's depthwise layer in MobileNet-v1 (128 -> 128 at 56 x 56)
+    N, Ci, Co, H, k = (64, 128, 128, 56, 1) if pointwise else (64, 256, 256, 28, 3)
     K = Ci * k * k
     rng = np.random.default_rng(4)
     x = rng.standard_normal((N, Ci, H, H)).astype(np.float32)
@@ -292,7 +293,7 @@ def wl_conv(nsets):
     for _ in range(nsets):
         sets.append(dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), gx=CT(), w=CT.from_numpy(w), b=CT.from_numpy(b),
                          gw=CT.from_numpy(np.zeros_like(w)), gb=CT.from_numpy(np.zeros_like(b)), cols=CT(), gcols=CT(), ones=CT()))
-    g = (k, k, 1, 1, 1, 1)
+    g = (k, k, 1, 1, k // 2, k // 2)
 
     def calls(i):
         t = sets[i]
@@ -310,7 +311,7 @@ def wl_conv(nsets):
             O.convmm_updateOutput(x[:ns], w, b, *g)
             O.convmm_updateGradInput((ns,) + x.shape[1:], gy[:ns], w, *g)
             O.convmm_accGradParameters(x[:ns], gy[:ns], np.zeros_like(w), np.zeros_like(b), *g, 1.0)
-        return time.perf_counter() - t0, reps * ns, f"{reps} passes over the first {ns} of {N} images of cfg5"
+        return time.perf_counter() - t0, reps * ns, f"{reps} passes over the first {ns} of {N} images"
 
     def verify():
         t = sets[0]
@@ -322,7 +323,7 @@ def wl_conv(nsets):
         t["gw"].fill(0.0), t["gb"].fill(0.0)
 
     return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="mfma",
-                desc=f"SpatialConvolutionMM fwd+gradInput+accGradParameters fp32 N={N} Cin={Ci} Cout={Co} {H}x{H} k3 s1 p1 bias")
+                desc=f"SpatialConvolutionMM fwd+gradInput+accGradParameters fp32 N={N} Cin={Ci} Cout={Co} {H}x{H} k{k} s1 p{k // 2} bias")
 
 
 def wl_dilconv(nsets):
@@ -536,7 +537,7 @@ def wl_copy(nsets):
 
 WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda n: wl_dw("cfg2", n), "cfg3": wl_bn, "cfg4": wl_pool,
              "dw147": lambda n: wl_dw("dw147", n), "dw14": lambda n: wl_dw("dw14", n), "pool71": lambda n: wl_pool(n, odd=True),
-             "cfg5": wl_conv, "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu,
+             "cfg5": wl_conv, "pw128": lambda n: wl_conv(n, pointwise=True), "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu,
              "bnrelu": wl_bnrelu, "bnrelu_unfused": lambda n: wl_bnrelu(n, fused=False)}
 
 

@@ -149,7 +149,7 @@ void THNN_Cuda_col2im(THCState *state, const float *col, int nImages, int channe
                       int kH, int kW, int padH, int padW, int dH, int dW, int dilH, int dilW, float *im);
 /* Several kernel families compute the same results; this forces one. `name` is one of THCUNN_DW_FORCE_DIRECT,
  * THCUNN_DW_SMALL, THCUNN_POOL_FORCE_DIRECT, THCUNN_POOL_RUNS, THCUNN_BN_FORCE_CHUNKED, THCUNN_CONV_FORCE_GENERIC,
- * THCUNN_CONV_GRADINPUT; `value` is what the environment variable of that name would hold (read once, when the
+ * THCUNN_CONV_GRADINPUT, THCUNN_CONV_POINTWISE; `value` is what the environment variable of that name would hold (read once, when the
  * library is loaded), NULL restores the choice by shape. Returns 0 for an unknown name. Not thread-safe
  * against concurrent calls of the entry points. */
 int THCUNN_setSwitch(const char *name, const char *value);

@@ -1375,6 +1375,7 @@ col2imKernel(const float *__restrict__ col, float *__restrict__ im, int nImg, in
 }
 
 #include "conv_pointwise.h"
+#include "conv_fewplanes.h"
 
 // ---- host side -----------------------------------------------------------------
 struct ConvCall {
@@ -1938,6 +1939,90 @@ bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const
   return true;
 }
 
+// ---- gradInput with one to four input planes (conv_fewplanes.h) ----
+template <int S, int T, int KC, int PADC>
+void launchFewPlanes(hipStream_t s, FpArgs a, const FpTaps &tp, const ConvGeom &g) {
+  using Sh = FpShape<S, T, KC, PADC>;
+  const int PR = (g.H + S - 1) / S, PC = (g.W + S - 1) / S;  // phase positions per image
+  a.tilesR = (int)tiles(PR, 4 * T), a.tilesC = (int)tiles(PC, 16);
+  a.magicTiles = dev::magicOf(a.tilesR * a.tilesC), a.magicTilesC = dev::magicOf(a.tilesC);
+  const int RR = Sh::CT ? Sh::RR : a.RR;
+  const int KKP = (g.kH * g.kW + 3) / 4 * 4;
+  convFewPlanesGradInputKernel<S, T, KC, PADC>
+      <<<g.N * a.tilesR * a.tilesC, 64 * kFpWaves, Sh::ldsBytes(RR, KKP), s>>>(a, tp);
+  THC_HIP_CHECK(hipGetLastError());
+}
+
+// false: not a shape for this kernel (the caller goes on to the other routes)
+bool convFewPlanesGradInput(THCState *state, const ConvGeom &g, const float *gy, const float *w, float *gi,
+                            const float *bias, bool runtimeOnly) {
+  const int S = g.dH;
+  if (g.Cin > 4 || g.dilH != 1 || g.dilW != 1 || g.dH != g.dW || S > 4 || g.padH < 0 || g.padW < 0) return false;
+  if ((long)g.Cout * g.L * 4 >= (1L << 31) || (long)g.Cin * g.H * g.W * 4 >= (1L << 31)) return false;
+  FpArgs a{};
+  FpTaps tp{};
+  a.gy = gy, a.w = w, a.bias = bias, a.gi = gi;
+  a.Cin = g.Cin, a.Cout = g.Cout, a.H = g.H, a.W = g.W, a.oH = g.oH, a.oW = g.oW, a.kH = g.kH, a.kW = g.kW;
+  a.magicCK = dev::magicOf(g.Cin * g.kH * g.kW), a.magicKK = dev::magicOf(g.kH * g.kW);
+  const int PR = (g.H + S - 1) / S, PC = (g.W + S - 1) / S;
+  const int Tg = S <= 2 ? 4 : S == 3 ? 2 : 1;  // rows per lane of the run-time variant
+  {  // block numbering: n * tiles + tile must divide back exactly
+    const long tl = tiles(PR, 4) * tiles(PC, 16);  // at most this many blocks per image (T >= 1)
+    if ((long)g.N * tl >= (1L << 31) || (double)g.N * tl * tl >= 4294967296.0) return false;
+  }
+  hipStream_t s = state->stream;
+  const bool square = g.kH == g.kW && g.padH == g.padW;
+  const int k = g.kH, pad = g.padH;
+  if (square && !runtimeOnly) {
+#define FEW_PLANES_SHAPE(S_, T_, K_, P_)                  \
+  if (S == S_ && k == K_ && pad == P_) {                  \
+    launchFewPlanes<S_, T_, K_, P_>(s, a, tp, g);         \
+    return true;                                          \
+  }
+    FEW_PLANES_SHAPE(2, 4, 7, 3)   // 7x7 stride 2: the first layer of ResNet / Inception-v1
+    FEW_PLANES_SHAPE(2, 4, 3, 1)   // 3x3 stride 2: MobileNet
+    FEW_PLANES_SHAPE(2, 4, 3, 0)   // 3x3 stride 2, unpadded: Inception-v3
+    FEW_PLANES_SHAPE(1, 8, 3, 1)   // 3x3: VGG
+    FEW_PLANES_SHAPE(1, 8, 5, 2)   // 5x5
+    FEW_PLANES_SHAPE(2, 4, 4, 1)   // 4x4 stride 2: the transposed convolutions of a generator
+    FEW_PLANES_SHAPE(4, 2, 11, 2)  // 11x11 stride 4: AlexNet
+#undef FEW_PLANES_SHAPE
+  }
+  // any other kernel size / padding: tap loops with run-time bounds
+  if (g.kH * g.kW > kFpMaxTaps) return false;
+  auto fill = [&](FpDim &d, int kk, int pd) {
+    d.lo = fpLo(pd, S, kk), d.hi = fpHi(pd, S, kk);
+    for (int ph = 0; ph < S; ++ph) d.rem[ph] = fpRem(ph, pd, S), d.q0[ph] = fpQ0(ph, pd, S), d.taps[ph] = fpTaps(ph, pd, S, kk);
+  };
+  fill(a.dh, g.kH, g.padH);
+  fill(a.dw, g.kW, g.padW);
+  a.RR = 4 * Tg + a.dh.hi - a.dh.lo, a.CC = 16 + a.dw.hi - a.dw.lo;
+  a.magicCC = dev::magicOf(a.CC);
+  const int pitch = Tg == 4 ? 28 : Tg == 2 ? 24 : 48;
+  if (a.CC > pitch || a.RR * a.CC > 64 * kFpMaxLoads || 2 * g.Cin * g.kH * g.kW > 64 * kFpMaxWLoads ||
+      a.RR * pitch >= 65536)
+    return false;
+  int cnt = 0;
+  for (int ph = 0; ph < S; ++ph)
+    for (int pw = 0; pw < S; ++pw) {
+      tp.first[ph * S + pw] = cnt;
+      for (int ta = 0; ta < a.dh.taps[ph]; ++ta)
+        for (int tb = 0; tb < a.dw.taps[pw]; ++tb) {
+          const unsigned tap = (a.dh.rem[ph] + ta * S) * g.kW + a.dw.rem[pw] + tb * S;
+          const unsigned off = (a.dh.q0[ph] - ta - a.dh.lo) * pitch + (a.dw.q0[pw] - tb - a.dw.lo);
+          tp.e[cnt++] = tap | off << 16;
+        }
+    }
+  for (int q = S * S; q <= 16; ++q) tp.first[q] = cnt;
+  switch (S) {
+    case 1: launchFewPlanes<1, 4, 0, 0>(s, a, tp, g); break;
+    case 2: launchFewPlanes<2, 4, 0, 0>(s, a, tp, g); break;
+    case 3: launchFewPlanes<3, 2, 0, 0>(s, a, tp, g); break;
+    default: launchFewPlanes<4, 1, 0, 0>(s, a, tp, g); break;
+  }
+  return true;
+}
+
 // gi(N, Cin, H, W) = conv^T(gy(N, Cout, oH, oW), w(Cout, K))
 // + bias[c] per plane of gi when bias != null (the transposed convolution's forward pass)
 void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const float *w, float *gi,
@@ -1954,6 +2039,10 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
   // (one to four input planes - the first layer of a network - would fill a sixteenth of the 64-row tiles of that
   // GEMM: 1.08 ms for 3 -> 64 planes 3x3 at 224x224, N = 32; the column GEMM below has K = Cin * kH * kW rows)
   const bool sliver = g.Cin <= 4 && g.kH * g.kW > 1;
+  const int route = g_switches.convGradInput;  // 1: phases, 2: columns, 3: few-plane kernel with run-time tap loops
+  if (g.Cin <= 4 && (g.kH * g.kW > 1 || g.dH > 1 || g.dW > 1) && !forceGeneric() && (route == 0 || route == 3) &&
+      convFewPlanesGradInput(state, g, gy, w, gi, bias, route == 3))
+    return;
   if (g.dH == 1 && g.dW == 1 && tpH >= 0 && tpW >= 0 && exact && !sliver && !forceGeneric() && goImgBytes < (1L << 30) &&
       (long)g.Cout * g.K < 0x7fffffffL / 4) {
     ConvGeom t = g;  // the transposed problem
@@ -1984,7 +2073,6 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
   }
   // With few input planes the phase GEMMs would use a sliver of their 64-row tiles; the column GEMM
   // (K rows) is the better shape then. Test switch THCUNN_CONV_GRADINPUT = "phases" / "columns" overrides.
-  const int route = g_switches.convGradInput;  // 1: phases, 2: columns
   const bool phasesPay = 2L * g.Cin >= (long)tiles(g.Cin, 64) * 64;
   const bool tryPhases = route == 1 ? true : route == 2 ? false : phasesPay;
   if (!forceGeneric() && tryPhases && gradInputByPhase(state, g, gy, w, gi, scratchBuf, bufName, bias)) return;

@@ -162,7 +162,7 @@ struct Switches {
   int poolRuns = -1;      // as dwSmall
   int bnChunked = 0;      // 1: the chunked two-pass kernels also where a channel fits one workgroup
   int convGeneric = 0;    // 1: first-generation convolution kernels
-  int convGradInput = 0;  // 1: phase route, 2: gradient-column route, 0: by shape
+  int convGradInput = 0;  // 1: phase route, 2: gradient-column route, 3: few-plane kernel with run-time tap loops, 0: by shape
   int convPointwise = 1;  // 0: never the weight-stationary 1x1 kernel; n > 1: at most n workgroups per row block
 };
 extern Switches g_switches;

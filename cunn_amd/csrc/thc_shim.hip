@@ -54,7 +54,7 @@ void dispatchError(const Error &e) {
 // -------------------------------------------------------------- switches ----
 static int switchValue(const char *name, const char *v, bool *known) {
   *known = true;
-  if (!strcmp(name, "THCUNN_CONV_GRADINPUT")) return !v ? 0 : !strcmp(v, "phases") ? 1 : !strcmp(v, "columns") ? 2 : 0;
+  if (!strcmp(name, "THCUNN_CONV_GRADINPUT")) return !v ? 0 : !strcmp(v, "phases") ? 1 : !strcmp(v, "columns") ? 2 : !strcmp(v, "planes") ? 3 : 0;
   if (!strcmp(name, "THCUNN_DW_SMALL") || !strcmp(name, "THCUNN_POOL_RUNS")) return v ? atoi(v) : -1;
   if (!strcmp(name, "THCUNN_CONV_POINTWISE")) return v ? atoi(v) : 1;
   if (!strcmp(name, "THCUNN_DW_FORCE_DIRECT") || !strcmp(name, "THCUNN_POOL_FORCE_DIRECT") ||

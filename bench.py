@@ -278,22 +278,24 @@ def wl_pool(nsets, odd=False):
                      f"N={N} C={Cc} {H}x{H}->{oM}x{oM} / {oA}x{oA}")
 
 
-def wl_conv(nsets, pointwise=False):
+def wl_conv(nsets, pointwise=False, first=False):
     from cunn_amd import CudaTensor as CT, THNN
     from oracle import oracle as O
     # pointwise: the 1x1 convolution behind the metric's depthwise layer in MobileNet-v1 (128 -> 128 at 56 x 56)
-    N, Ci, Co, H, k = (64, 128, 128, 56, 1) if pointwise else (64, 256, 256, 28, 3)
+    # first: the first layer of ResNet (3 -> 64 planes, 7x7 stride 2 at 224 x 224)
+    N, Ci, Co, H, k, st = (64, 128, 128, 56, 1, 1) if pointwise else (32, 3, 64, 224, 7, 2) if first else (64, 256, 256, 28, 3, 1)
     K = Ci * k * k
+    oH = (H + 2 * (k // 2) - k) // st + 1
     rng = np.random.default_rng(4)
     x = rng.standard_normal((N, Ci, H, H)).astype(np.float32)
-    gy = rng.standard_normal((N, Co, H, H)).astype(np.float32)
+    gy = rng.standard_normal((N, Co, oH, oH)).astype(np.float32)
     w = (rng.standard_normal((Co, K)) * np.sqrt(2.0 / K)).astype(np.float32)
     b = rng.uniform(-0.02, 0.02, Co).astype(np.float32)
     sets = []
     for _ in range(nsets):
         sets.append(dict(x=CT.from_numpy(x), gy=CT.from_numpy(gy), y=CT(), gx=CT(), w=CT.from_numpy(w), b=CT.from_numpy(b),
                          gw=CT.from_numpy(np.zeros_like(w)), gb=CT.from_numpy(np.zeros_like(b)), cols=CT(), gcols=CT(), ones=CT()))
-    g = (k, k, 1, 1, k // 2, k // 2)
+    g = (k, k, st, st, k // 2, k // 2)
 
     def calls(i):
         t = sets[i]
@@ -301,7 +303,7 @@ def wl_conv(nsets, pointwise=False):
                 ("convmm_updateGradInput", lambda: THNN.SpatialConvolutionMM_updateGradInput(t["x"], t["gy"], t["gx"], t["w"], t["gcols"], t["ones"], *g)),
                 ("convmm_accGradParameters", lambda: THNN.SpatialConvolutionMM_accGradParameters(t["x"], t["gy"], t["gw"], t["gb"], t["cols"], t["ones"], *g, 1.0))]
 
-    fl = 2.0 * Co * K * H * H * N
+    fl = 2.0 * Co * K * oH * oH * N
     work = {"convmm_updateOutput": (fl, "flops"), "convmm_updateGradInput": (fl, "flops"), "convmm_accGradParameters": (fl, "flops")}
     ns = 4  # images of the CPU sample
 
@@ -323,7 +325,7 @@ def wl_conv(nsets, pointwise=False):
         t["gw"].fill(0.0), t["gb"].fill(0.0)
 
     return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="mfma",
-                desc=f"SpatialConvolutionMM fwd+gradInput+accGradParameters fp32 N={N} Cin={Ci} Cout={Co} {H}x{H} k{k} s1 p{k // 2} bias")
+                desc=f"SpatialConvolutionMM fwd+gradInput+accGradParameters fp32 N={N} Cin={Ci} Cout={Co} {H}x{H} k{k} s{st} p{k // 2} bias")
 
 
 def wl_dilconv(nsets):
@@ -537,7 +539,7 @@ def wl_copy(nsets):
 
 WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda n: wl_dw("cfg2", n), "cfg3": wl_bn, "cfg4": wl_pool,
              "dw147": lambda n: wl_dw("dw147", n), "dw14": lambda n: wl_dw("dw14", n), "pool71": lambda n: wl_pool(n, odd=True),
-             "cfg5": wl_conv, "pw128": lambda n: wl_conv(n, pointwise=True), "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu,
+             "cfg5": wl_conv, "pw128": lambda n: wl_conv(n, pointwise=True), "conv1": lambda n: wl_conv(n, first=True), "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu,
              "bnrelu": wl_bnrelu, "bnrelu_unfused": lambda n: wl_bnrelu(n, fused=False)}
 
 

@@ -95,7 +95,7 @@ struct FpShape {
   static constexpr int NLW = CT ? (OC * 4 * KK + 63) / 64 : kFpMaxWLoads;
   static constexpr int NQ = T * S * S;  // accumulators per lane
   // floats of LDS a wave parks its chunk in
-  __host__ __device__ static constexpr int priv(int rr, int kkp) { return OC * rr * PITCH + OC * 4 * kkp; }
+  __host__ __device__ static constexpr int priv(int rr, int kkp) { return OC * rr * PITCH + OC * 4 * kkp + 64; }
   __host__ __device__ static constexpr size_t ldsBytes(int rr, int kkp) {
     const size_t a = (size_t)kFpWaves * priv(rr, kkp), b = (size_t)kFpWaves * (NQ < kFpRedQ ? NQ : kFpRedQ) * 256;
     return (a > b ? a : b) * sizeof(float);
@@ -117,7 +117,7 @@ convFewPlanesGradInputKernel(FpArgs p, FpTaps tp) {
   const int loH = CT ? Sh::LO : p.dh.lo, loW = CT ? Sh::LO : p.dw.lo;
   const int plane = RR * PITCH;                 // floats per parked output plane
   const int wBase = OC * plane;                 // where the weights start
-  float *lds = ldsAll + wave * Sh::priv(RR, KKP);  // patch[OC][RR][PITCH], weights[OC][4][KKP]
+  float *lds = ldsAll + wave * Sh::priv(RR, KKP);  // patch[OC][RR][PITCH], weights[OC][4][KKP], 64 spare
 
   int item = dev::xcdRemap(blockIdx.x, gridDim.x);
   const int n = dev::fastDiv(item, p.magicTiles);
@@ -142,6 +142,17 @@ convFewPlanesGradInputKernel(FpArgs p, FpTaps tp) {
     lOff[k] = inPatch ? rr * PITCH + cc : -1;
   }
   const int nlg = CT ? NLG : (RR * CC + 63) / 64;
+  // element e = lane + 64 k of a chunk's weights is (o, c, tap) = (e / (Cin KK), ...): it goes to weights[o][c][tap];
+  // elements past the chunk (the loads cover OC * 4 * KK) go to the lane's spare slot
+  const int nlw = CT ? NLW : (OC * p.Cin * KK + 63) / 64;
+  int wOff[NLW];
+#pragma unroll
+  for (int k = 0; k < NLW; ++k) {
+    const int e = lane + 64 * k;
+    const int o_ = dev::fastDiv(e, p.magicCK), rem = e - o_ * p.Cin * KK;
+    const int c = dev::fastDiv(rem, p.magicKK), tap = rem - c * KK;
+    wOff[k] = o_ < OC ? wBase + (o_ * 4 + c) * KKP + tap : wBase + OC * 4 * KKP + lane;
+  }
 
   // The output planes go to the waves in groups of 4 (group g to wave g mod 4), a group in chunks of OC:
   // chunk number ci of this wave starts at plane
@@ -158,13 +169,11 @@ convFewPlanesGradInputKernel(FpArgs p, FpTaps tp) {
         for (int k = 0; k < NLG; ++k)
           if (CT || k < nlg) gv[o][k] = __builtin_amdgcn_raw_buffer_load_b32(gyr, gOff[k], (o0 + o) * gyPlaneBytes, 0);
       }
-    const float *wsrc = p.w + (long)o0 * p.Cin * KK;
-    const int cnt = oc * p.Cin * KK;
+    // the weights of the chunk are contiguous; what lies past the end of the matrix reads as 0
+    const __amdgpu_buffer_rsrc_t wr = dev::makeRsrc(p.w + (long)o0 * p.Cin * KK, (long)(p.Cout - o0) * p.Cin * KK * 4);
 #pragma unroll
-    for (int k = 0; k < NLW; ++k) {
-      const int e = lane + 64 * k;
-      if (e < cnt) wv[k] = wsrc[e];
-    }
+    for (int k = 0; k < NLW; ++k)
+      if (CT || k < nlw) wv[k] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(wr, lane * 4 + 256 * k, 0, 0));
   };
   auto park = [&](int o0) {  // registers -> LDS
     const int oc = min(OC, p.Cout - o0);
@@ -176,16 +185,9 @@ convFewPlanesGradInputKernel(FpArgs p, FpTaps tp) {
           if (CT ? (64 * (k + 1) <= Sh::RR * Sh::CC || lOff[k] >= 0) : (k < nlg && lOff[k] >= 0))
             lds[o * plane + lOff[k]] = __uint_as_float(gv[o][k]);
       }
-    const int cnt = oc * p.Cin * KK;
 #pragma unroll
-    for (int k = 0; k < NLW; ++k) {
-      const int e = lane + 64 * k;
-      if (e < cnt) {
-        const int oc_ = dev::fastDiv(e, p.magicCK), rem = e - oc_ * p.Cin * KK;  // (o, c * KK + tap)
-        const int c = dev::fastDiv(rem, p.magicKK), tap = rem - c * KK;
-        lds[wBase + (oc_ * 4 + c) * KKP + tap] = wv[k];
-      }
-    }
+    for (int k = 0; k < NLW; ++k)
+      if (CT || k < nlw) lds[wOff[k]] = wv[k];
   };
 
   float4v acc[T][S][S];
@@ -199,10 +201,18 @@ convFewPlanesGradInputKernel(FpArgs p, FpTaps tp) {
   const int laneB = lr * T * PITCH + lc;  // the lane's corner of the parked patch
   const int laneA = wBase + cA * KKP;     // the lane's plane of the weights
 
+  float bias[4] = {0.f, 0.f, 0.f, 0.f};  // fetched now: a load next to the stores would make every store wait for the one before
+  if (p.bias) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      if (c < p.Cin) bias[c] = p.bias[c];
+  }
+  __builtin_amdgcn_s_setprio(2);  // setting up and winding down go ahead of the other waves' multiplications
   if (firstPlane(0) < p.Cout) fetch(firstPlane(0));
   for (int ci = 0; firstPlane(ci) < p.Cout; ++ci) {
     const int o0 = firstPlane(ci);
     const int oc = min(OC, p.Cout - o0);
+    __builtin_amdgcn_s_setprio(2);
     // the reads of the chunk before are done (their values went into MFMAs already issued); LDS runs a wave's
     // accesses in order, so the wave needs no barrier with itself - only the compiler must keep the order
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -211,6 +221,7 @@ convFewPlanesGradInputKernel(FpArgs p, FpTaps tp) {
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
     if (firstPlane(ci + 1) < p.Cout) fetch(firstPlane(ci + 1));
+    __builtin_amdgcn_s_setprio(0);
 
     for (int o = 0; o < oc; ++o) {
       const float *gp = lds + o * plane + laneB;
@@ -284,12 +295,7 @@ convFewPlanesGradInputKernel(FpArgs p, FpTaps tp) {
   const long giImg = (long)p.Cin * p.H * p.W;
   const __amdgpu_buffer_rsrc_t gir = dev::makeRsrc(p.gi + n * giImg, giImg * 4);
   const int giPlaneBytes = p.H * p.W * 4;
-  float bias[4] = {0.f, 0.f, 0.f, 0.f};
-  if (p.bias) {
-#pragma unroll
-    for (int c = 0; c < 4; ++c)
-      if (c < p.Cin) bias[c] = p.bias[c];
-  }
+  __builtin_amdgcn_s_setprio(2);
   constexpr int QB = NQ < kFpRedQ ? NQ : kFpRedQ;
   float4v *red = reinterpret_cast<float4v *>(ldsAll);  // [wave][QB][64 lanes]
 #pragma unroll
@@ -308,8 +314,9 @@ convFewPlanesGradInputKernel(FpArgs p, FpTaps tp) {
       const int h = S * (I0 + lr * T + t) + ph, w = S * (J0 + lc) + pw;
       const int off = (h < p.H && w < p.W) ? (h * p.W + w) * 4 : dev::kBufOob;
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        if (c < p.Cin) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[c] + bias[c]), gir, off, c * giPlaneBytes, 0);
+      for (int c = 0; c < 4; ++c)  // a plane that does not exist is an offset out of range: no branch between the stores
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[c] + bias[c]), gir, c < p.Cin ? off : dev::kBufOob,
+                                              c < p.Cin ? c * giPlaneBytes : 0, 0);
     }
   }
 }

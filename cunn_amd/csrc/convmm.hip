@@ -1958,7 +1958,8 @@ bool convFewPlanesGradInput(THCState *state, const ConvGeom &g, const float *gy,
                             const float *bias, bool runtimeOnly) {
   const int S = g.dH;
   if (g.Cin > 4 || g.dilH != 1 || g.dilW != 1 || g.dH != g.dW || S > 4 || g.padH < 0 || g.padW < 0) return false;
-  if ((long)g.Cout * g.L * 4 >= (1L << 31) || (long)g.Cin * g.H * g.W * 4 >= (1L << 31)) return false;
+  if ((long)g.Cout * g.L * 4 >= (1L << 31) || (long)g.Cin * g.H * g.W * 4 >= (1L << 31) || (long)g.Cout * g.K * 4 >= (1L << 31))
+    return false;
   FpArgs a{};
   FpTaps tp{};
   a.gy = gy, a.w = w, a.bias = bias, a.gi = gi;

@@ -1501,23 +1501,32 @@ void planTiles(FwdPlan &pl, int M, long Ncols, int nkt, bool wideOk) {
   pl.mTiles = (int)tiles(M, pl.bm);
   pl.total = pl.mTiles * (int)tiles(Ncols, pl.bn);
   const int cus = residentSlots(nullptr);
+  // Which tiles to split along K, and how finely: the workgroups go to the CUs in launch order (up to three
+  // share a CU), so a CU's time is the sum over what it is dealt. In units of one k-tile of one workgroup alone
+  // on its CU: a workgroup costs its k-tiles + 4 (prologue, epilogue), a split tile 0.006 more per partial
+  // (written, then read by the fold), and a CU that only ever holds one workgroup runs at 0.85 of the rate
+  // (nothing covers its barriers) - constants fitted to measured sweeps over S on 14x14 ... 56x56 layers.
+  // Candidates: no split; the last, partial round split S ways; every tile split S ways (S <= 16, >= 4 k-tiles
+  // per split). E.g. 196 tiles on 256 CUs: 5 splits (980 workgroups, 4 per CU at most) beat 2 (392: 136 CUs
+  // carry two halves, 120 one) by 15 %; 136 tiles left over after a full round: 3 splits, not 1.
+  const int maxS = std::max(1, std::min(nkt / 4, 16));
+  const int q = pl.total / cus, r = pl.total % cus;
+  auto perWg = [&](int S) { return (double)launch::ceilDiv(nkt, S) + 4.0; };
+  // a split has to promise 5 % before it is taken: the model is coarse and the fold is one more launch
+  double best = 0.95 * launch::ceilDiv(pl.total, cus) * perWg(1) / (pl.total <= cus ? 0.85 : 1.0);
   int nSplit = 1;
   pl.tail = 0;
-  if (pl.total > cus) {
-    pl.tail = pl.total % cus;
-    // at most one split per CU, >= 4 k-tiles each (finer splits - ceil(cus / tail) - measured slower: the
-    // partial tiles cost more than the balance gains)
-    if (pl.tail > 0) nSplit = std::min(nkt / 4, cus / pl.tail);
-  } else {
-    // fewer tiles than CUs: every tile is split along K so that the grid occupies the chip
-    pl.tail = pl.total;
-    // (two workgroups per CU measured best on 7x7 and 14x14 layers: each further split is another partial tile
-    // to write and fold)
-    nSplit = std::min(nkt / 4, std::min(residentSlots((const void *)convFwdPaddedKernel<2>), 2 * cus) / pl.total);
-  }
-  if (nSplit < 2) {
-    pl.tail = 0;
-    nSplit = 1;
+  for (int S = 2; S <= maxS; ++S) {
+    if (launch::ceilDiv(nkt, launch::ceilDiv(nkt, S)) != S) continue;  // the same pieces as a smaller S
+    if (q > 0 && r > 0) {
+      const double t = q * perWg(1) + launch::ceilDiv(r * S, cus) * perWg(S) + 0.006 * r * S;
+      if (t < best) best = t, nSplit = S, pl.tail = r;
+    }
+    if (pl.total <= 2 * cus) {
+      const int n = launch::ceilDiv(pl.total * S, cus);
+      const double t = n * perWg(S) / (n == 1 ? 0.85 : 1.0) + 0.006 * pl.total * S;
+      if (t < best) best = t, nSplit = S, pl.tail = pl.total;
+    }
   }
   pl.full = pl.total - pl.tail;
   pl.ktPerSplit = launch::ceilDiv(nkt, nSplit);

@@ -367,8 +367,8 @@ struct FwdArgs {
 // 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 accumulator tile. Split workgroups store their
 // partial tile, the others add the bias and store to out(n, row, l).
 // biasLds: the tile's bias values in LDS (index = row - m0, zeros where there is no bias or row), or null.
-template <int TBN = BN>
-__device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g, const float16v (&acc)[2][2], int bx,
+template <int TBN = BN, int TI = 2>
+__device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g, const float16v (&acc)[TI][2], int bx,
                                             int by, int m0, int j0, int wm, int wn, int grp, int idx,
                                             const float *biasLds = nullptr, int toPartial = -1) {
   const int rowHalf = grp * 4;
@@ -377,7 +377,7 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
 #pragma unroll
     for (int tj = 0; tj < 2; ++tj)
 #pragma unroll
-      for (int ti = 0; ti < 2; ++ti)
+      for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
         for (int v = 0; v < 16; ++v)
           dst[(wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3)) * TBN + wn * 64 + tj * 32 + idx] = acc[ti][tj][v];
@@ -387,10 +387,10 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
     constexpr bool BIAS = decltype(withBias)::value;
     // the lane's 32 bias values first: a load between the stores would wait for each store before it
     // (the compiler must assume that out and bias overlap)
-    float bv[2][16];
+    float bv[TI][16];
     if (BIAS) {
 #pragma unroll
-      for (int ti = 0; ti < 2; ++ti)
+      for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           if (biasLds) {  // 4 consecutive rows: one 16-byte LDS read
@@ -414,7 +414,7 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
       const int oh = l / g.oW, ow = l - oh * g.oW;
       float *dst = p.out + (long)n * p.outImg + (long)oh * p.outSH + ow * p.outSW;
 #pragma unroll
-      for (int ti = 0; ti < 2; ++ti)
+      for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
@@ -735,6 +735,19 @@ __device__ __forceinline__ void mfmaHalf(const float4 *aSrc, const float4 *bSrc,
     acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv1[j], acc[1][1], 0, 0, 0);
   }
 }
+// the same for a wave that multiplies 32 rows: 3 ds_read_b128 and 8 MFMAs
+template <int OA, int OB>
+__device__ __forceinline__ void mfmaHalf(const float4 *aSrc, const float4 *bSrc, float16v (&acc)[1][2]) {
+  const float4 a0 = aSrc[OA];
+  const float4 b0 = bSrc[OB], b1 = bSrc[OB + 32];
+  const float av0[4] = {a0.x, a0.y, a0.z, a0.w};
+  const float bv0[4] = {b0.x, b0.y, b0.z, b0.w}, bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv0[j], acc[0][0], 0, 0, 0);
+    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv1[j], acc[0][1], 0, 0, 0);
+  }
+}
 
 // Forward kernel for images that carry their zero border in memory (padH = padW = 0 in g,
 // K % BK == 0, 16-byte loadable weight rows). On this part every ordinary vector-ALU
@@ -746,14 +759,17 @@ __device__ __forceinline__ void mfmaHalf(const float4 *aSrc, const float4 *bSrc,
 //  * the loop is unrolled over the two LDS buffers, so every LDS address is base + immediate
 // Rows past M and columns past the batch are clamped to valid ones and dropped in the epilogue.
 // WM = 2: 128 x 128 tiles, the four waves as 2 x 2; WM = 1: 64 x 256 tiles, the four waves side by side,
-// for row counts whose last 128-row tile would be at most half full. A wave multiplies 64 x 64 either way.
+// for row counts whose last 128-row tile would be at most half full; a wave multiplies 64 x 64 either way.
+// WM = 0: 32 x 256 tiles, a wave multiplies 32 x 64, for 32 rows or fewer left over (32-plane layers).
 // (bx, by): position among the tiles that start at tile0 and split; whole: the workgroup reduces all of K
 // of tile bx and writes the output itself
 // LINEAR: 1x1 windows - the tap offsets are an arithmetic sequence, computed by the scalar unit instead of
 // read from the table
 template <int WM, bool LINEAR = false>
 __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &g, int bx, int by, bool whole) {
-  constexpr int TBM = 64 * WM, TBN = 256 / WM;
+  constexpr int TBM = WM == 0 ? 32 : 64 * WM, TBN = WM == 2 ? 128 : 256;
+  constexpr int TI = WM == 0 ? 1 : 2;         // 32-row blocks of a wave
+  constexpr int NA = WM == 2 ? 2 : 1;         // 16-byte groups of weights a lane loads per k-tile
   constexpr int AP = TBM + 8, BP = TBN + 8;  // float4 per k-group row
   constexpr int NB = WM == 2 ? 8 : 16;        // image elements a lane gathers per k-tile
   __shared__ float4 As[2][BK / 4][AP];
@@ -766,9 +782,9 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   const int m0 = mTile * TBM, j0 = nTile * TBN;
   if (t < TBM) biasS[t] = p.bias && m0 + t < p.M ? p.bias[m0 + t] : 0.f;  // visible after the first barrier
 
-  float16v acc[2][2];
+  float16v acc[TI][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -776,9 +792,10 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
 
   const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)p.w, 0, p.wBytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.xBytes, 0x00020000);
-  // weights: WM = 2 - a lane loads 8 consecutive k of row t / 2; WM = 1 - 4 consecutive k of row t / 4
-  // image:   WM = 2 - a lane gathers 8 taps of column t % 128; WM = 1 - all 16 taps of column t
-  const int rowA = WM == 2 ? t >> 1 : t >> 2;
+  // weights: WM = 2 - a lane loads 8 consecutive k of row t / 2; WM = 1 - 4 consecutive k of row t / 4;
+  //          WM = 0 - the same of row (t / 4) % 32: both halves of the workgroup fetch and park the same values
+  // image:   WM = 2 - a lane gathers 8 taps of column t % 128; WM < 2 - all 16 taps of column t
+  const int rowA = WM == 2 ? t >> 1 : WM == 1 ? t >> 2 : (t >> 2) & 31;
   const int kgA = WM == 2 ? (t & 1) * 2 : t & 3;
   const int colB = WM == 2 ? t & 127 : t;
   const int kgB = WM == 2 ? (t >> 7) * 2 : 0;
@@ -795,7 +812,7 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   const int ktBegin = by * p.ktPerSplit;  // by == 0 for whole tiles
   const int nkt = whole ? g.K / BK : min(g.K / BK, ktBegin + p.ktPerSplit);  // this workgroup reduces k-tiles [ktBegin, nkt)
 
-  u32x4 ra[WM];
+  u32x4 ra[NA];
   unsigned rb[NB];
   // The tap offsets of a wave and k-tile are fetched with scalar loads one tile ahead of their use,
   // so that no wave waits on the scalar cache inside the loop (the table has spare entries at its end).
@@ -815,7 +832,7 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   auto loadTiles = [&](int kt) {
     const int k0 = __builtin_amdgcn_readfirstlane(kt * BK);
 #pragma unroll
-    for (int i = 0; i < WM; ++i) ra[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, aOff + 16 * i, k0 * 4, 0);
+    for (int i = 0; i < NA; ++i) ra[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, aOff + 16 * i, k0 * 4, 0);
 #pragma unroll
     for (int i = 0; i < NB / 4; ++i) {
       rb[4 * i + 0] = __builtin_amdgcn_raw_buffer_load_b32(xr, posOff, e[i].x, 0);
@@ -830,7 +847,7 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   auto storeTiles = [&](auto bufc) {
     constexpr int b = decltype(bufc)::value;
 #pragma unroll
-    for (int i = 0; i < WM; ++i) aDst[b * BUFA + i * AP] = ra[i];
+    for (int i = 0; i < NA; ++i) aDst[b * BUFA + i * AP] = ra[i];
 #pragma unroll
     for (int i = 0; i < NB / 4; ++i) bDst[b * BUFB + i * BP] = u32x4{rb[4 * i], rb[4 * i + 1], rb[4 * i + 2], rb[4 * i + 3]};
   };
@@ -879,7 +896,7 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   step(Buf0{}, Buf1{}, kt, kt + 1 < nkt, kt + 2 < nkt);
   if (kt + 1 < nkt) step(Buf1{}, Buf0{}, kt + 1, kt + 2 < nkt, false);
   if (kt + 2 < nkt) step(Buf0{}, Buf1{}, kt + 2, false, false);
-  fwdEpilogue<TBN>(p, g, acc, bx, by, m0, j0, wm, wn, grp, idx, biasS, whole ? 0 : 1);
+  fwdEpilogue<TBN, TI>(p, g, acc, bx, by, m0, j0, wm, wn, grp, idx, biasS, whole ? 0 : 1);
 }
 
 template <int WM, bool LINEAR = false>
@@ -929,7 +946,7 @@ __device__ __forceinline__ void fwdTailFixupBody(const FwdArgs &p, const ConvGeo
   }
   const int r = e / p.bn, c = e - r * p.bn;
   const int row = mTile * p.bm + r;
-  if (row >= p.M) return;
+  if (r >= p.bm || row >= p.M) return;  // 32 x 256 tiles fill half of a partial
   const float b = p.bias ? p.bias[row] : 0.f;
   const float vals[4] = {v.x + b, v.y + b, v.z + b, v.w + b};
 #pragma unroll
@@ -1497,7 +1514,10 @@ struct FwdPlan {
 // Tiles of an M x Ncols output reduced over nkt k-tiles; wideOk: the 64 x 256 tile shape may be used.
 void planTiles(FwdPlan &pl, int M, long Ncols, int nkt, bool wideOk) {
   const bool wide = wideOk && tiles(M, 64) * 64 < tiles(M, BM) * BM;
-  pl.bm = wide ? 64 : BM, pl.bn = wide ? 256 : BN;
+  // 32-row tiles when they cut the padded rows by a quarter or more (a wave then issues half the MFMAs per
+  // element it gathers)
+  const bool low = wideOk && tiles(M, 32) * 32 * 4 <= tiles(M, 64) * 64 * 3;
+  pl.bm = low ? 32 : wide ? 64 : BM, pl.bn = low || wide ? 256 : BN;
   pl.mTiles = (int)tiles(M, pl.bm);
   pl.total = pl.mTiles * (int)tiles(Ncols, pl.bn);
   const int cus = residentSlots(nullptr);
@@ -1566,10 +1586,14 @@ void launchFwdKernels(hipStream_t s, const FwdPlan &pl, FwdArgs p, float *partia
     p.partial = partial;
     const dim3 grid(pl.full + pl.tail * p.nSplit);
     if (p.tapStride > 0) {
-      if (pl.bm == 64)
+      if (pl.bm == 32)
+        convFwdPaddedKernel<0, true><<<grid, dev::kBlock, 0, s>>>(p, gk);
+      else if (pl.bm == 64)
         convFwdPaddedKernel<1, true><<<grid, dev::kBlock, 0, s>>>(p, gk);
       else
         convFwdPaddedKernel<2, true><<<grid, dev::kBlock, 0, s>>>(p, gk);
+    } else if (pl.bm == 32) {
+      convFwdPaddedKernel<0><<<grid, dev::kBlock, 0, s>>>(p, gk);
     } else if (pl.bm == 64) {
       convFwdPaddedKernel<1><<<grid, dev::kBlock, 0, s>>>(p, gk);
     } else {

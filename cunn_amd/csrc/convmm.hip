@@ -1003,23 +1003,28 @@ struct GradWeightArgs {
 // would spend most of their multiplications on padding: the four waves all own the whole tile and take one
 // position group (4 of the 16 positions) of every k-tile each, i.e. a wave is a split of its own - it stores
 // its partial under split index 4 * split + wave and the fold adds them like any other splits.
-template <int OA, int OB>
-__device__ __forceinline__ void mfmaGroupPair(const float *aSrc, const float *bSrc, float16v (&acc)[2][2]) {
+template <int OA, int OB, int TI, int TJ>
+__device__ __forceinline__ void mfmaGroupPair(const float *aSrc, const float *bSrc, float16v (&acc)[TI][TJ]) {
   // lanes 0-31 hold position OA / OB of the group, lanes 32-63 the next one (aSrc / bSrc already point there)
-  const float a0 = aSrc[OA], a1 = aSrc[OA + 32 * 4];
-  const float b0 = bSrc[OB], b1 = bSrc[OB + 32 * 4];
-  acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-  acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-  acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-  acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+  float a[TI], b[TJ];
+#pragma unroll
+  for (int i = 0; i < TI; ++i) a[i] = aSrc[OA + i * 32 * 4];
+#pragma unroll
+  for (int j = 0; j < TJ; ++j) b[j] = bSrc[OB + j * 32 * 4];
+#pragma unroll
+  for (int i = 0; i < TI; ++i)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
 }
 
-template <bool L16, int WMODE>
+// (TI, TJ): 32-row and 32-column blocks of a small tile (WMODE = 0 only): 64 x 64, 32 x 64, 32 x 128, 64 x 32 ...
+template <bool L16, int WMODE, int TI = 2, int TJ = 2>
 __global__ void __launch_bounds__(dev::kBlock, 3)
 convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   constexpr bool TINY = WMODE == 0;
+  static_assert(TINY || (TI == 2 && TJ == 2), "block counts are a parameter of the small tiles only");
   constexpr int WM = TINY ? 1 : WMODE;  // loader layout: 64 rows as in the 64 x 256 shape
-  constexpr int TBM = 64 * WM, TBN = TINY ? 64 : 256 / WM;
+  constexpr int TBM = TINY ? 32 * TI : 64 * WM, TBN = TINY ? 32 * TJ : 256 / WM;
   constexpr int AP = TBM + 8;   // float4 per position-group row of As
   constexpr int GP = TBN + 4;   // of Bs: the 4 groups of a wave's scalar stores hit disjoint banks
   constexpr int NB = TBN / 16;  // columns a lane gathers per k-tile
@@ -1037,18 +1042,19 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   const int ktEnd = min(p.totalKt, ktBegin + p.ktPerSplit);
   const int kOob = 0x7fffffff;
 
-  float16v acc[2][2];
+  float16v acc[TI][TJ];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TJ; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   // ---- A loader. WM = 2: row o = t >> 1, positions 8 * (t & 1) .. + 7 of the k-tile as two float4;
-  //                WM = 1: row o = t >> 2, positions 4 * (t & 3) .. + 3 as one float4
+  //                WM = 1: row o = t >> 2, positions 4 * (t & 3) .. + 3 as one float4 (32-row tiles: both halves
+  //                of the workgroup fetch and park the same rows)
   const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc((void *)p.gy, 0, p.gyBytes, 0x00020000);
-  const int rowA = WM == 2 ? t >> 1 : t >> 2;
+  const int rowA = WM == 2 ? t >> 1 : (t >> 2) & (TBM - 1);
   const int pgA = WM == 2 ? (t & 1) * 2 : t & 3;  // first position group (of 4 positions) of the lane
   const int rowOffA = min(m0 + rowA, p.M - 1) * g.L * 4;  // rows past M are clamped and dropped in the epilogue
   const int imgStrideA = p.M * g.L * 4;
@@ -1154,7 +1160,7 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   auto step = [&](auto cur, auto nxt, bool store, bool load) {
     constexpr int C = decltype(cur)::value;
     if constexpr (TINY)
-      mfmaGroupPair<C * BUFA * 4, C * BUFB * 4>(aTiny, bTiny, acc);
+      mfmaGroupPair<C * BUFA * 4, C * BUFB * 4, TI, TJ>(aTiny, bTiny, acc);
     else
       mfmaHalf<C * BUFA, C * BUFB>(aSrc, bSrc, acc);
     __builtin_amdgcn_sched_barrier(0);
@@ -1162,7 +1168,7 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
     if (load) loadTiles();
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (TINY)
-      mfmaGroupPair<C * BUFA * 4 + 2, C * BUFB * 4 + 2>(aTiny, bTiny, acc);
+      mfmaGroupPair<C * BUFA * 4 + 2, C * BUFB * 4 + 2, TI, TJ>(aTiny, bTiny, acc);
     else
       mfmaHalf<C * BUFA + 2 * AP, C * BUFB + 2 * GP>(aSrc, bSrc, acc);
     __syncthreads();
@@ -1186,11 +1192,11 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   // lane holds column (lane & 31), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
   float *dst = p.partial + (long)(TINY ? split * 4 + wave : split) * p.M * p.Ncols;
 #pragma unroll
-  for (int tj = 0; tj < 2; ++tj) {
+  for (int tj = 0; tj < TJ; ++tj) {
     const int col = j0 + wn * 64 + tj * 32 + idx;
     if (col >= p.Ncols) continue;
 #pragma unroll
-    for (int ti = 0; ti < 2; ++ti)
+    for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + grp * 4 + (v & 3);
@@ -1201,7 +1207,7 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
     // the 2 (WM = 2) or 4 (WM = 1) lanes that loaded parts of a row are neighbours inside a quad
     rowSum = dev::dppAdd<0xB1>(rowSum);
     if (WM == 1) rowSum = dev::dppAdd<0x4E>(rowSum);
-    if ((t & (WM == 2 ? 1 : 3)) == 0 && m0 + rowA < p.M) {
+    if ((t & (WM == 2 ? 1 : 3)) == 0 && m0 + rowA < p.M && (t >> 2) < TBM) {
       if (TINY) {  // four partial slots per workgroup: the row sums go to the first, the others add nothing
         float *bp = p.biasPartial + (long)split * 4 * p.M + m0 + rowA;
         bp[0] = rowSum, bp[p.M] = 0.f, bp[2 * (long)p.M] = 0.f, bp[3 * (long)p.M] = 0.f;
@@ -2208,15 +2214,51 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
   const bool l16 = Lk % BK == 0;
   // tile shape: 64 x 256 where it covers gradWeight (Cout x K) with less padding than 128 x 128
   const bool wide = fast && tiles(g.Cout, 64) * 64 * tiles(g.K, 256) * 256 < tiles(g.Cout, BM) * BM * tiles(g.K, BN) * BN;
-  // 64 x 64 tiles (the waves of a workgroup split the positions instead of the tile) where the large shapes
-  // would multiply at least four times as much padding: small gradWeights are bound by memory, not by the matrix pipe
-  const long bigArea = std::min(tiles(g.Cout, 64) * 64 * tiles(g.K, 256) * 256, tiles(g.Cout, BM) * BM * tiles(g.K, BN) * BN);
-  const int tinyPct = 120;  // 64 x 64 tiles whenever they cut the padded area by a fifth: measured faster down to that
-  const bool tiny = fast && tiles(g.Cout, 64) * 64 * tiles(g.K, 64) * 64 * tinyPct <= bigArea * 100;
-  const int mT = (int)tiles(g.Cout, tiny || wide ? 64 : BM), nT = (int)tiles(g.K, tiny ? 64 : wide ? 256 : BN);
+  // Small tiles (the waves of a workgroup split the positions instead of the tile; blocks of 32 rows x 32 columns:
+  // 1x1, 1x2, 1x4, 2x1, 2x2) where the large shapes would mostly multiply padding. The shape is the one with
+  // the least tiles x cost per tile and k-tile; the costs are measured (first layers, 32- and 64-plane layers at
+  // 56x56 ... 149x149): the gather of the image patch weighs more than the matrix instructions, so a tile is not
+  // cheaper in proportion to its area.
+  struct Shape {
+    int ti, tj, cost;
+  };
+  static const Shape kSmall[] = {{2, 2, 88}, {1, 4, 90}, {1, 2, 50}, {2, 1, 50}, {1, 1, 33}};
+  const int kBigCost = 250;  // a 128 x 128 or 64 x 256 tile
+  long bestCost = std::min(tiles(g.Cout, 64) * tiles(g.K, 256), tiles(g.Cout, BM) * tiles(g.K, BN)) * (long)kBigCost;
+  int tI = 0, tJ = 0;
+  if (fast)
+    for (const Shape &sh : kSmall) {
+      const long c = (long)tiles(g.Cout, 32 * sh.ti) * tiles(g.K, 32 * sh.tj) * sh.cost;
+      if (c < bestCost) bestCost = c, tI = sh.ti, tJ = sh.tj;
+    }
+  const bool tiny = tI > 0;
+  const int mT = (int)tiles(g.Cout, tiny ? 32 * tI : wide ? 64 : BM), nT = (int)tiles(g.K, tiny ? 32 * tJ : wide ? 256 : BN);
+  struct TinyKernel {
+    const void *fn;
+    void (*launch)(dim3, hipStream_t, const GradWeightArgs &, const ConvGeom &);
+  };
+  auto tinyKernel = [&](auto l16c, auto tic, auto tjc) {
+    constexpr bool L = decltype(l16c)::value;
+    constexpr int I = decltype(tic)::value, J = decltype(tjc)::value;
+    return TinyKernel{(const void *)convGradWeightKernel<L, 0, I, J>,
+                      [](dim3 grid, hipStream_t st, const GradWeightArgs &q, const ConvGeom &gk) {
+                        convGradWeightKernel<L, 0, I, J><<<grid, dev::kBlock, 0, st>>>(q, gk);
+                      }};
+  };
+  auto pickTiny = [&](auto l16c) {
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I4 = std::integral_constant<int, 4>;
+    if (tI == 1 && tJ == 1) return tinyKernel(l16c, I1{}, I1{});
+    if (tI == 1 && tJ == 2) return tinyKernel(l16c, I1{}, I2{});
+    if (tI == 1 && tJ == 4) return tinyKernel(l16c, I1{}, I4{});
+    if (tI == 2 && tJ == 1) return tinyKernel(l16c, I2{}, I1{});
+    return tinyKernel(l16c, I2{}, I2{});
+  };
+  const TinyKernel tk = l16 ? pickTiny(std::true_type{}) : pickTiny(std::false_type{});
   const void *kern =
       !fast  ? (const void *)convGemmKernel<kGradWeight>
-      : tiny ? (l16 ? (const void *)convGradWeightKernel<true, 0> : (const void *)convGradWeightKernel<false, 0>)
+      : tiny ? tk.fn
       : l16  ? (wide ? (const void *)convGradWeightKernel<true, 1> : (const void *)convGradWeightKernel<true, 2>)
              : (wide ? (const void *)convGradWeightKernel<false, 1> : (const void *)convGradWeightKernel<false, 2>);
   // Every split leaves a partial copy of gradWeight (64 KB per tile) for the fold: three workgroups per CU
@@ -2278,10 +2320,8 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     q.magicOW = dev::magicOf(g.oW);
     q.Lvalid = g.L;
     const dim3 grid(mT * nT * wgSplits);
-    if (tiny && l16)
-      convGradWeightKernel<true, 0><<<grid, dev::kBlock, 0, s>>>(q, gk);
-    else if (tiny)
-      convGradWeightKernel<false, 0><<<grid, dev::kBlock, 0, s>>>(q, gk);
+    if (tiny)
+      tk.launch(grid, s, q, gk);
     else if (l16 && wide)
       convGradWeightKernel<true, 1><<<grid, dev::kBlock, 0, s>>>(q, gk);
     else if (l16)

@@ -312,44 +312,54 @@ dwAccGradStage1(const float *__restrict__ in, const float *__restrict__ gradOut,
 }
 
 // Stage 2: one wave per (c, j) folds the partials of all slots in a fixed order and accumulates
-// scale * sum into the caller's tensors. A lane owns one tap (lane % TP) and every PH-th slot
-// (PH = 64 / TP slot phases, lane / TP): a load instruction of the wave reads PH whole runs as the
-// stage-1 workgroups wrote them; the phases are then added in a fixed association. The old value is
-// requested before the partials so that the read-modify-write costs no second round trip.
+// scale * sum into the caller's tensors. A lane owns four taps (one 16-byte group of a run, lane % Q) and every
+// PH-th slot (PH = 64 / Q slot phases, lane / Q): a load instruction of the wave reads PH whole runs as the
+// stage-1 workgroups wrote them, and up to 8 of them are in flight before the first add, so a batch of 64 images
+// is one memory round trip. The phases are then added in a fixed association. The old values are requested before
+// the partials so that the read-modify-write costs no second round trip.
 template <int TP>
 __global__ void __launch_bounds__(dev::kWave)
 dwAccGradStage2(const float *__restrict__ partial, float *__restrict__ gradWeight, Strides4 gs,
                 float *__restrict__ gradBias, Strides2 bs, int M, int kW, int T, int nslots, float scale, int CJ) {
-  constexpr int PH = dev::kWave / TP;
+  constexpr int Q = TP / 4, PH = dev::kWave / Q;
   constexpr int U = 8;  // loads in flight per lane
   const int cj = blockIdx.x;
-  const int t = threadIdx.x % TP, ph = threadIdx.x / TP;
+  const int q = threadIdx.x % Q, ph = threadIdx.x / Q;
   const int c = cj / M, j = cj - c * M;
-  float *dst = nullptr;
-  if (ph == 0 && t < T - 1) {
-    const int kh = t / kW, kw = t - kh * kW;
-    dst = gradWeight + j * gs.s0 + c * gs.s1 + kh * gs.s2 + kw * gs.s3;
-  } else if (ph == 0 && t == T - 1 && gradBias) {
-    dst = gradBias + j * bs.s0 + c * bs.s1;
-  }
-  const float old = dst ? *dst : 0.f;
-  const long step = (long)CJ * TP;  // floats between the runs of consecutive slots
-  const float *p = partial + (long)cj * TP + t;
-  float v = 0.f;
-  int sl = ph;
-  if (t < T) {
-    for (; sl + (U - 1) * PH < nslots; sl += U * PH) {
-      float a[U];
+  float *dst[4];
+  float old[4];
 #pragma unroll
-      for (int u = 0; u < U; ++u) a[u] = p[(long)(sl + u * PH) * step];
-#pragma unroll
-      for (int u = 0; u < U; ++u) v += a[u];
+  for (int e = 0; e < 4; ++e) {
+    const int t = q * 4 + e;
+    dst[e] = nullptr;
+    if (ph == 0 && t < T - 1) {
+      const int kh = t / kW, kw = t - kh * kW;
+      dst[e] = gradWeight + j * gs.s0 + c * gs.s1 + kh * gs.s2 + kw * gs.s3;
+    } else if (ph == 0 && t == T - 1 && gradBias) {
+      dst[e] = gradBias + j * bs.s0 + c * bs.s1;
     }
-    for (; sl < nslots; sl += PH) v += p[(long)sl * step];
+    old[e] = dst[e] ? *dst[e] : 0.f;
   }
-  if (PH == 4) v += __shfl_down(v, 32);
-  v += __shfl_down(v, TP);
-  if (dst) *dst = old + scale * v;
+  const long step = (long)CJ * TP;  // floats between the runs of consecutive slots
+  const float *p = partial + (long)cj * TP + q * 4;
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s0 = ph; s0 < nslots; s0 += U * PH) {
+    float4 a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int sl = s0 + u * PH;
+      a[u] = sl < nslots ? *reinterpret_cast<const float4 *>(p + (long)sl * step) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) v.x += a[u].x, v.y += a[u].y, v.z += a[u].z, v.w += a[u].w;
+  }
+  float r[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+#pragma unroll
+    for (int m = dev::kWave / 2; m >= Q; m >>= 1) r[e] += __shfl_down(r[e], m);
+    if (dst[e]) *dst[e] = old[e] + scale * r[e];
+  }
 }
 
 // Any geometry: one workgroup per (c, j, tap) - tap == kH*kW is the bias - that

@@ -2226,7 +2226,7 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     int ti, tj, cost;
   };
   static const Shape kSmall[] = {{2, 2, 88}, {1, 4, 90}, {1, 2, 50}, {2, 1, 50}, {1, 1, 33}};
-  const int kBigCost = 250;  // a 128 x 128 or 64 x 256 tile
+  const int kBigCost = 260;  // a 128 x 128 or 64 x 256 tile
   long bestCost = std::min(tiles(g.Cout, 64) * tiles(g.K, 256), tiles(g.Cout, BM) * tiles(g.K, BN)) * (long)kBigCost;
   int tI = 0, tJ = 0;
   if (fast)

@@ -518,6 +518,49 @@ def wl_bnrelu(nsets, fused=True):
                      + ("fused entry points" if fused else "four separate calls"))
 
 
+def wl_convrelu(nsets, fused=True):
+    """Beyond the five configurations: a 1x1 convolution (128 -> 128 planes at 56 x 56, N = 64) followed by ReLU, forward,
+    as the fused entry point (include/THCUNN_fused.h) or as the two calls it replaces."""
+    from cunn_amd import CudaTensor as CT, THNN
+    from oracle import oracle as O
+    N, Ci, Co, H = 64, 128, 128, 56
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((N, Ci, H, H)).astype(np.float32)
+    w = (rng.standard_normal((Co, Ci)) * np.sqrt(2.0 / Ci)).astype(np.float32)
+    b = rng.uniform(-0.02, 0.02, Co).astype(np.float32)
+    sets = [dict(x=CT.from_numpy(x), y=CT(), a=CT(), w=CT.from_numpy(w), b=CT.from_numpy(b), cols=CT(), ones=CT()) for _ in range(nsets)]
+    g = (1, 1, 1, 1, 0, 0)
+
+    def calls(i):
+        t = sets[i]
+        if fused:
+            return [("convrelu_updateOutput", lambda: THNN.SpatialConvolutionMMReLU_updateOutput(t["x"], t["a"], t["w"], t["b"], t["cols"], t["ones"], *g))]
+        return [("convmm_updateOutput", lambda: THNN.SpatialConvolutionMM_updateOutput(t["x"], t["y"], t["w"], t["b"], t["cols"], t["ones"], *g)),
+                ("threshold_updateOutput", lambda: THNN.Threshold_updateOutput(t["y"], t["a"], 0.0, 0.0, False))]
+
+    fl = 2.0 * Co * Ci * H * H * N
+    work = ({"convrelu_updateOutput": (fl, "flops")} if fused else
+            {"convmm_updateOutput": (fl, "flops"), "threshold_updateOutput": (0, "flops")})
+    ns = 4
+
+    def cpu(reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            O.threshold_updateOutput(O.convmm_updateOutput(x[:ns], w, b, *g), 0.0, 0.0)
+        return time.perf_counter() - t0, reps * ns, f"{reps} passes over {ns} images"
+
+    def verify():
+        t = sets[0]
+        for _, fn in calls(0):
+            fn()
+        ref = O.threshold_updateOutput(O.convmm_updateOutput(x[:ns], w, b, *g), 0.0, 0.0)
+        np.testing.assert_allclose(t["a"].numpy()[:ns], ref, rtol=1e-5, atol=1e-4)
+
+    return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="mfma",
+                desc=f"SpatialConvolutionMM + ReLU forward fp32 N={N} Cin={Ci} Cout={Co} {H}x{H} k1 bias, "
+                     + ("fused entry point" if fused else "two separate calls"))
+
+
 def wl_copy(nsets):
     """Calibration: plain device-to-device copy of 128 MB (2 x 128 MB of HBM traffic per launch)."""
     from cunn_amd import CudaTensor as CT
@@ -540,7 +583,8 @@ def wl_copy(nsets):
 WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda n: wl_dw("cfg2", n), "cfg3": wl_bn, "cfg4": wl_pool,
              "dw147": lambda n: wl_dw("dw147", n), "dw14": lambda n: wl_dw("dw14", n), "pool71": lambda n: wl_pool(n, odd=True),
              "cfg5": wl_conv, "pw128": lambda n: wl_conv(n, pointwise=True), "conv1": lambda n: wl_conv(n, first=True), "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu,
-             "bnrelu": wl_bnrelu, "bnrelu_unfused": lambda n: wl_bnrelu(n, fused=False)}
+             "bnrelu": wl_bnrelu, "bnrelu_unfused": lambda n: wl_bnrelu(n, fused=False),
+             "convrelu": wl_convrelu, "convrelu_unfused": lambda n: wl_convrelu(n, fused=False)}
 
 
 PREROLL_SAMPLES = 12   # event samples per entry point collected before the timed region, whatever --warmup is

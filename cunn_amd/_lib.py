@@ -30,6 +30,8 @@ ENTRY_POINTS = [
     "SpatialDepthWiseConvolution_accGradParameters_noAlloc",
     # no counterpart in the reference: BatchNormalization + Threshold(0, 0) in one pass (include/THCUNN_fused.h)
     "BatchNormalizationReLU_updateOutput", "BatchNormalizationReLU_backward",
+    # no counterpart in the reference: SpatialConvolutionMM + Threshold(0, 0) in one pass (include/THCUNN_fused.h)
+    "SpatialConvolutionMMReLU_updateOutput",
 ]
 
 _T = C.c_void_p  # THCudaTensor* / THCudaLongTensor* / THCState*
@@ -64,6 +66,7 @@ SIGNATURES = {
     "SpatialDepthWiseConvolution_accGradParameters_noAlloc": [_T] * 5 + [_i] * 6 + [_f],
     "BatchNormalizationReLU_updateOutput": [_T] * 9 + [_b, _d, _d],
     "BatchNormalizationReLU_backward": [_T] * 12 + [_b, _d, _d],
+    "SpatialConvolutionMMReLU_updateOutput": [_T] * 7 + [_i] * 6,
 }
 
 _LP = C.POINTER(C.c_long)

@@ -47,7 +47,8 @@ struct PwDone {
 // NW = 8 is one workgroup per CU, two waves per SIMD that take turns on the matrix pipe and meet at every chunk's
 // barrier: they advance together. (Two independent workgroups of 4 waves per CU do not - the SIMD favours the
 // older wave, one workgroup of each pair finishes at 60 % of the time and the other runs the rest alone.)
-template <int K, int MR, int WR, int CT, int NW>
+// RELU: the stored value is v > 0 ? v : 0.
+template <int K, int MR, int WR, int CT, int NW, bool RELU = false>
 __global__ void __launch_bounds__(64 * NW, 2)
 convPointwiseKernel(PwArgs p) {
   constexpr int BLK = 64 * NW;
@@ -163,7 +164,10 @@ convPointwiseKernel(PwArgs p) {
   auto storeOne = [&](const Done &d, int i) {
     const int q = i / (MR * 16), r = (i / 16) % MR, v = i % 16;
     const int rowBase = m0 + 32 * r + 8 * (v >> 2) + (v & 3);  // wave-uniform: a scalar offset
-    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(d.acc[q][r][v]), outr, d.voff[q][r][v >> 2], rowBase * p.L * 4, 0);
+    float o = d.acc[q][r][v];
+    // one instruction between the MFMAs: max(v, 0) is v > 0 ? v : 0 for every input (a NaN gives 0, -0 gives +0)
+    if (RELU) asm volatile("v_max_f32 %0, 0, %1" : "=v"(o) : "v"(o));
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(o), outr, d.voff[q][r][v >> 2], rowBase * p.L * 4, 0);
   };
   // second operand of MFMA s of column tile ct: lane (j = lane % 32, kk = lane / 32) holds x[2s + kk][position j]
   auto bAddr = [&](int buf, int ct) {

@@ -359,6 +359,7 @@ struct FwdArgs {
   // workgroup full + split * tail + i reduces split `split` of tile tile0 + i (tile0 = full)
   int full, tail;
   float *partial;
+  int relu;           // != 0: the stored value is v > 0 ? v : 0 (Threshold(0, 0) applied to the output)
   const int *taps;    // padded kernel: byte offset of tap (c, kh, kw) inside a (zero-padded) image, per k
   int tapStride;      // > 0 (1x1 windows): tap k sits at byte offset k * tapStride, no table is read
 };
@@ -418,7 +419,9 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
-          if (row < p.M) dst[(long)row * p.outRow] = BIAS ? acc[ti][tj][v] + bv[ti][v] : acc[ti][tj][v];
+          float o = BIAS ? acc[ti][tj][v] + bv[ti][v] : acc[ti][tj][v];
+          if (p.relu) o = o > 0.f ? o : 0.f;
+          if (row < p.M) dst[(long)row * p.outRow] = o;
         }
     }
   };
@@ -948,7 +951,11 @@ __device__ __forceinline__ void fwdTailFixupBody(const FwdArgs &p, const ConvGeo
   const int row = mTile * p.bm + r;
   if (r >= p.bm || row >= p.M) return;  // 32 x 256 tiles fill half of a partial
   const float b = p.bias ? p.bias[row] : 0.f;
-  const float vals[4] = {v.x + b, v.y + b, v.z + b, v.w + b};
+  float vals[4] = {v.x + b, v.y + b, v.z + b, v.w + b};
+  if (p.relu) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) vals[i] = vals[i] > 0.f ? vals[i] : 0.f;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const long col = (long)nTile * p.bn + c + i;
@@ -1636,7 +1643,7 @@ void launchFwdKernels(hipStream_t s, const FwdPlan &pl, FwdArgs p, float *partia
 
 // out(nImages, M, L) = bias + W(M x K) * im2col(x); `scratch` holds plan.scratchFloats floats
 void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const float *w, const float *x, float *out,
-                       const float *bias, int M, int nImages, const ConvGeom &g) {
+                       const float *bias, int M, int nImages, const ConvGeom &g, bool relu = false) {
   const bool fast = pl.tapEntries > 0;
   if (fast && !(launch::aligned16(scratch) && (pl.weightFloats > 0 || launch::aligned16(w))))
     error("SpatialConvolutionMM: internal error, convolution scratch or weights not 16-byte aligned");
@@ -1673,6 +1680,7 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
   p.w = w;
   p.out = out;
   p.bias = bias;
+  p.relu = relu ? 1 : 0;
   p.M = M;
   p.Ncols = nImages * g.L;
   p.outImg = (long)M * g.L, p.outRow = g.L, p.outSH = g.oW, p.outSW = 1;
@@ -1720,10 +1728,10 @@ bool pwShape(int M, int K, PwShape *sh) {
   return true;
 }
 
-template <int K, int MR, int WR, int CT, int NW>
+template <int K, int MR, int WR, int CT, int NW, bool RELU>
 void launchPointwiseShape(hipStream_t s, PwArgs p, int device) {
   constexpr size_t lds = 2 * (size_t)K * 32 * CT * sizeof(float);
-  auto kernel = convPointwiseKernel<K, MR, WR, CT, NW>;
+  auto kernel = convPointwiseKernel<K, MR, WR, CT, NW, RELU>;
   if (lds > 64 * 1024) {  // once per kernel instance and device: allow more than 64 KB of dynamic LDS
     static std::atomic<bool> raised[64];
     if (!raised[device].load()) {
@@ -1743,7 +1751,8 @@ void launchPointwiseShape(hipStream_t s, PwArgs p, int device) {
 }
 
 // out(N, M, L) = bias + W(M x K) x(N, K, L) on the weight-stationary kernel; false: the shape is not one of its
-bool convPointwise(THCState *state, const ConvGeom &g, const float *x, const float *w, const float *bias, float *out) {
+bool convPointwise(THCState *state, const ConvGeom &g, const float *x, const float *w, const float *bias, float *out,
+                   bool relu = false) {
   if (forceGeneric() || g_switches.convPointwise == 0) return false;
   if (g.kH != 1 || g.kW != 1 || g.dH != 1 || g.dW != 1 || g.padH != 0 || g.padW != 0) return false;
   const long P = (long)g.N * g.L;
@@ -1764,7 +1773,10 @@ bool convPointwise(THCState *state, const ConvGeom &g, const float *x, const flo
   hipStream_t s = state->stream;
 #define PW_CASE(KK, MRR, WRR, CTT, NWW)                                              \
   if (g.K == KK && sh.mr == MRR && sh.wr == WRR && sh.ct == CTT && sh.nw == NWW) {   \
-    launchPointwiseShape<KK, MRR, WRR, CTT, NWW>(s, p, device);                      \
+    if (relu)                                                                        \
+      launchPointwiseShape<KK, MRR, WRR, CTT, NWW, true>(s, p, device);              \
+    else                                                                             \
+      launchPointwiseShape<KK, MRR, WRR, CTT, NWW, false>(s, p, device);             \
     return true;                                                                     \
   }
   PW_CASE(32, 2, 4, 16, 8) PW_CASE(32, 1, 4, 16, 8) PW_CASE(32, 1, 2, 16, 8)
@@ -1779,10 +1791,11 @@ bool convPointwise(THCState *state, const ConvGeom &g, const float *x, const flo
 // unspecified afterwards.
 
 // out(N, Cout, oH, oW) = bias + conv(x(N, Cin, H, W), w(Cout, K))
+// relu: out = Threshold(0, 0) of that, applied as the values are stored
 void convForward(THCState *state, const ConvGeom &g, const float *x, const float *w, const float *bias, float *out,
-                 THCudaTensor *scratchBuf, const char *bufName) {
+                 THCudaTensor *scratchBuf, const char *bufName, bool relu = false) {
   if ((long)g.N * g.Cout == 0) return;
-  if (convPointwise(state, g, x, w, bias, out)) return;
+  if (convPointwise(state, g, x, w, bias, out, relu)) return;
   hipStream_t s = state->stream;
   // images per launch so that the flat column index n*L + l fits an int
   int group = (int)std::min<long>(g.N, std::max<long>(1, 0x7fffffffL / 2 / g.L));
@@ -1799,7 +1812,7 @@ void convForward(THCState *state, const ConvGeom &g, const float *x, const float
       int cnt = std::min(group, g.N - n0);
       if (cnt != std::min(group, g.N)) pl = planFwdImplicit(g.Cout, cnt, g, launch::aligned16(w));
       launchFwdImplicit(s, pl, scratch, w, x + (long)n0 * g.Cin * g.H * g.W, out + (long)n0 * g.Cout * g.L, bias, g.Cout,
-                        cnt, g);
+                        cnt, g, relu);
     }
     return;
   }
@@ -1821,6 +1834,7 @@ void convForward(THCState *state, const ConvGeom &g, const float *x, const float
     convGemmKernel<kForward><<<grid, dev::kBlock, 0, s>>>(p, g);
     THC_HIP_CHECK(hipGetLastError());
   }
+  if (relu) reluInPlace(s, out, (long)g.N * g.Cout * g.L);  // the first-generation kernel has no such epilogue
 }
 
 // Taps and gy indices of phase ph along one axis (see PhaseAxis).
@@ -2373,7 +2387,7 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
 // ---- entry-point bodies shared by SpatialConvolutionMM and SpatialDilatedConvolution --------
 void convUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output, THCudaTensor *weight,
                       THCudaTensor *bias, THCudaTensor *columns, int kW, int kH, int dW, int dH, int padW, int padH,
-                      int dilW, int dilH, ConvFlavor flavor) {
+                      int dilW, int dilH, ConvFlavor flavor, bool relu = false) {
   THC_ARG_CHECK(output != nullptr, 3, "output tensor expected");
   ConvCall call = convSetup(input, nullptr, weight, bias, "weight", kH, kW, dH, dW, padH, padW, dilH, dilW, flavor);
   ConvGeom &g = call.g;
@@ -2383,7 +2397,7 @@ void convUpdateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output
   else
     resize(state, output, {g.Cout, g.oH, g.oW});
   if (!isContiguous(erase(output))) error("output tensor has to be contiguous");
-  convForward(state, g, in.ptr(), data(weight), bias ? data(bias) : nullptr, data(output), columns, "columns");
+  convForward(state, g, in.ptr(), data(weight), bias ? data(bias) : nullptr, data(output), columns, "columns", relu);
 }
 
 void convUpdateGradInput(THCState *state, THCudaTensor *input, THCudaTensor *gradOutput, THCudaTensor *gradInput,
@@ -2530,6 +2544,18 @@ void THNN_CudaSpatialConvolutionMM_updateOutput(THCState *state, THCudaTensor *i
   THNN_ENTER
   (void)ones;  // never read; `columns` is used (and resized) only as scratch
   convUpdateOutput(state, input, output, weight, bias, columns, kW, kH, dW, dH, padW, padH, 1, 1, kConvMM);
+  THNN_LEAVE
+}
+
+// No counterpart in the reference (include/THCUNN_fused.h): SpatialConvolutionMM_updateOutput followed by
+// Threshold_updateOutput(0, 0), the clamp applied as the convolution stores its values.
+void THNN_CudaSpatialConvolutionMMReLU_updateOutput(THCState *state, THCudaTensor *input, THCudaTensor *output,
+                                                    THCudaTensor *weight, THCudaTensor *bias, THCudaTensor *columns,
+                                                    THCudaTensor *ones, int kW, int kH, int dW, int dH, int padW,
+                                                    int padH) {
+  THNN_ENTER
+  (void)ones;
+  convUpdateOutput(state, input, output, weight, bias, columns, kW, kH, dW, dH, padW, padH, 1, 1, kConvMM, true);
   THNN_LEAVE
 }
 

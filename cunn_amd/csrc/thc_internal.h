@@ -171,6 +171,8 @@ extern Switches g_switches;
 // THNN_CudaSpatialDepthWiseConvolution_accGradParameters_noAlloc (dwconv.hip). Called when a state is
 // made, so that the entry point itself finds the address in a table.
 void dwNoAllocInit(int device);
+// x[i] = x[i] > 0 ? x[i] : 0 over n contiguous floats (threshold.hip)
+void reluInPlace(hipStream_t stream, float *x, long n);
 
 // THCUNN_check_dim_size (lib/THCUNN/common.h:69-75)
 void checkDimSize(const Tensor *t, const char *name, int dim, int dimSize, long size);

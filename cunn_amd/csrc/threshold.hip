@@ -59,6 +59,14 @@ void launchThreshold(hipStream_t s, const float *x, const float *other, float *o
   }
 }
 
+}  // namespace
+
+namespace thc {
+void reluInPlace(hipStream_t s, float *x, long n) { launchThreshold<false>(s, x, nullptr, x, n, 0.f, 0.f); }
+}  // namespace thc
+
+namespace {
+
 // A tensor's elements as a contiguous device array: the tensor's own memory when it is
 // contiguous, else a packed temporary that `commit` scatters back through the strides.
 class Packed {

@@ -1,5 +1,6 @@
 /*
- * THCUNN_fused.h - entry points that fuse two neighbouring modules of the path into one pass.
+ * THCUNN_fused.h - entry points that fuse two neighbouring modules of the path into one pass
+ * (BatchNormalization + ReLU forward and backward, SpatialConvolutionMM + ReLU forward).
  *
  * Nothing here has a prototype in the reference: lib/THCUNN/generic/THCUNN.h declares one function per module and
  * the nn modules call them one after the other, so `conv -> BatchNormalization -> Threshold(0, 0)` writes the
@@ -43,6 +44,18 @@ void THNN_CudaBatchNormalizationReLU_backward(
     THCudaTensor *runningMean_, THCudaTensor *runningVar_,
     THCudaTensor *saveMean_, THCudaTensor *saveStd_,
     bool train, double scale, double eps);
+
+/* output = max(SpatialConvolutionMM(input), 0): THNN_CudaSpatialConvolutionMM_updateOutput
+ * (lib/THCUNN/generic/SpatialConvolutionMM.cu:58-209) followed by Threshold_updateOutput(threshold 0, value 0)
+ * (lib/THCUNN/generic/Threshold.cu:7-35) - v > 0 ? v : 0 applied as the convolution stores its values, so the
+ * pre-activation never reaches memory. Arguments and side effects are those of the plain call. The backward pass
+ * of the pair is the plain one: Threshold_updateGradInput(output, gradOutput) - the sign of the stored output is the
+ * sign of the pre-activation wherever it matters - then SpatialConvolutionMM_updateGradInput / _accGradParameters. */
+void THNN_CudaSpatialConvolutionMMReLU_updateOutput(
+    THCState *state, THCudaTensor *input, THCudaTensor *output, THCudaTensor *weight,
+    THCudaTensor *bias,         /* [OPTIONAL] */
+    THCudaTensor *columns, THCudaTensor *ones,
+    int kW, int kH, int dW, int dH, int padW, int padH);
 
 #ifdef __cplusplus
 }

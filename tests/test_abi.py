@@ -20,7 +20,8 @@ def test_library_exports_every_declared_symbol():
     from cunn_amd import _lib
     lib = _lib.load()
     declared = _declared("THCUNN.h") + _declared("THCShim.h") + _declared("THCUNN_fused.h")
-    assert len(_declared("THCUNN_fused.h")) == 2   # BatchNormalization + ReLU, forward and backward
+    # BatchNormalization + ReLU, forward and backward; SpatialConvolutionMM + ReLU, forward
+    assert len(_declared("THCUNN_fused.h")) == 3
     # 14 hot-path + 9 dilated / transposed convolution + 2 Threshold + the no-allocation accGradParameters variant
     assert len(_declared("THCUNN.h")) == 26
     # the test hooks: the two column kernels and the kernel-family switch

@@ -1905,7 +1905,8 @@ bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const
   // split along K so that a workgroup reduces about the same number of k-tiles whatever its phase and the
   // grid holds about two workgroups per CU. Split phases leave partial tiles for the batched fold.
   const bool wide = tiles(g.Cin, 64) * 64 < tiles(g.Cin, BM) * BM;
-  const int bm = wide ? 64 : BM, bn = wide ? 256 : BN;
+  const bool low = tiles(g.Cin, 32) * 32 * 4 <= tiles(g.Cin, 64) * 64 * 3;  // as in planTiles
+  const int bm = low ? 32 : wide ? 64 : BM, bn = low || wide ? 256 : BN;
   const int mTiles = (int)tiles(g.Cin, bm);
   struct Split {
     int tiles, nSplit, ktPerSplit;
@@ -1982,7 +1983,9 @@ bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const
       maxTiles = std::max(maxTiles, it.tiles), maxSplit = std::max(maxSplit, a.nSplit);
     }
     const dim3 grid(maxTiles, maxSplit, set.count);
-    if (wide)
+    if (low)
+      convFwdPaddedBatchKernel<0><<<grid, dev::kBlock, 0, s>>>(batch);
+    else if (wide)
       convFwdPaddedBatchKernel<1><<<grid, dev::kBlock, 0, s>>>(batch);
     else
       convFwdPaddedBatchKernel<2><<<grid, dev::kBlock, 0, s>>>(batch);
@@ -2128,10 +2131,10 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
     }
     return;
   }
-  // With few input planes the phase GEMMs would use a sliver of their 64-row tiles; the column GEMM
-  // (K rows) is the better shape then. Test switch THCUNN_CONV_GRADINPUT = "phases" / "columns" overrides.
-  const bool phasesPay = 2L * g.Cin >= (long)tiles(g.Cin, 64) * 64;
-  const bool tryPhases = route == 1 ? true : route == 2 ? false : phasesPay;
+  // Every other geometry goes phase by phase (with 32-row tiles that measured faster than the gradient columns
+  // below down to 8 input planes: 8 -> 16 3x3 stride 2 at 128x128, N = 32: 37 against 62 us); the columns remain for
+  // what that route refuses and for the test switch THCUNN_CONV_GRADINPUT = "columns".
+  const bool tryPhases = route != 2;
   if (!forceGeneric() && tryPhases && gradInputByPhase(state, g, gy, w, gi, scratchBuf, bufName, bias)) return;
   // Gradient columns of a group of images at a time (<= 128 MB so the buffer stays cache resident), then
   // the col2im gather. gradCol[n][k][l] = sum_o W[o][k] * gy[n][o][l] is itself a 1x1 convolution of gy

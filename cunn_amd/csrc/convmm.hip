@@ -488,12 +488,36 @@ padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int 
 
 // The same for small planes (7x7 ... 28x28 stages: a workgroup per plane would leave most lanes idle): a lane per
 // 16-byte group of the whole destination. Workgroups past copyBlocks build the tap table.
+// ANY: planes of any size (9x9 = a bordered 7x7 plane): a group may straddle two planes and the last elements of
+// the destination may not fill a group.
+template <bool ANY>
 __global__ void __launch_bounds__(dev::kBlock)
 padPlanesFlatKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int padTop, int padLeft, int Hp, int Wp,
                     long total4, int copyBlocks, int *taps, int tapEntries, ConvGeom tg) {
   if ((int)blockIdx.x >= copyBlocks) {
     for (int k = (blockIdx.x - copyBlocks) * dev::kBlock + threadIdx.x; k < tapEntries; k += (gridDim.x - copyBlocks) * dev::kBlock)
       taps[k] = tapOffset(k, tg);
+    return;
+  }
+  if (ANY) {
+    // total4 counts elements here
+    const int plane = Hp * Wp;
+    const unsigned magicPlane = dev::magicOf(plane), magicW = dev::magicOf(Wp);
+    auto fetch = [&](unsigned e) {
+      const int pl = dev::fastDiv((int)e, magicPlane), j = (int)e - pl * plane;
+      const int hp = dev::fastDiv(j, magicW), wp = j - hp * Wp;
+      const int h = hp - padTop, w = wp - padLeft;
+      return (((unsigned)h < (unsigned)H) & ((unsigned)w < (unsigned)W)) ? x[(long)pl * H * W + h * W + w] : 0.f;
+    };
+    const long groups = (total4 + 3) >> 2;
+    for (long i = (long)blockIdx.x * dev::kBlock + threadIdx.x; i < groups; i += (long)copyBlocks * dev::kBlock) {
+      const unsigned e = (unsigned)(i * 4);
+      if (e + 4 <= (unsigned long)total4) {
+        reinterpret_cast<float4 *>(xp)[i] = make_float4(fetch(e), fetch(e + 1), fetch(e + 2), fetch(e + 3));
+      } else {
+        for (unsigned q = e; q < (unsigned long)total4; ++q) xp[q] = fetch(q);
+      }
+    }
     return;
   }
   const int plane4 = (Hp * Wp) >> 2;
@@ -524,8 +548,15 @@ void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int 
   if (plane % 4 == 0 && plane < 4096 && launch::aligned16(xp) && total4 * (plane / 4) < 0xffffffffL) {
     const int copyBlocks = (int)std::min<long>((total4 + dev::kBlock - 1) / dev::kBlock, 16384);
     const int tapBlocks = taps ? std::max(1, std::min(16, launch::ceilDiv(tapEntries, dev::kBlock))) : 0;
-    padPlanesFlatKernel<<<copyBlocks + tapBlocks, dev::kBlock, 0, s>>>(x, xp, H, W, padTop, padLeft, Hp, Wp, total4, copyBlocks,
-                                                                      taps, tapEntries, g);
+    padPlanesFlatKernel<false><<<copyBlocks + tapBlocks, dev::kBlock, 0, s>>>(x, xp, H, W, padTop, padLeft, Hp, Wp, total4,
+                                                                             copyBlocks, taps, tapEntries, g);
+  } else if (plane < 1024 && launch::aligned16(xp) && planes * plane * (long)plane < 0xffffffffL) {
+    // small planes of any size (a bordered 7x7 or 13x13 plane): a workgroup per plane would leave most of its lanes idle
+    const long total = planes * plane;
+    const int copyBlocks = (int)std::min<long>(((total + 3) / 4 + dev::kBlock - 1) / dev::kBlock, 16384);
+    const int tapBlocks = taps ? std::max(1, std::min(16, launch::ceilDiv(tapEntries, dev::kBlock))) : 0;
+    padPlanesFlatKernel<true><<<copyBlocks + tapBlocks, dev::kBlock, 0, s>>>(x, xp, H, W, padTop, padLeft, Hp, Wp, total,
+                                                                            copyBlocks, taps, tapEntries, g);
   } else if (plane % 4 == 0 && launch::aligned16(xp))
     padPlanesKernel<true><<<dim3(gx, launch::ceilDiv(plane / 4, dev::kBlock)), dev::kBlock, 0, s>>>(
         x, xp, H, W, padTop, padLeft, Hp, Wp, (int)planes, taps, tapEntries, g);

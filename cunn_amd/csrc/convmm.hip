@@ -360,6 +360,10 @@ struct FwdArgs {
   int full, tail;
   float *partial;
   int relu;           // != 0: the stored value is v > 0 ? v : 0 (Threshold(0, 0) applied to the output)
+  // padded kernel: the output spans fewer than 2^31 bytes (outBytes) - whole row tiles are then stored with a
+  // per-lane column offset and a scalar row offset, no address arithmetic on the vector ALU
+  int outBytes;       // 0: not applicable
+  unsigned magicL, magicOW;  // reciprocals of L and oW (dev::magicOf), 0: divide
   const int *taps;    // padded kernel: byte offset of tap (c, kh, kw) inside a (zero-padded) image, per k
   int tapStride;      // > 0 (1x1 windows): tap k sits at byte offset k * tapStride, no table is read
 };
@@ -368,10 +372,19 @@ struct FwdArgs {
 // 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 accumulator tile. Split workgroups store their
 // partial tile, the others add the bias and store to out(n, row, l).
 // biasLds: the tile's bias values in LDS (index = row - m0, zeros where there is no bias or row), or null.
+// column (n, l) -> (n, oh, ow): through the reciprocals when the launch provides them
+__device__ __forceinline__ void splitColumn(const FwdArgs &p, const ConvGeom &g, unsigned col, int &n, int &oh, int &ow) {
+  n = p.magicL ? dev::fastDiv((int)col, p.magicL) : (int)(col / (unsigned)g.L);
+  const int l = (int)col - n * g.L;
+  oh = p.magicOW ? dev::fastDiv(l, p.magicOW) : l / g.oW;
+  ow = l - oh * g.oW;
+}
+
+// biasDone: the accumulators started from the bias (whole tiles of the padded kernel)
 template <int TBN = BN, int TI = 2>
 __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g, const float16v (&acc)[TI][2], int bx,
                                             int by, int m0, int j0, int wm, int wn, int grp, int idx,
-                                            const float *biasLds = nullptr, int toPartial = -1) {
+                                            const float *biasLds = nullptr, int toPartial = -1, bool biasDone = false) {
   const int rowHalf = grp * 4;
   if (toPartial < 0 ? p.nSplit > 1 : toPartial != 0) {
     float *dst = p.partial + ((long)bx * p.nSplit + by) * (BM * BN);  // both tile shapes hold BM * BN elements
@@ -382,6 +395,31 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
 #pragma unroll
         for (int v = 0; v < 16; ++v)
           dst[(wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3)) * TBN + wn * 64 + tj * 32 + idx] = acc[ti][tj][v];
+    return;
+  }
+  if (biasDone && p.outBytes > 0 && m0 + wm * 64 + TI * 32 <= p.M) {
+    // every row of the wave exists: 64 stores of (per-lane column offset, scalar row offset); a column past the
+    // batch is an offset out of range
+    const __amdgpu_buffer_rsrc_t orr = dev::makeRsrc(p.out, p.outBytes);
+    const int rowBase = __builtin_amdgcn_readfirstlane(m0 + wm * 64);
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+      const unsigned col = (unsigned)j0 + wn * 64 + tj * 32 + idx;
+      int n, oh, ow;
+      splitColumn(p, g, min(col, (unsigned)p.Ncols - 1), n, oh, ow);
+      const int voff = col < (unsigned)p.Ncols
+                           ? (int)(((long)n * p.outImg + (long)oh * p.outSH + ow * p.outSW + (long)rowHalf * p.outRow) * 4)
+                           : dev::kBufOob;
+#pragma unroll
+      for (int ti = 0; ti < TI; ++ti)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          float o = acc[ti][tj][v];
+          if (p.relu) o = o > 0.f ? o : 0.f;
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(o), orr, voff,
+                                                (rowBase + ti * 32 + 8 * (v >> 2) + (v & 3)) * p.outRow * 4, 0);
+        }
+    }
     return;
   }
   auto store = [&](auto withBias) {
@@ -410,9 +448,8 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
     for (int tj = 0; tj < 2; ++tj) {
       const unsigned col = (unsigned)j0 + wn * 64 + tj * 32 + idx;  // Ncols < 2^31
       if (col >= (unsigned)p.Ncols) continue;
-      const unsigned n = col / (unsigned)g.L;
-      const int l = (int)(col - n * (unsigned)g.L);
-      const int oh = l / g.oW, ow = l - oh * g.oW;
+      int n, oh, ow;
+      splitColumn(p, g, col, n, oh, ow);
       float *dst = p.out + (long)n * p.outImg + (long)oh * p.outSH + ow * p.outSW;
 #pragma unroll
       for (int ti = 0; ti < TI; ++ti)
@@ -425,7 +462,7 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
         }
     }
   };
-  if (p.bias)
+  if (p.bias && !biasDone)
     store(std::true_type{});
   else
     store(std::false_type{});
@@ -817,12 +854,6 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   if (t < TBM) biasS[t] = p.bias && m0 + t < p.M ? p.bias[m0 + t] : 0.f;  // visible after the first barrier
 
   float16v acc[TI][2];
-#pragma unroll
-  for (int i = 0; i < TI; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc((void *)p.w, 0, p.wBytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.xBytes, 0x00020000);
@@ -838,9 +869,8 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   int posOff;
   {
     const unsigned lg = min((unsigned)j0 + colB, (unsigned)p.Ncols - 1);  // Ncols < 2^31
-    const int n = (int)(lg / (unsigned)g.L);
-    const int l = (int)(lg - (unsigned)n * (unsigned)g.L);
-    const int oh = l / g.oW, ow = l - oh * g.oW;
+    int n, oh, ow;
+    splitColumn(p, g, lg, n, oh, ow);
     posOff = ((n * g.Cin * g.H + oh * g.dH) * g.W + ow * g.dW) * 4;
   }
   const int ktBegin = by * p.ktPerSplit;  // by == 0 for whole tiles
@@ -921,6 +951,19 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
     loadTaps(ktBegin + 2);
   }
   __syncthreads();
+  // the accumulators of a whole tile start from the bias (in LDS since the barrier): no addition in the epilogue
+  {
+    const int grpRow = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (whole) b4 = *reinterpret_cast<const float4 *>(biasS + wm * 64 + i * 32 + 8 * q + grpRow);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j][4 * q] = b4.x, acc[i][j][4 * q + 1] = b4.y, acc[i][j][4 * q + 2] = b4.z, acc[i][j][4 * q + 3] = b4.w;
+      }
+  }
   int kt = ktBegin;
   for (; kt + 3 < nkt; kt += 2) {  // tile kt sits in buffer 0, tile kt + 1 in registers
     step(Buf0{}, Buf1{}, kt, true, true);
@@ -930,7 +973,7 @@ __device__ __forceinline__ void fwdPaddedBody(const FwdArgs &p, const ConvGeom &
   step(Buf0{}, Buf1{}, kt, kt + 1 < nkt, kt + 2 < nkt);
   if (kt + 1 < nkt) step(Buf1{}, Buf0{}, kt + 1, kt + 2 < nkt, false);
   if (kt + 2 < nkt) step(Buf0{}, Buf1{}, kt + 2, false, false);
-  fwdEpilogue<TBN, TI>(p, g, acc, bx, by, m0, j0, wm, wn, grp, idx, biasS, whole ? 0 : 1);
+  fwdEpilogue<TBN, TI>(p, g, acc, bx, by, m0, j0, wm, wn, grp, idx, biasS, whole ? 0 : 1, whole);
 }
 
 template <int WM, bool LINEAR = false>
@@ -1715,6 +1758,14 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
   p.M = M;
   p.Ncols = nImages * g.L;
   p.outImg = (long)M * g.L, p.outRow = g.L, p.outSH = g.oW, p.outSW = 1;
+  if (fast) {
+    const long span = ((long)(nImages - 1) * p.outImg + (long)(M - 1) * p.outRow + (long)(g.oH - 1) * p.outSH +
+                       (long)(g.oW - 1) * p.outSW + 1) * 4;
+    p.outBytes = span < 0x7fffffffL ? (int)span : 0;
+    // (the reciprocal division is exact while dividend * divisor < 2^32)
+    p.magicL = (long)p.Ncols * g.L < 0xffffffffL ? dev::magicOf(g.L) : 0;
+    p.magicOW = (long)g.L * g.oW < 0xffffffffL ? dev::magicOf(g.oW) : 0;
+  }
   p.xBytes = (int)((long)nImages * gk.Cin * gk.H * gk.W * sizeof(float));
   p.wBytes = (int)((long)M * gk.K * sizeof(float));
   p.vecA = (gk.K % 4 == 0) && launch::aligned16(w);
@@ -2003,6 +2054,13 @@ bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const
       a.Ncols = cnt * gk.L;
       a.out = gi + (long)n0 * g.Cin * g.H * g.W + (long)P.h0 * g.W + P.w0;
       a.outImg = (long)g.Cin * g.H * g.W, a.outRow = g.H * g.W, a.outSH = g.dH * g.W, a.outSW = g.dW;
+      {
+        const long span = ((long)(cnt - 1) * a.outImg + (long)(g.Cin - 1) * a.outRow + (long)(P.h.n - 1) * a.outSH +
+                           (long)(P.w.n - 1) * a.outSW + 1) * 4;
+        a.outBytes = span < 0x7fffffffL ? (int)span : 0;
+        a.magicL = (long)a.Ncols * gk.L < 0xffffffffL ? dev::magicOf(gk.L) : 0;
+        a.magicOW = (long)gk.L * gk.oW < 0xffffffffL ? dev::magicOf(gk.oW) : 0;
+      }
       a.xBytes = (int)(cnt * imgFloats * 4);
       a.wBytes = (int)((long)g.Cin * P.Kp * 4);
       a.vecA = true;

@@ -1076,6 +1076,7 @@ struct GradWeightArgs {
   int totalKt, ktPerSplit;  // k-tiles of BK positions over the N*L positions; per split
   int gyBytes, xBytes;      // < 2^31
   unsigned magicOW;
+  unsigned magicKK, magicKW;  // reciprocals of kH * kW and kW (dev::magicOf)
   int Lvalid;               // positions of an image (g.L may count the padding of the gradOutput rows)
 };
 
@@ -1141,9 +1142,9 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   const int imgStrideA = p.M * g.L * 4;
   int nA, lA;  // L16: scalar image and position of the k-tile; else: of this lane's first group
   {
-    const long r = (long)ktBegin * BK + (L16 ? 0 : pgA * 4);
-    nA = (int)(r / g.L);
-    lA = (int)(r - (long)nA * g.L);
+    const unsigned r = (unsigned)ktBegin * BK + (L16 ? 0 : pgA * 4);  // N * L < 2^31
+    nA = (int)(r / (unsigned)g.L);
+    lA = (int)(r - (unsigned)nA * (unsigned)g.L);
   }
   // ---- B loader: position t & 15 of the k-tile, columns (t >> 4) + 16 i
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.xBytes, 0x00020000);
@@ -1154,8 +1155,8 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       const int k = min(j0 + cB + 16 * i, p.Ncols - 1);  // columns past K are dropped in the epilogue
-      const int c = k / KK, rem = k - c * KK;
-      const int kh = rem / g.kW, kw = rem - kh * g.kW;
+      const int c = dev::fastDiv(k, p.magicKK), rem = k - c * KK;
+      const int kh = dev::fastDiv(rem, p.magicKW), kw = rem - kh * g.kW;
       tapOff[i] = ((c * g.H + kh * g.dilH) * g.W + kw * g.dilW) * 4;
     }
   }
@@ -1163,9 +1164,9 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   const int rowStepB = g.dH * g.W * 4, colStepB = g.dW * 4;
   int lB, nOffB;  // position inside the image, byte offset of the image (>= xBytes past the batch: loads return 0)
   {
-    const long r = (long)ktBegin * BK + rB;
-    const int n = (int)(r / g.L);
-    lB = (int)(r - (long)n * g.L);
+    const unsigned r = (unsigned)ktBegin * BK + rB;
+    const int n = (int)(r / (unsigned)g.L);
+    lB = (int)(r - (unsigned)n * (unsigned)g.L);
     nOffB = n * imgStrideB;
   }
 
@@ -2427,6 +2428,7 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     q.gyBytes = (int)gyBytes;
     q.xBytes = (int)(xpFloats * 4);
     q.magicOW = dev::magicOf(g.oW);
+    q.magicKK = dev::magicOf(g.kH * g.kW), q.magicKW = dev::magicOf(g.kW);
     q.Lvalid = g.L;
     const dim3 grid(mT * nT * wgSplits);
     if (tiny)

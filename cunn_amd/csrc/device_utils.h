@@ -84,6 +84,11 @@ __device__ __forceinline__ float4 bufLoad4(__amdgpu_buffer_rsrc_t r, int byteOff
   u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byteOff, 0, 0);
   return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
 }
+// the same with the non-temporal hint: for the last reader of a tensor
+__device__ __forceinline__ float4 bufLoadStream4(__amdgpu_buffer_rsrc_t r, int byteOff) {
+  u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byteOff, 0, 2);
+  return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+}
 __device__ __forceinline__ void bufStore4(__amdgpu_buffer_rsrc_t r, int byteOff, float4 f) {
   u32x4 v = {__float_as_uint(f.x), __float_as_uint(f.y), __float_as_uint(f.z), __float_as_uint(f.w)};
   __builtin_amdgcn_raw_buffer_store_b128(v, r, byteOff, 0, 0);

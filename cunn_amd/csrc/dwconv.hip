@@ -568,12 +568,12 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
   const int nMul = ONE ? 1 : g.M;
   if (ONE) {
     typename S::InFlight fl;
-    S::issue(fl, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
+    S::template issue<true>(fl, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
     const int n4 = (nOut * g.oW) >> 2;
     const __amdgpu_buffer_rsrc_t rs = dev::makeRsrc(gradOut + ((long)plane * g.oH + oh0) * g.oW, (long)n4 * 16);
     float4 gv[dev::kLoadBatch];
 #pragma unroll
-    for (int u = 0; u < dev::kLoadBatch; ++u) gv[u] = dev::bufLoad4(rs, (u * dev::kBlock + threadIdx.x) * 16);  // past the end reads 0
+    for (int u = 0; u < dev::kLoadBatch; ++u) gv[u] = dev::bufLoadStream4(rs, (u * dev::kBlock + threadIdx.x) * 16);  // past the end reads 0
     S::commit(smem, fl, g.W, nIn);
 #pragma unroll
     for (int u = 0; u < dev::kLoadBatch; ++u) {

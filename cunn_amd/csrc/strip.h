@@ -95,6 +95,7 @@ struct Strip {
     float4 v[kLoadBatch];
     int off[kLoadBatch];
   };
+  template <bool STREAM = false>
   __device__ static void issue(InFlight &f, const float *plane, int H, int W, int r0, int nRows) {
     const int tid = threadIdx.x, nt = blockDim.x;
     const int W4 = W >> 2, total = nRows * W4;
@@ -108,7 +109,8 @@ struct Strip {
       const int gr = r0 + r;
       const bool ok = i < total && (unsigned)gr < (unsigned)H;
       f.off[u] = (i < total) ? r * p + kStripPadL + (ST == 1 ? (c4 << 2) : (c4 << 1)) : -1;
-      f.v[u] = bufLoad4(rs, ok ? (gr * W + (c4 << 2)) * 4 : kBufOob);
+      f.v[u] = STREAM ? bufLoadStream4(rs, ok ? (gr * W + (c4 << 2)) * 4 : kBufOob)
+                      : bufLoad4(rs, ok ? (gr * W + (c4 << 2)) * 4 : kBufOob);
     }
   }
   __device__ static void commit(float *dst, const InFlight &f, int W, int nRows) {

@@ -638,7 +638,7 @@ poolBwdStrip(const float *__restrict__ gradOut, const long *__restrict__ indices
       int r = dev::fastDiv(i, magicPitch), cc = i - r * pitch - dev::kStripPadL;
       int ph = ph0 + r;
       int v = -2;
-      if (cc >= 0 && r < stageRows && ph >= 0 && ph < g.oH) v = (int)(ip[(long)ph * g.oW + cc] - TH_INDEX_BASE);
+      if (cc >= 0 && r < stageRows && ph >= 0 && ph < g.oH) v = (int)(__builtin_nontemporal_load(ip + (long)ph * g.oW + cc) - TH_INDEX_BASE);
       is[i] = __int_as_float(v);
     }
   } else {

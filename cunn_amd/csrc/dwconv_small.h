@@ -102,8 +102,9 @@ dwSmallAccGrad(const float *__restrict__ in, const float *__restrict__ gradOut, 
   const int oPlane = g.oH * g.oW;
   const long gFirst = (long)b.q0 * oPlane + b.o0 * g.oW;
   SmallRun run, grun;
-  smallIssue(run, in, (long)b.q0 * g.sH * g.sW + b.rLo * g.sW, b.np * b.nr * g.sW, g.srcFloats);
-  smallIssue(grun, gradOut, gFirst, b.np * b.nOut * g.oW, g.outFloats);
+  // (both tensors are read here for the last time in a training step)
+  smallIssue<true>(run, in, (long)b.q0 * g.sH * g.sW + b.rLo * g.sW, b.np * b.nr * g.sW, g.srcFloats);
+  smallIssue<true>(grun, gradOut, gFirst, b.np * b.nOut * g.oW, g.outFloats);
   smallZero(xs, g.xsFloats);
   __syncthreads();
   smallScatter<1, PAD>(xs, run, b, g);

@@ -61,6 +61,8 @@ struct SmallRun {
   int lead, count;
 };
 // tensor: first element of the tensor (16-byte aligned); first: index of the run's first element; total: elements of the tensor
+// STREAM: with the non-temporal hint (the run's last reader)
+template <bool STREAM = false>
 __device__ __forceinline__ void smallIssue(SmallRun &r, const float *__restrict__ tensor, long first, int count, long total) {
   r.lead = (int)(first & 3), r.count = count;
   const float *base = tensor + (first - r.lead);
@@ -70,7 +72,8 @@ __device__ __forceinline__ void smallIssue(SmallRun &r, const float *__restrict_
 #pragma unroll
   for (int u = 0; u < dev::kLoadBatch; ++u) {
     const int e = (u * dev::kBlock + (int)threadIdx.x) * 4;
-    r.v[u] = dev::bufLoad4(rs, e + 4 <= span ? e * 4 : dev::kBufOob);
+    r.v[u] = STREAM ? dev::bufLoadStream4(rs, e + 4 <= span ? e * 4 : dev::kBufOob)
+                    : dev::bufLoad4(rs, e + 4 <= span ? e * 4 : dev::kBufOob);
     if (e < span && e + 4 > span) {  // the last, partial group of the run: whole if the tensor goes on, else by element
       if (e + 4 <= avail) {
         r.v[u] = *reinterpret_cast<const float4 *>(base + e);
@@ -141,6 +144,8 @@ struct SmallIdxRun {
   long2 v[2 * dev::kLoadBatch];
   int lead, count;
 };
+typedef long i64x2v __attribute__((ext_vector_type(2)));
+template <bool STREAM = false>
 __device__ __forceinline__ void smallIssueIdx(SmallIdxRun &r, const long *__restrict__ tensor, long first, int count, long total) {
   r.lead = (int)(first & 1), r.count = count;
   const long *base = tensor + (first - r.lead);
@@ -150,8 +155,14 @@ __device__ __forceinline__ void smallIssueIdx(SmallIdxRun &r, const long *__rest
   for (int u = 0; u < 2 * dev::kLoadBatch; ++u) {
     const int e = (u * dev::kBlock + (int)threadIdx.x) * 2;
     r.v[u] = make_long2(0, 0);
-    if (e + 2 <= span || (e < span && e + 2 <= avail))
-      r.v[u] = *reinterpret_cast<const long2 *>(base + e);
+    if (e + 2 <= span || (e < span && e + 2 <= avail)) {
+      if (STREAM) {
+        const i64x2v q = __builtin_nontemporal_load(reinterpret_cast<const i64x2v *>(base + e));
+        r.v[u] = make_long2(q.x, q.y);
+      } else {
+        r.v[u] = *reinterpret_cast<const long2 *>(base + e);
+      }
+    }
     else if (e < span)
       r.v[u].x = base[e];
   }

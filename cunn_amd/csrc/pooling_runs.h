@@ -160,7 +160,7 @@ poolRunBwd(const float *__restrict__ gradOut, const long *__restrict__ indices, 
   SmallRun run;
   SmallIdxRun irun;
   smallIssue(run, gradOut, srcFirst, srcCount, g.srcFloats);
-  if (MAX) smallIssueIdx(irun, indices, srcFirst, srcCount, g.srcFloats);
+  if (MAX) smallIssueIdx<true>(irun, indices, srcFirst, srcCount, g.srcFloats);  // their only use
   smallZero(gs, g.xsFloats);
   if (MAX) smallFill(reinterpret_cast<float *>(is), g.xsFloats, __int_as_float(-1));
   __syncthreads();

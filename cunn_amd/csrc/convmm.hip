@@ -1606,9 +1606,6 @@ void planTiles(FwdPlan &pl, int M, long Ncols, int nkt, bool wideOk) {
   // element it gathers)
   const bool low = wideOk && tiles(M, 32) * 32 * 4 <= tiles(M, 64) * 64 * 3;
   pl.bm = low ? 32 : wide ? 64 : BM, pl.bn = low || wide ? 256 : BN;
-  if (const char *e = getenv("THCUNN_XBM")) {  // EXPERIMENT
-    if (wideOk && atoi(e) > 0) pl.bm = atoi(e), pl.bn = pl.bm == 128 ? 128 : 256;
-  }
   pl.mTiles = (int)tiles(M, pl.bm);
   pl.total = pl.mTiles * (int)tiles(Ncols, pl.bn);
   const int cus = residentSlots(nullptr);

@@ -50,9 +50,9 @@ def _traffic(*kernels):
 
 MEASURED_TRAFFIC_BYTES = {
     ("cfg1", "dw_updateOutput"): _traffic((26658.6, 50207.7)),
-    ("cfg2", "dw_updateOutput"): _traffic((50224.5, 25123.4)),
-    ("cfg2", "dw_updateGradInput"): _traffic((12836.5, 100354.0)),
-    ("cfg2", "dw_accGradParameters"): _traffic((63007.5, 512.0), (541.0, 12.0)),
+    ("cfg2", "dw_updateOutput"): _traffic((50222.7, 25130.5)),
+    ("cfg2", "dw_updateGradInput"): _traffic((12840.5, 100352.0)),
+    ("cfg2", "dw_accGradParameters"): _traffic((63024.6, 512.0), (558.5, 12.0)),
     ("cfg3", "bn_updateOutput"): _traffic((25722.0, 51041.0)),
     ("cfg3", "bn_backward"): _traffic((56377.2, 51211.0)),
     ("cfg4", "maxpool_updateOutput"): _traffic((103481.2, 150592.2)),
@@ -60,9 +60,9 @@ MEASURED_TRAFFIC_BYTES = {
     ("cfg4", "avgpool_updateOutput"): _traffic((101707.4, 50176.0)),
     ("cfg4", "avgpool_updateGradInput"): _traffic((30467.5, 200744.3)),
     # bordered copy + GEMM + tail fold (+ flipped weights for gradInput; + partial fold for the weight gradient)
-    ("cfg5", "convmm_updateOutput"): _traffic((25983.0, 57606.1), (109420.3, 68419.4), (8237.0, 1024.0)),
-    ("cfg5", "convmm_updateGradInput"): _traffic((25983.0, 57606.1), (109420.3, 68419.4), (8237.0, 1024.0), (5180.1, 2304.0)),
-    ("cfg5", "convmm_accGradParameters"): _traffic((25983.0, 57606.1), (70844.7, 48405.0), (25371.6, 2305.0)),
+    ("cfg5", "convmm_updateOutput"): _traffic((25978.1, 57606.1), (109212.5, 67553.5), (8239.5, 1024.0)),
+    ("cfg5", "convmm_updateGradInput"): _traffic((25978.1, 57606.1), (109212.5, 67553.5), (8239.5, 1024.0), (5176.1, 2304.0)),
+    ("cfg5", "convmm_accGradParameters"): _traffic((25978.1, 57606.1), (70327.3, 48405.0), (25371.7, 2305.0)),
 }
 
 

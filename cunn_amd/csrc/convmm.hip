@@ -630,41 +630,40 @@ struct PhaseSet {
   int count;
 };
 
-// Phase weights Wp(Cin x Kp): Wp[c][(o, a, b)] = w[o][c][h.k0 + a*h.kStep][w.k0 + b*w.kStep], zero from K to Kp.
-// grid = (chunks, phases)
+// Phase weights Wp(Cin x Kp): Wp[c][(o, a, b)] = w[o][c][h.k0 + a*h.kStep][w.k0 + b*w.kStep], zero from K to Kp, and the
+// tap table of each phase: entry k = (o, a, b) is the byte offset of gy element (o, q0h - a*qStepH, q0w - b*qStepW) of
+// the bordered image, 0 from K on.
+// grid = (chunks of a weight row, Cin + 1, phases): blocks with blockIdx.y == Cin write the tap table.
 __global__ void __launch_bounds__(dev::kBlock)
-phaseWeightsKernel(const float *__restrict__ w, float *__restrict__ dst, PhaseSet set, int Cin, int kH, int kW) {
-  const Phase &P = set.ph[blockIdx.y];
-  const long total = (long)Cin * P.Kp;
-  const int taps = P.h.nk * P.w.nk;
-  float *d = dst + P.wOfs;
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
-    const int k = (int)(i % P.Kp);
-    const int c = (int)(i / P.Kp);
+phaseSetupKernel(const float *__restrict__ w, float *__restrict__ dst, int *__restrict__ taps, PhaseSet set, int Cin, int kH,
+                 int kW, int Hp, int Wp, int top, int left) {
+  const Phase &P = set.ph[blockIdx.z];
+  const int tp = P.h.nk * P.w.nk;
+  const unsigned magicTp = dev::magicOf(tp), magicNk = dev::magicOf(P.w.nk);
+  const int c = blockIdx.y;
+  if (c == Cin) {
+    const int entries = P.Kp + 2 * BK;
+    int *d = taps + P.tapOfs;
+    for (int k = blockIdx.x * dev::kBlock + threadIdx.x; k < entries; k += gridDim.x * dev::kBlock) {
+      int v = 0;
+      if (k < P.K) {
+        const int o = dev::fastDiv(k, magicTp), r = k - o * tp;
+        const int a = dev::fastDiv(r, magicNk), b = r - a * P.w.nk;
+        v = ((o * Hp + top + P.h.q0 - a * P.h.qStep) * Wp + left + P.w.q0 - b * P.w.qStep) * 4;
+      }
+      d[k] = v;
+    }
+    return;
+  }
+  float *d = dst + P.wOfs + (long)c * P.Kp;
+  const long oStride = (long)Cin * kH * kW;
+  const float *src = w + ((long)c * kH + P.h.k0) * kW + P.w.k0;
+  for (int k = blockIdx.x * dev::kBlock + threadIdx.x; k < P.Kp; k += gridDim.x * dev::kBlock) {
     float v = 0.f;
     if (k < P.K) {
-      const int o = k / taps, r = k - o * taps;
-      const int a = r / P.w.nk, b = r - a * P.w.nk;
-      v = w[(((long)o * Cin + c) * kH + P.h.k0 + a * P.h.kStep) * kW + P.w.k0 + b * P.w.kStep];
-    }
-    d[i] = v;
-  }
-}
-
-// Tap tables of the phases: byte offset of (o, a, b) inside a bordered gy image (Hp x Wp planes, gy at
-// row top, column left), relative to the position's own (i, j); 0 for the entries beyond K.
-__global__ void __launch_bounds__(dev::kBlock)
-phaseTapsKernel(int *__restrict__ taps, PhaseSet set, int Hp, int Wp, int top, int left) {
-  const Phase &P = set.ph[blockIdx.y];
-  const int entries = P.Kp + 2 * BK;
-  const int tp = P.h.nk * P.w.nk;
-  int *d = taps + P.tapOfs;
-  for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < entries; k += gridDim.x * blockDim.x) {
-    int v = 0;
-    if (k < P.K) {
-      const int o = k / tp, r = k - o * tp;
-      const int a = r / P.w.nk, b = r - a * P.w.nk;
-      v = ((o * Hp + top + P.h.q0 - a * P.h.qStep) * Wp + left + P.w.q0 - b * P.w.qStep) * 4;
+      const int o = dev::fastDiv(k, magicTp), r = k - o * tp;
+      const int a = dev::fastDiv(r, magicNk), b = r - a * P.w.nk;
+      v = src[o * oStride + (a * P.h.kStep) * kW + b * P.w.kStep];
     }
     d[k] = v;
   }
@@ -2021,9 +2020,14 @@ bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const
   float *wph = buf + tapTotal;
   float *partial = wph + wTotal;
   float *gyp = partial + partialTotal;
-  phaseTapsKernel<<<dim3(8, set.count), dev::kBlock, 0, s>>>(taps, set, (int)Hp, (int)Wp, top, left);
-  THC_HIP_CHECK(hipGetLastError());
-  phaseWeightsKernel<<<dim3(64, set.count), dev::kBlock, 0, s>>>(w, wph, set, g.Cin, g.kH, g.kW);
+  {
+    int maxKp = 0;
+    for (int i = 0; i < set.count; ++i) maxKp = std::max(maxKp, set.ph[i].Kp);
+    if (g.Cin + 1 > 65535) return false;
+    const int chunks = std::max(1, std::min(8, launch::ceilDiv(maxKp + 2 * BK, 4 * dev::kBlock)));
+    phaseSetupKernel<<<dim3(chunks, g.Cin + 1, set.count), dev::kBlock, 0, s>>>(w, wph, taps, set, g.Cin, g.kH, g.kW, (int)Hp,
+                                                                              (int)Wp, top, left);
+  }
   THC_HIP_CHECK(hipGetLastError());
   for (int n0 = 0; n0 < g.N; n0 += group) {
     const int cnt = std::min(group, g.N - n0);

@@ -338,6 +338,7 @@ convGemmKernel(GemmArgs p, ConvGeom g) {
 constexpr int FPITCH = BM + 8;  // float4 per k-group row: +8 keeps the 2 k-groups a lane pair writes in disjoint banks
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 struct FwdArgs {
   const float *w;     // (M x K) row-major
@@ -345,6 +346,9 @@ struct FwdArgs {
   float *out;         // element (n, row, oh, ow) at out[n * outImg + row * outRow + oh * outSH + ow * outSW]
   long outImg;        // dense output (nImages, M, oH, oW): M * L, L, oW, 1
   int outRow, outSH, outSW;
+  // != 0 (outSW == 2, outSH == 2 * row length): every element is the top-left corner of a 2 x 2 block of out
+  // whose other three elements get the bias (or 0) - the gradInput of a 1x1 convolution with stride 2
+  int dilate;
   const float *bias;  // M or null
   int M, Ncols;       // Ncols = nImages * L
   int mTiles;
@@ -416,8 +420,17 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
         for (int v = 0; v < 16; ++v) {
           float o = acc[ti][tj][v];
           if (p.relu) o = o > 0.f ? o : 0.f;
-          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(o), orr, voff,
-                                                (rowBase + ti * 32 + 8 * (v >> 2) + (v & 3)) * p.outRow * 4, 0);
+          const int soff = (rowBase + ti * 32 + 8 * (v >> 2) + (v & 3)) * p.outRow * 4;
+          if (p.dilate) {
+            // the element and its right neighbour, then the two below: 8-byte stores, a wave covers whole rows
+            const float z = biasLds ? biasLds[wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3)] : 0.f;
+            const u32x2 top = {__float_as_uint(o), __float_as_uint(z)}, bottom = {__float_as_uint(z), __float_as_uint(z)};
+            const int below = col < (unsigned)p.Ncols ? voff + (p.outSH >> 1) * 4 : dev::kBufOob;
+            __builtin_amdgcn_raw_buffer_store_b64(top, orr, voff, soff, 0);
+            __builtin_amdgcn_raw_buffer_store_b64(bottom, orr, below, soff, 0);
+          } else {
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(o), orr, voff, soff, 0);
+          }
         }
     }
     return;
@@ -458,7 +471,14 @@ __device__ __forceinline__ void fwdEpilogue(const FwdArgs &p, const ConvGeom &g,
           const int row = m0 + wm * 64 + ti * 32 + 8 * (v >> 2) + rowHalf + (v & 3);
           float o = BIAS ? acc[ti][tj][v] + bv[ti][v] : acc[ti][tj][v];
           if (p.relu) o = o > 0.f ? o : 0.f;
-          if (row < p.M) dst[(long)row * p.outRow] = o;
+          if (row < p.M) {
+            float *q = dst + (long)row * p.outRow;
+            q[0] = o;
+            if (p.dilate) {
+              const float z = p.bias ? p.bias[row] : 0.f;
+              q[1] = z, q[p.outSH >> 1] = z, q[(p.outSH >> 1) + 1] = z;
+            }
+          }
         }
     }
   };
@@ -1029,6 +1049,20 @@ __device__ __forceinline__ void fwdTailFixupBody(const FwdArgs &p, const ConvGeo
 #pragma unroll
     for (int i = 0; i < 4; ++i) vals[i] = vals[i] > 0.f ? vals[i] : 0.f;
   }
+  if (p.dilate) {
+    // four neighbouring columns of one output row: their 2 x 2 blocks are 8 consecutive floats of two rows of out
+    const long col = (long)nTile * p.bn + c;
+    const int n = (int)(col / g.L);
+    const int l = (int)(col - (long)n * g.L);
+    const int oh = l / g.oW, ow = l - oh * g.oW;
+    float *q = p.out + (long)n * p.outImg + (long)row * p.outRow + (long)oh * p.outSH + ow * 2;
+    if (col + 3 < p.Ncols && ow + 3 < g.oW && ((uintptr_t)q & 15) == 0 && (p.outSH & 7) == 0) {
+      float4 *top = reinterpret_cast<float4 *>(q), *bottom = reinterpret_cast<float4 *>(q + (p.outSH >> 1));
+      top[0] = make_float4(vals[0], b, vals[1], b), top[1] = make_float4(vals[2], b, vals[3], b);
+      bottom[0] = bottom[1] = make_float4(b, b, b, b);
+      return;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const long col = (long)nTile * p.bn + c + i;
@@ -1036,7 +1070,9 @@ __device__ __forceinline__ void fwdTailFixupBody(const FwdArgs &p, const ConvGeo
     const int n = (int)(col / g.L);
     const int l = (int)(col - (long)n * g.L);
     const int oh = l / g.oW, ow = l - oh * g.oW;
-    p.out[(long)n * p.outImg + (long)row * p.outRow + (long)oh * p.outSH + ow * p.outSW] = vals[i];
+    float *q = p.out + (long)n * p.outImg + (long)row * p.outRow + (long)oh * p.outSH + ow * p.outSW;
+    q[0] = vals[i];
+    if (p.dilate) q[1] = b, q[p.outSH >> 1] = b, q[(p.outSH >> 1) + 1] = b;
   }
 }
 
@@ -1713,8 +1749,16 @@ void launchFwdKernels(hipStream_t s, const FwdPlan &pl, FwdArgs p, float *partia
 }
 
 // out(nImages, M, L) = bias + W(M x K) * im2col(x); `scratch` holds plan.scratchFloats floats
+// Where the output elements go when not into a dense (nImages, M, oH, oW) tensor.
+struct OutMap {
+  long outImg;
+  int outRow, outSH, outSW;
+  int dilate;  // FwdArgs::dilate
+};
+
 void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const float *w, const float *x, float *out,
-                       const float *bias, int M, int nImages, const ConvGeom &g, bool relu = false) {
+                       const float *bias, int M, int nImages, const ConvGeom &g, bool relu = false,
+                       const OutMap *om = nullptr) {
   const bool fast = pl.tapEntries > 0;
   if (fast && !(launch::aligned16(scratch) && (pl.weightFloats > 0 || launch::aligned16(w))))
     error("SpatialConvolutionMM: internal error, convolution scratch or weights not 16-byte aligned");
@@ -1755,9 +1799,10 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
   p.M = M;
   p.Ncols = nImages * g.L;
   p.outImg = (long)M * g.L, p.outRow = g.L, p.outSH = g.oW, p.outSW = 1;
+  if (om) p.outImg = om->outImg, p.outRow = om->outRow, p.outSH = om->outSH, p.outSW = om->outSW, p.dilate = om->dilate;
   if (fast) {
     const long span = ((long)(nImages - 1) * p.outImg + (long)(M - 1) * p.outRow + (long)(g.oH - 1) * p.outSH +
-                       (long)(g.oW - 1) * p.outSW + 1) * 4;
+                       (long)(g.oW - 1) * p.outSW + 1 + (p.dilate ? p.outSH / 2 + 1 : 0)) * 4;
     p.outBytes = span < 0x7fffffffL ? (int)span : 0;
     // (the reciprocal division is exact while dividend * divisor < 2^32)
     p.magicL = (long)p.Ncols * g.L < 0xffffffffL ? dev::magicOf(g.L) : 0;
@@ -2194,6 +2239,38 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
   if (g.Cin <= 4 && (g.kH * g.kW > 1 || g.dH > 1 || g.dW > 1) && !forceGeneric() && (route == 0 || route == 3) &&
       convFewPlanesGradInput(state, g, gy, w, gi, bias, route == 3))
     return;
+  // 1x1 window, stride 2, no padding, even extents (the shortcut and reduction layers of a residual network):
+  // gradInput is W^T gradOutput at the even positions and the bias (or 0) everywhere else. One pointwise pass of
+  // the forward kernels over gradOutput whose epilogue writes each element's whole 2 x 2 block - contiguous
+  // 8-byte stores - instead of four phases that each write every other element of every other row.
+  if (g.kH == 1 && g.kW == 1 && g.dH == 2 && g.dW == 2 && g.padH == 0 && g.padW == 0 && g.H == 2 * g.oH && g.W == 2 * g.oW &&
+      route == 0 && !forceGeneric() && ((uintptr_t)gi & 7) == 0 && (long)g.Cout * g.oH * g.oW * 4 < (1L << 30) &&
+      (long)g.Cout * g.K < 0x7fffffffL / 4) {
+    ConvGeom t = g;
+    t.Cin = g.Cout, t.Cout = g.Cin;
+    t.H = t.oH = g.oH, t.W = t.oW = g.oW;
+    t.dH = t.dW = 1;
+    t.K = g.Cout;
+    t.L = g.oH * g.oW;
+    OutMap om{(long)g.Cin * g.H * g.W, g.H * g.W, 2 * g.W, 2, 1};
+    int group = (int)std::min<long>(g.N, std::max<long>(1, 0x7fffffffL / 2 / t.L));
+    group = (int)std::min<long>(group, std::max<long>(1, ((1L << 31) - 1 - 4096) / ((long)g.Cout * t.L * 4)));
+    FwdPlan pl = planFwdImplicit(t.Cout, std::min(group, g.N), t);
+    long need = pl.scratchFloats;
+    if (g.N % group != 0) need = std::max(need, planFwdImplicit(t.Cout, g.N % group, t).scratchFloats);
+    const long wfFloats = ((long)g.Cout * g.K + 3) / 4 * 4;
+    Temp tmp;
+    float *buf = scratchFloats(state, scratchBuf, wfFloats + need, tmp, bufName);
+    flipWeightKernel<<<launch::directGrid((long)g.Cout * g.K, dev::kBlock), dev::kBlock, 0, s>>>(w, buf, g.Cout, g.Cin, 1, 1);
+    THC_HIP_CHECK(hipGetLastError());
+    for (int n0 = 0; n0 < g.N; n0 += group) {
+      int cnt = std::min(group, g.N - n0);
+      if (cnt != std::min(group, g.N)) pl = planFwdImplicit(t.Cout, cnt, t);
+      launchFwdImplicit(s, pl, buf + wfFloats, buf, gy + (long)n0 * g.Cout * g.L, gi + (long)n0 * g.Cin * g.H * g.W, bias,
+                        t.Cout, cnt, t, false, &om);
+    }
+    return;
+  }
   if (g.dH == 1 && g.dW == 1 && tpH >= 0 && tpW >= 0 && exact && !sliver && !forceGeneric() && goImgBytes < (1L << 30) &&
       (long)g.Cout * g.K < 0x7fffffffL / 4) {
     ConvGeom t = g;  // the transposed problem

@@ -28,6 +28,11 @@ CASES = [
     (2, 64, 32, 14, 14, 1, 1, 0),    # gradWeight 32 x 64
     (4, 64, 64, 28, 28, 3, 1, 1),    # 13 tiles of 64 x 256: every tile split along K
     (9, 128, 128, 14, 14, 3, 1, 1),  # 14 tiles of 128 x 128
+    (2, 64, 128, 16, 16, 1, 2, 0),   # 1x1 stride 2, even extents: gradInput written as 2 x 2 blocks by one pointwise pass
+    (3, 20, 24, 10, 14, 1, 2, 0),    # the same with 20 rows (element-wise stores) and K = 24
+    (2, 40, 256, 8, 12, 1, 2, 0),    # 40 rows: a full 32-row tile and a partial one
+    (2, 256, 64, 8, 8, 1, 2, 0),     # every tile split along K: the blocks are written by the fold
+    (2, 64, 128, 15, 17, 1, 2, 0),   # odd extents: phase by phase
 ]
 
 
@@ -63,3 +68,25 @@ def test_conv_tile_shapes(case, bias):
     np.testing.assert_allclose(tgw.numpy(), rgw, rtol=1e-3, atol=1e-3, err_msg="gradWeight")
     if bias:
         np.testing.assert_allclose(tgb.numpy(), rgb, rtol=1e-3, atol=1e-3, err_msg="gradBias")
+
+
+@pytest.mark.parametrize("case", [(2, 96, 48, 9, 11), (3, 16, 20, 6, 6), (2, 128, 256, 7, 7)])
+@pytest.mark.parametrize("bias", [True, False])
+def test_transposed_1x1_stride2_forward(case, bias):
+    """SpatialFullConvolution (lib/THCUNN/generic/SpatialFullDilatedConvolution.cu:141-165) with a 1x1 window, stride 2 and
+    output padding 1: every input element lands on the top-left corner of a 2 x 2 output block, the rest is the bias."""
+    print("case", case, "bias", bias, flush=True)
+    N, Ci, Co, H, W = case
+    THNN, CT = cunn_amd.THNN, cunn_amd.CudaTensor
+    rng = np.random.default_rng(91)
+    x = rng.standard_normal((N, Ci, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Ci, Co, 1, 1)) * 0.2).astype(np.float32)
+    b = rng.standard_normal(Co).astype(np.float32) if bias else None
+    g = (1, 1, 2, 2, 0, 0, 1, 1)
+    ref = O.fullconv_updateOutput(x, w, b, 1, 1, 2, 2, 0, 0, adjW=1, adjH=1)
+    out = CT()
+    THNN.SpatialFullConvolution_updateOutput(CT.from_numpy(x), out, CT.from_numpy(w), CT.from_numpy(b) if bias else None,
+                                             CT(), CT(), *g)
+    got = out.numpy()
+    assert got.shape == ref.shape == (N, Co, 2 * H, 2 * W)
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-4)

@@ -1135,16 +1135,22 @@ __device__ __forceinline__ void mfmaGroupPair(const float *aSrc, const float *bS
 }
 
 // (TI, TJ): 32-row and 32-column blocks of a small tile (WMODE = 0 only): 64 x 64, 32 x 64, 32 x 128, 64 x 32 ...
-template <bool L16, int WMODE, int TI = 2, int TJ = 2>
+// B4: 4 consecutive positions of a column are 4 consecutive floats of the image (unit stride along the row, and the
+// 4 positions never straddle two output rows - or the rows follow each other without a gap): a lane then fetches
+// one such group for each of its columns with one 16-byte load (any 4-byte alignment) and parks it with one
+// ds_write_b128, a quarter of the instructions of the element-wise gather.
+template <bool L16, int WMODE, int TI = 2, int TJ = 2, bool B4 = false>
 __global__ void __launch_bounds__(dev::kBlock, 3)
 convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   constexpr bool TINY = WMODE == 0;
   static_assert(TINY || (TI == 2 && TJ == 2), "block counts are a parameter of the small tiles only");
+  static_assert(!(TINY && B4), "the small tiles gather element by element");
   constexpr int WM = TINY ? 1 : WMODE;  // loader layout: 64 rows as in the 64 x 256 shape
   constexpr int TBM = TINY ? 32 * TI : 64 * WM, TBN = TINY ? 32 * TJ : 256 / WM;
   constexpr int AP = TBM + 8;   // float4 per position-group row of As
   constexpr int GP = TBN + 4;   // of Bs: the 4 groups of a wave's scalar stores hit disjoint banks
-  constexpr int NB = TBN / 16;  // columns a lane gathers per k-tile
+  constexpr int NB = B4 ? TBN / 64 : TBN / 16;  // columns a lane gathers per k-tile
+  constexpr int CS = B4 ? 64 : 16;              // distance between a lane's columns
   __shared__ float4 As[2][BK / 4][AP];
   __shared__ float4 Bs[2][BK / 4][GP];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -1182,14 +1188,15 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
     lA = (int)(r - (unsigned)nA * (unsigned)g.L);
   }
   // ---- B loader: position t & 15 of the k-tile, columns (t >> 4) + 16 i
+  //      (B4: positions 4 * (t & 3) .. + 3, columns (t >> 2) + 64 i)
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.xBytes, 0x00020000);
-  const int rB = t & 15, cB = t >> 4;
+  const int rB = B4 ? (t & 3) * 4 : t & 15, cB = B4 ? t >> 2 : t >> 4;
   int tapOff[NB];
   {
     const int KK = g.kH * g.kW;
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-      const int k = min(j0 + cB + 16 * i, p.Ncols - 1);  // columns past K are dropped in the epilogue
+      const int k = min(j0 + cB + CS * i, p.Ncols - 1);  // columns past K are dropped in the epilogue
       const int c = dev::fastDiv(k, p.magicKK), rem = k - c * KK;
       const int kh = dev::fastDiv(rem, p.magicKW), kw = rem - kh * g.kW;
       tapOff[i] = ((c * g.H + kh * g.dilH) * g.W + kw * g.dilW) * 4;
@@ -1206,7 +1213,8 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
   }
 
   u32x4 ra[WM];
-  unsigned rb[NB];
+  unsigned rb[B4 ? 1 : NB];
+  u32x4 rb4[B4 ? NB : 1];
   // loads the k-tile the position counters stand on, then advances them by BK (L >= BK: one wrap at most)
   auto loadTiles = [&]() {
     if constexpr (L16) {
@@ -1235,14 +1243,19 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
       const int oh = dev::fastDiv(lq, p.magicOW), ow = lq - oh * g.oW;
       const int posOff = nOffB + oh * rowStepB + ow * colStepB;
 #pragma unroll
-      for (int i = 0; i < NB; ++i)
-        rb[i] = __builtin_amdgcn_raw_buffer_load_b32(xr, (int)((unsigned)posOff + (unsigned)tapOff[i]), 0, 0);
+      for (int i = 0; i < NB; ++i) {
+        if constexpr (B4)
+          rb4[i] = __builtin_amdgcn_raw_buffer_load_b128(xr, (int)((unsigned)posOff + (unsigned)tapOff[i]), 0, 0);
+        else
+          rb[i] = __builtin_amdgcn_raw_buffer_load_b32(xr, (int)((unsigned)posOff + (unsigned)tapOff[i]), 0, 0);
+      }
       lB += BK;
       if (lB >= g.L) lB -= g.L, nOffB += imgStrideB;
     }
   };
   u32x4 *aDst = reinterpret_cast<u32x4 *>(&As[0][pgA][rowA]);
   unsigned *bDst = reinterpret_cast<unsigned *>(&Bs[0][rB >> 2][cB]) + (rB & 3);
+  u32x4 *bDst4 = reinterpret_cast<u32x4 *>(&Bs[0][rB >> 2][cB]);
   constexpr int BUFA = (BK / 4) * AP, BUFB = (BK / 4) * GP;  // float4 per LDS buffer
   // The workgroups of the first column tile also sum the gradOutput elements they pass on (each element of a
   // row is loaded by exactly one lane of exactly one of them): the bias gradient without a second pass over gy.
@@ -1262,7 +1275,12 @@ convGradWeightKernel(GradWeightArgs p, ConvGeom g) {
       }
     }
 #pragma unroll
-    for (int i = 0; i < NB; ++i) bDst[buf * BUFB * 4 + 64 * i] = rb[i];  // column + 16 = 16 float4 further
+    for (int i = 0; i < NB; ++i) {
+      if constexpr (B4)
+        bDst4[buf * BUFB + 64 * i] = rb4[i];
+      else
+        bDst[buf * BUFB * 4 + 64 * i] = rb[i];  // column + 16 = 16 float4 further
+    }
   };
   const int grp = lane >> 5, idx = lane & 31;
   const float4 *aSrc = &As[0][grp][wm * 64 + idx];
@@ -2444,11 +2462,28 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     return tinyKernel(l16c, I2{}, I2{});
   };
   const TinyKernel tk = l16 ? pickTiny(std::true_type{}) : pickTiny(std::false_type{});
-  const void *kern =
-      !fast  ? (const void *)convGemmKernel<kGradWeight>
-      : tiny ? tk.fn
-      : l16  ? (wide ? (const void *)convGradWeightKernel<true, 1> : (const void *)convGradWeightKernel<true, 2>)
-             : (wide ? (const void *)convGradWeightKernel<false, 1> : (const void *)convGradWeightKernel<false, 2>);
+  // 16-byte gathers of the image: unit stride along a row, and groups of 4 positions that stay inside an output row
+  // (or output rows that follow each other in the image without a gap: kW = 1, no padding, unit stride down too)
+  const bool b4 = fast && !tiny && !padGy && g.dW == 1 &&
+                  (g.oW % 4 == 0 || (g.dH == 1 && g.W + 2 * g.padW == g.oW));
+  struct BigKernel {
+    const void *fn;
+    void (*launch)(dim3, hipStream_t, const GradWeightArgs &, const ConvGeom &);
+  };
+  auto bigKernel = [](auto l16c, auto wmc, auto b4c) {
+    constexpr bool L = decltype(l16c)::value, B = decltype(b4c)::value;
+    constexpr int W = decltype(wmc)::value;
+    return BigKernel{(const void *)convGradWeightKernel<L, W, 2, 2, B>,
+                     [](dim3 grid, hipStream_t st, const GradWeightArgs &q, const ConvGeom &gk) {
+                       convGradWeightKernel<L, W, 2, 2, B><<<grid, dev::kBlock, 0, st>>>(q, gk);
+                     }};
+  };
+  auto pickBig = [&](auto l16c, auto wmc) { return b4 ? bigKernel(l16c, wmc, std::true_type{}) : bigKernel(l16c, wmc, std::false_type{}); };
+  auto pickBigW = [&](auto l16c) {
+    return wide ? pickBig(l16c, std::integral_constant<int, 1>{}) : pickBig(l16c, std::integral_constant<int, 2>{});
+  };
+  const BigKernel bk = l16 ? pickBigW(std::true_type{}) : pickBigW(std::false_type{});
+  const void *kern = !fast ? (const void *)convGemmKernel<kGradWeight> : tiny ? tk.fn : bk.fn;
   // Every split leaves a partial copy of gradWeight (64 KB per tile) for the fold: three workgroups per CU
   // measured better than the four that fit (less partial traffic for the same matrix-pipe load), two when
   // gradWeight is one or two tiles and the partials are most of the traffic. The small tiles stream: as many
@@ -2511,14 +2546,8 @@ void convGradWeight(THCState *state, const ConvGeom &g, const float *x, const fl
     const dim3 grid(mT * nT * wgSplits);
     if (tiny)
       tk.launch(grid, s, q, gk);
-    else if (l16 && wide)
-      convGradWeightKernel<true, 1><<<grid, dev::kBlock, 0, s>>>(q, gk);
-    else if (l16)
-      convGradWeightKernel<true, 2><<<grid, dev::kBlock, 0, s>>>(q, gk);
-    else if (wide)
-      convGradWeightKernel<false, 1><<<grid, dev::kBlock, 0, s>>>(q, gk);
     else
-      convGradWeightKernel<false, 2><<<grid, dev::kBlock, 0, s>>>(q, gk);
+      bk.launch(grid, s, q, gk);
   } else {
     GemmArgs p{};
     p.a = gy;

@@ -33,6 +33,12 @@ CASES = [
     (2, 40, 256, 8, 12, 1, 2, 0),    # 40 rows: a full 32-row tile and a partial one
     (2, 256, 64, 8, 8, 1, 2, 0),     # every tile split along K: the blocks are written by the fold
     (2, 64, 128, 15, 17, 1, 2, 0),   # odd extents: phase by phase
+    # weight gradient on large tiles with the image gathered 16 bytes at a time (unit stride; 4 positions inside a row)
+    (2, 32, 128, 12, 12, 3, 1, 1),   # 128 x 128 tiles, rows of 12, every k-tile inside one image
+    (2, 40, 130, 8, 16, 3, 1, 1),    # ragged rows and columns, unaligned groups
+    (2, 64, 64, 12, 12, 3, 1, 1),    # 64 x 256 tiles
+    (4, 128, 128, 14, 14, 1, 1, 0),  # rows of 14: groups straddle rows that follow each other without a gap (1x1, no padding)
+    (3, 128, 128, 14, 12, 3, 1, 0),  # output rows of 10: element-wise gather
 ]
 
 

@@ -1049,14 +1049,22 @@ __device__ __forceinline__ void fwdTailFixupBody(const FwdArgs &p, const ConvGeo
 #pragma unroll
     for (int i = 0; i < 4; ++i) vals[i] = vals[i] > 0.f ? vals[i] : 0.f;
   }
+  // (n, oh, ow) of the first of the four columns by one division (through the reciprocals when the launch provides
+  // them), the others by stepping
+  const long col0 = (long)nTile * p.bn + c;
+  if (col0 >= p.Ncols) return;
+  int n, oh, ow;
+  if (col0 + 3 < 0x7fffffffL) {
+    splitColumn(p, g, (unsigned)col0, n, oh, ow);
+  } else {
+    n = (int)(col0 / g.L);
+    const int l = (int)(col0 - (long)n * g.L);
+    oh = l / g.oW, ow = l - oh * g.oW;
+  }
   if (p.dilate) {
     // four neighbouring columns of one output row: their 2 x 2 blocks are 8 consecutive floats of two rows of out
-    const long col = (long)nTile * p.bn + c;
-    const int n = (int)(col / g.L);
-    const int l = (int)(col - (long)n * g.L);
-    const int oh = l / g.oW, ow = l - oh * g.oW;
     float *q = p.out + (long)n * p.outImg + (long)row * p.outRow + (long)oh * p.outSH + ow * 2;
-    if (col + 3 < p.Ncols && ow + 3 < g.oW && ((uintptr_t)q & 15) == 0 && (p.outSH & 7) == 0) {
+    if (col0 + 3 < p.Ncols && ow + 3 < g.oW && ((uintptr_t)q & 15) == 0 && (p.outSH & 7) == 0) {
       float4 *top = reinterpret_cast<float4 *>(q), *bottom = reinterpret_cast<float4 *>(q + (p.outSH >> 1));
       top[0] = make_float4(vals[0], b, vals[1], b), top[1] = make_float4(vals[2], b, vals[3], b);
       bottom[0] = bottom[1] = make_float4(b, b, b, b);
@@ -1065,14 +1073,18 @@ __device__ __forceinline__ void fwdTailFixupBody(const FwdArgs &p, const ConvGeo
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const long col = (long)nTile * p.bn + c + i;
-    if (col >= p.Ncols) break;
-    const int n = (int)(col / g.L);
-    const int l = (int)(col - (long)n * g.L);
-    const int oh = l / g.oW, ow = l - oh * g.oW;
+    if (col0 + i >= p.Ncols) break;
     float *q = p.out + (long)n * p.outImg + (long)row * p.outRow + (long)oh * p.outSH + ow * p.outSW;
-    q[0] = vals[i];
-    if (p.dilate) q[1] = b, q[p.outSH >> 1] = b, q[(p.outSH >> 1) + 1] = b;
+    if (p.dilate) {  // the block's rows start on 8-byte boundaries (even extents, 8-byte aligned tensor)
+      *reinterpret_cast<float2 *>(q) = make_float2(vals[i], b);
+      *reinterpret_cast<float2 *>(q + (p.outSH >> 1)) = make_float2(b, b);
+    } else {
+      q[0] = vals[i];
+    }
+    if (++ow == g.oW) {
+      ow = 0;
+      if (++oh == g.oH) oh = 0, ++n;
+    }
   }
 }
 

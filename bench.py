@@ -60,9 +60,9 @@ MEASURED_TRAFFIC_BYTES = {
     ("cfg4", "avgpool_updateOutput"): _traffic((101707.4, 50176.0)),
     ("cfg4", "avgpool_updateGradInput"): _traffic((30467.5, 200744.3)),
     # bordered copy + GEMM + tail fold (+ flipped weights for gradInput; + partial fold for the weight gradient)
-    ("cfg5", "convmm_updateOutput"): _traffic((25978.1, 57606.1), (109212.5, 67553.5), (8239.5, 1024.0)),
-    ("cfg5", "convmm_updateGradInput"): _traffic((25978.1, 57606.1), (109212.5, 67553.5), (8239.5, 1024.0), (5176.1, 2304.0)),
-    ("cfg5", "convmm_accGradParameters"): _traffic((25978.1, 57606.1), (70327.3, 48405.0), (25371.7, 2305.0)),
+    ("cfg5", "convmm_updateOutput"): _traffic((25983.1, 57606.1), (109213.0, 68873.4), (8228.5, 1024.0)),
+    ("cfg5", "convmm_updateGradInput"): _traffic((25983.1, 57606.1), (109213.0, 68873.4), (8228.5, 1024.0), (5172.6, 2304.0)),
+    ("cfg5", "convmm_accGradParameters"): _traffic((25983.1, 57606.1), (72209.9, 48405.0), (25371.7, 2305.0)),
 }
 
 

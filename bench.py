@@ -11,11 +11,17 @@ stride 2 pad 1 (the MobileNet stride-2 layer). Inputs live in HBM before the tim
 region; four buffer sets are rotated so that no step finds its inputs in the
 256 MB Infinity Cache from the step before.
 
-Prints ONE JSON line: images/s for the whole job, plus
+Prints ONE JSON line: images/s for the whole job (K steps between two
+synchronisations, nothing but the entry-point calls on the stream), plus
   roofline     - the dominant entry point's algorithmic bytes (or flops) per launch
                  over its average duration measured with HIP events on the
-                 stream the kernels run on, against MI355X's published peak
-                 (median, min and the whole step's fraction beside it);
+                 stream the kernels run on, over the same K steps run a second
+                 time with that entry point bracketed, against MI355X's published
+                 peak (median, min and the whole step's fraction beside it);
+                 roofline.cold: the same figures when the entry points of a step
+                 work on different buffer sets, so that no call finds in the
+                 Infinity Cache what an earlier call of the step touched;
+                 roofline.copy_gbs: what a plain 128 MiB copy reaches in this run;
   cpu_baseline - the CPU oracle (a port of the reference algorithm) timed on
                  this host's cores on a bounded sample of the same workload;
   workloads    - with --all, the same figures for the other four configurations.
@@ -38,32 +44,27 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 FP32_MFMA_PEAK_TFLOPS = 157.3
 METRIC = "DW-conv fwd+bwd images/s + achieved HBM GB/s (% of peak), 1 MI355X"
 
-# HBM bytes per entry-point call measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch; the
-# profiles/*_hbm_traffic.txt and profiles/cfg5_mfma_util.txt summaries give the runs and the copy-kernel scale
-# factors: FETCH_SIZE x 2, WRITE_SIZE x 1), summed over the kernels an entry point launches.
+# HBM bytes per entry-point call, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch) and kept
+# beside the summaries they come from: profiles/hbm_traffic_table.txt has one row per kernel of an entry point with the
+# raw counter averages, the summary file and the commit the counters were collected at. Scale factors from the copy
+# kernel of known size: FETCH_SIZE x 2, WRITE_SIZE x 1.
 _KIB = 1024
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_table.txt")
 
 
-def _traffic(*kernels):
-    return int(sum(f * 2.0 + w for f, w in kernels) * _KIB)
-
-
-MEASURED_TRAFFIC_BYTES = {
-    ("cfg1", "dw_updateOutput"): _traffic((26658.6, 50207.7)),
-    ("cfg2", "dw_updateOutput"): _traffic((50222.7, 25130.5)),
-    ("cfg2", "dw_updateGradInput"): _traffic((12840.5, 100352.0)),
-    ("cfg2", "dw_accGradParameters"): _traffic((63024.6, 512.0), (558.5, 12.0)),
-    ("cfg3", "bn_updateOutput"): _traffic((25722.0, 51041.0)),
-    ("cfg3", "bn_backward"): _traffic((56377.2, 51211.0)),
-    ("cfg4", "maxpool_updateOutput"): _traffic((103481.2, 150592.2)),
-    ("cfg4", "maxpool_updateGradInput"): _traffic((76828.4, 200725.9)),
-    ("cfg4", "avgpool_updateOutput"): _traffic((101707.4, 50176.0)),
-    ("cfg4", "avgpool_updateGradInput"): _traffic((30467.5, 200744.3)),
-    # bordered copy + GEMM + tail fold (+ flipped weights for gradInput; + partial fold for the weight gradient)
-    ("cfg5", "convmm_updateOutput"): _traffic((25983.1, 57606.1), (109213.0, 68873.4), (8228.5, 1024.0)),
-    ("cfg5", "convmm_updateGradInput"): _traffic((25983.1, 57606.1), (109213.0, 68873.4), (8228.5, 1024.0), (5172.6, 2304.0)),
-    ("cfg5", "convmm_accGradParameters"): _traffic((25983.1, 57606.1), (72209.9, 48405.0), (25371.7, 2305.0)),
-}
+def load_traffic(path=TRAFFIC_TABLE):
+    """{(workload, entry point): dict(bytes=..., source=..., commit=...)}; empty when the table is missing."""
+    out = {}
+    if not os.path.exists(path):
+        return out
+    for line in open(path):
+        line = line.split("#", 1)[0].split()
+        if len(line) != 7:
+            continue
+        wl, entry, _kernel, fetch, write, source, commit = line
+        e = out.setdefault((wl, entry), dict(bytes=0, source=source, commit=commit))
+        e["bytes"] += int((float(fetch) * 2.0 + float(write)) * _KIB)
+    return out
 
 
 class Hip:
@@ -72,6 +73,7 @@ class Hip:
         self.lib.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
         self.lib.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
         self.lib.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.lib.hipStreamQuery.argtypes = [C.c_void_p]
 
     def check(self, rc, what):
         if rc != 0:
@@ -93,7 +95,16 @@ class Hip:
         self.check(self.lib.hipEventElapsedTime(C.byref(ms), a, b), "hipEventElapsedTime")
         return float(ms.value)
 
-    def sync(self):
+    def sync(self, stream=None):
+        # With a stream: poll it until it has drained instead of sleeping in the runtime - the wake-up after a
+        # blocking wait costs tens of microseconds, a sizeable part of a 20-step timed region of 1.4 ms.
+        if stream is not None:
+            while True:
+                rc = self.lib.hipStreamQuery(stream)
+                if rc == 0:
+                    break
+                if rc != 600:  # hipErrorNotReady
+                    self.check(rc, "hipStreamQuery")
         self.check(self.lib.hipDeviceSynchronize(), "hipDeviceSynchronize")
 
 
@@ -588,21 +599,57 @@ WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda
 
 
 PREROLL_SAMPLES = 12   # event samples per entry point collected before the timed region, whatever --warmup is
+COLD_SETS = 8          # buffer sets of the cache-cold ordering
+COPY_LAUNCHES = 24     # launches of the copy kernel that give the in-run streaming ceiling
 
 
-def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds):
-    wl = WORKLOADS[name](nsets)
+def copy_ceiling(hip, stream):
+    """What a plain float4 copy reaches on this part in this run: COPY_LAUNCHES launches of 128 MiB rotating through
+    four buffer pairs (1 GiB, so nothing is found in the 256 MB Infinity Cache), timed by the wall clock between two
+    synchronisations and, each launch on its own, by HIP events."""
+    wl = wl_copy(4)
+    wl["verify"]()
+    fns = [wl["calls"](i)[0][1] for i in range(4)]
+    nbytes = wl["work"]["copy"][0]
+    for i in range(8):
+        fns[i % 4]()
+    ev = [(hip.event(), hip.event()) for _ in range(COPY_LAUNCHES)]
+    hip.sync()
+    t0 = time.perf_counter()
+    for i in range(COPY_LAUNCHES):
+        fns[i % 4]()
+    hip.sync()
+    wall = time.perf_counter() - t0
+    for i, (a, b) in enumerate(ev):
+        hip.record(a, stream)
+        fns[i % 4]()
+        hip.record(b, stream)
+    hip.sync()
+    med = float(np.median([hip.elapsed_ms(a, b) for a, b in ev]))
+    return dict(copy_gbs=round(nbytes * COPY_LAUNCHES / wall / 1e9, 1), copy_gbs_event_median=round(nbytes / (med * 1e-3) / 1e9, 1),
+                copy_bytes_per_launch=nbytes, copy_launches=COPY_LAUNCHES)
+
+
+def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=False, cold_sets=COLD_SETS):
+    ncold = cold_sets if nsets > 1 and name != "copy" else nsets
+    wl = WORKLOADS[name](max(nsets, ncold))
     wl["verify"]()                       # parity against the oracle in this very run
     names = [n for n, _ in wl["calls"](0)]
+    # cache-cold ordering: the entry points of one step work on different buffer sets, `stride` sets apart, so that
+    # no call finds a tensor that an earlier call of the same step (or of the step before) has touched
+    stride = max(1, ncold // len(names))
     cursor = [0]                         # buffer sets keep rotating across the phases below
 
-    def run(nsteps, bracket):
+    def run(nsteps, bracket, cold=False):
         """nsteps steps back to back; HIP events around the entry points named in `bracket`."""
         ev = {n: [(hip.event(), hip.event()) for _ in range(nsteps)] for n in bracket}
-        hip.sync()
+        hip.sync(stream)
         t0 = time.perf_counter()
         for i in range(nsteps):
-            for n, fn in wl["calls"](cursor[0] % nsets):
+            c = cursor[0]
+            step = ([wl["calls"]((c + j * stride) % ncold)[j] for j in range(len(names))] if cold
+                    else wl["calls"](c % nsets))
+            for n, fn in step:
                 if n in ev:
                     hip.record(ev[n][i][0], stream)
                     fn()
@@ -610,53 +657,89 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds):
                 else:
                     fn()
             cursor[0] += 1
-        hip.sync()
+        hip.sync(stream)
         wall = time.perf_counter() - t0
         return wall, {n: [hip.elapsed_ms(a, b) for a, b in ev[n]] for n in bracket}
+
+    def table(per_kernel):
+        kern = {}
+        for n in names:
+            med, avg = float(np.median(per_kernel[n])), float(np.mean(per_kernel[n]))
+            amount, kind = wl["work"][n]
+            if kind == "bytes":
+                scale, peak, unit = 1e9, HBM_PEAK_GBS, "GB/s"
+            else:
+                scale, peak, unit = 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
+            amount = max(amount, 1)       # entry points with no algorithmic traffic of their own (the unfused ReLU steps)
+            kern[n] = dict(avg_ms=avg, median_ms=med, min_ms=float(np.min(per_kernel[n])), samples=len(per_kernel[n]),
+                           achieved=amount / (avg * 1e-3) / scale, achieved_median=amount / (med * 1e-3) / scale,
+                           peak=peak, unit=unit, frac=amount / (avg * 1e-3) / scale / peak,
+                           frac_median=amount / (med * 1e-3) / scale / peak, algorithmic=amount, kind=kind)
+        return kern
+
+    step_work = sum(wl["work"][n][0] for n in names)
+    step_scale, step_peak = (1e9, HBM_PEAK_GBS) if wl["bound"] == "hbm" else (1e12, FP32_MFMA_PEAK_TFLOPS)
+
+    def step_frac(ms):
+        return round(step_work / (ms * 1e-3) / step_scale / step_peak, 4)
 
     # pre-roll (untimed, reported as preroll_steps): one plain step on every buffer set, so that every
     # output / gradInput / scratch storage has its final size before anything is measured (a first call at
     # a new size allocates), then PREROLL_SAMPLES steps per entry point with HIP events around that entry
     # point alone (events around neighbouring launches would add their own few microseconds to each
     # other's bracket) - that finds the dominant kernel and times the others
-    run(nsets, [])
-    preroll = nsets
+    for i in range(max(nsets, ncold)):
+        for _, fn in wl["calls"](i):
+            fn()
+    preroll = max(nsets, ncold)
     per_kernel = {}
     for n in names:
         per_kernel.update(run(PREROLL_SAMPLES, [n])[1])
         preroll += PREROLL_SAMPLES
     dominant = max(names, key=lambda n: float(np.median(per_kernel[n])))
     run(warmup, [])                      # the W warm-up steps asked for
-    # the timed region: exactly `steps` steps; only the dominant kernel is bracketed by events,
-    # so the measurement perturbs the step as little as possible
-    wall, dom = run(steps, [dominant])
+    # the timed region: exactly `steps` steps between two synchronisations, nothing but the entry-point calls on
+    # the stream - this gives `value`. Recording an event pair costs the step several microseconds (two more
+    # packets for the command processor, and the kernel behind a record starts later), so the pass that brackets
+    # the dominant entry point for `roofline` is a second run of the same `steps` steps right behind the first.
+    wall, _ = run(steps, [])
+    wall_ev, dom = run(steps, [dominant])
     per_kernel[dominant] = dom[dominant]
-    kern = {}
-    for n in names:
-        med, avg = float(np.median(per_kernel[n])), float(np.mean(per_kernel[n]))
-        amount, kind = wl["work"][n]
-        if kind == "bytes":
-            scale, peak, unit = 1e9, HBM_PEAK_GBS, "GB/s"
-        else:
-            scale, peak, unit = 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
-        amount = max(amount, 1)           # entry points with no algorithmic traffic of their own (the unfused ReLU steps)
-        kern[n] = dict(avg_ms=avg, median_ms=med, min_ms=float(np.min(per_kernel[n])), samples=len(per_kernel[n]),
-                       achieved=amount / (avg * 1e-3) / scale, achieved_median=amount / (med * 1e-3) / scale,
-                       peak=peak, unit=unit, frac=amount / (avg * 1e-3) / scale / peak,
-                       frac_median=amount / (med * 1e-3) / scale / peak, algorithmic=amount, kind=kind)
+    kern = table(per_kernel)
     ms_per_step = wall * 1e3 / steps
     d = kern[dominant]
-    step_work = sum(wl["work"][n][0] for n in names)
-    step_scale, step_peak = (1e9, HBM_PEAK_GBS) if wl["bound"] == "hbm" else (1e12, FP32_MFMA_PEAK_TFLOPS)
+    traffic = load_traffic().get((name, dominant))
     roofline = dict(bound=wl["bound"], kernel=dominant, achieved=round(d["achieved"], 3), peak=d["peak"], unit=d["unit"],
-                    frac=round(d["frac"], 4), traffic=MEASURED_TRAFFIC_BYTES.get((name, dominant)),
+                    frac=round(d["frac"], 4), traffic=traffic["bytes"] if traffic else None,
+                    traffic_source=(f"profiles/{traffic['source']} at commit {traffic['commit']}" if traffic else None),
                     algorithmic_per_launch=d["algorithmic"], avg_launch_ms=round(d["avg_ms"], 5),
                     median_launch_ms=round(d["median_ms"], 5), min_launch_ms=round(d["min_ms"], 5),
                     frac_median=round(d["frac_median"], 4), samples=d["samples"],
-                    step_frac=round(step_work / (ms_per_step * 1e-3) / step_scale / step_peak, 4),
-                    algorithmic_per_step=step_work)
+                    step_frac=step_frac(ms_per_step), algorithmic_per_step=step_work,
+                    ms_per_step_bracketed=round(wall_ev * 1e3 / steps, 5))
+    extra = 0
+    if ncold > 1 and ncold >= 2 * len(names):
+        # cache-cold variant, outside the timed steps: the same entry points, each on a buffer set that nothing has
+        # touched for at least `stride` - 1 whole steps (more than 1 GB of traffic at cfg2)
+        run(ncold, [], cold=True)
+        cold_pk = {}
+        for n in names:
+            cold_pk.update(run(PREROLL_SAMPLES, [n], cold=True)[1])
+        cold_wall, _ = run(max(steps, 20), [], cold=True)
+        ck = table(cold_pk)
+        cold_ms = cold_wall * 1e3 / max(steps, 20)
+        cdom = max(names, key=lambda n: ck[n]["median_ms"])
+        roofline["cold"] = dict(
+            order=f"entry point j of step s on buffer set (s + {stride} j) mod {ncold}", sets=ncold, kernel=cdom,
+            frac=round(ck[cdom]["frac_median"], 4), ms_per_step=round(cold_ms, 5), step_frac=step_frac(cold_ms),
+            entry_points={n: dict(median_ms=round(ck[n]["median_ms"], 5), min_ms=round(ck[n]["min_ms"], 5),
+                                  frac=round(ck[n]["frac_median"], 4)) for n in names})
+        extra += ncold + len(names) * PREROLL_SAMPLES + max(steps, 20)
+    if ceiling:
+        roofline.update(copy_ceiling(hip, stream))
     res = dict(workload=wl["desc"], images_per_s=wl["images"] / (ms_per_step * 1e-3), ms_per_step=ms_per_step,
                device_ms_per_step=float(sum(kern[n]["median_ms"] for n in names)), roofline=roofline, preroll_steps=preroll,
+               untimed_steps_after=steps + extra,
                kernels={n: {k: (round(v, 5) if isinstance(v, float) else v) for k, v in kern[n].items()} for n in names})
     if cpu_seconds > 0 and name != "copy":
         from oracle import oracle as O
@@ -676,6 +759,7 @@ def main():
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
     ap.add_argument("--all", action="store_true", help="also time the other four configurations")
     ap.add_argument("--sets", type=int, default=4, help="buffer sets rotated between steps (1 = cache-warm variant)")
+    ap.add_argument("--cold-sets", type=int, default=COLD_SETS, help="buffer sets of the cache-cold ordering (0 = skip it)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU time budget of the oracle baseline (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -690,7 +774,8 @@ def main():
     stream = lib.THCState_getCurrentStream(st)
     hip = Hip()
 
-    main_res = run_workload(args.workload, args.steps, args.warmup, hip, stream, args.sets, args.cpu_seconds)
+    main_res = run_workload(args.workload, args.steps, args.warmup, hip, stream, args.sets, args.cpu_seconds, ceiling=True,
+                            cold_sets=args.cold_sets)
     out = {
         "metric": METRIC, "value": round(main_res["images_per_s"], 1), "unit": "images/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(main_res["ms_per_step"], 5),
@@ -699,6 +784,7 @@ def main():
                    "entry": "C ABI libTHCUNN.so (THNN_Cuda*) via ctypes"},
         "device_ms_per_step": round(main_res["device_ms_per_step"], 5),
         "preroll_steps": main_res["preroll_steps"],
+        "untimed_steps_after": main_res["untimed_steps_after"],
         "roofline": main_res["roofline"],
         "cpu_baseline": main_res.get("cpu_baseline"),
         "kernels": main_res["kernels"],

@@ -445,7 +445,7 @@ dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strid
       loadTaps<KS>(weight, ws, j, c, w);
       b = bias ? bias[j * bs.s0 + c * bs.s1] : 0.f;
     }
-    float *o = out + (((long)plane * nMul + j) * g.oH + oh0) * g.oW;
+    const __amdgpu_buffer_rsrc_t orr = dev::makeRsrc(out + (((long)plane * nMul + j) * g.oH + oh0) * g.oW, (long)total * 16);
     for (int i = threadIdx.x; i < total; i += blockDim.x) {
       const int r = dev::fastDiv(i, g.magicOW4), b4 = i - r * oW4;
       const float *p = smem + r * ST * pitch;
@@ -459,7 +459,7 @@ dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strid
 #pragma unroll
           for (int q = 0; q < 4; ++q) acc[q] = fmaf(win[q * ST + kw], w[kh * KS + kw], acc[q]);
       }
-      dev::storeStream4(o + (long)r * g.oW + b4 * 4, make_float4(acc[0], acc[1], acc[2], acc[3]));
+      dev::bufStoreStream4(orr, i * 16, make_float4(acc[0], acc[1], acc[2], acc[3]));  // r * oW + b4 * 4 = 4 i
     }
   }
 }
@@ -503,7 +503,7 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
   // h0 + hl = ST*a + dy picks, per staged gradOutput row qh, the kernel row kh = dy + PAD - qh*ST; dy is
   // a run-time value, so those taps are selected into per-lane weights instead of being resolved at compile time.
   const int total = nRows * W4;
-  float *o = gradIn + ((long)plane * g.H + h0) * g.W;
+  const __amdgpu_buffer_rsrc_t orr = dev::makeRsrc(gradIn + ((long)plane * g.H + h0) * g.W, (long)total * 16);
   constexpr int kUnroll = ST == 1 ? 1 : 2;  // the wave shifts of the stride-1 window do not unroll
 #pragma unroll kUnroll
   for (int i = threadIdx.x; i < total; i += blockDim.x) {
@@ -540,7 +540,7 @@ dwGradInputStrip(const float *__restrict__ gradOut, const float *__restrict__ we
           }
       }
     }
-    dev::storeStream4(o + (long)i * 4, make_float4(acc[0], acc[1], acc[2], acc[3]));
+    dev::bufStoreStream4(orr, i * 16, make_float4(acc[0], acc[1], acc[2], acc[3]));
   }
 }
 
@@ -564,27 +564,24 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
   const int nOut = min(g.tileRows, g.oH - oh0);
   const int nIn = (nOut - 1) * ST + KS;
   const int pitch = S::pitch(g.W);
-  float *gs = smem + S::floats((g.tileRows - 1) * ST + KS, g.W);  // multiple of 4 floats
+  float *gs = smem + S::floats((g.tileRows - 1) * ST + KS, g.W);  // multiple of 4 floats (staged gradOutput band: !ONE only)
   const int nMul = ONE ? 1 : g.M;
+  const int oW4 = g.oW >> 2;
+  const int total = nOut * oW4;
+  // ONE: item i of the band (4 consecutive outputs, memory order) is float4 i of the gradOutput band, and the lane
+  // that loads float4 u * kBlock + tid is the lane that works on item u * kBlock + tid: gradOutput never leaves
+  // the registers it was loaded into (no LDS copy, 3 KB less LDS per workgroup at 28 x 28 outputs).
+  float4 gv[dev::kLoadBatch];
   if (ONE) {
     typename S::InFlight fl;
     S::template issue<true>(fl, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
-    const int n4 = (nOut * g.oW) >> 2;
-    const __amdgpu_buffer_rsrc_t rs = dev::makeRsrc(gradOut + ((long)plane * g.oH + oh0) * g.oW, (long)n4 * 16);
-    float4 gv[dev::kLoadBatch];
+    const __amdgpu_buffer_rsrc_t rs = dev::makeRsrc(gradOut + ((long)plane * g.oH + oh0) * g.oW, (long)total * 16);
 #pragma unroll
     for (int u = 0; u < dev::kLoadBatch; ++u) gv[u] = dev::bufLoadStream4(rs, (u * dev::kBlock + threadIdx.x) * 16);  // past the end reads 0
     S::commit(smem, fl, g.W, nIn);
-#pragma unroll
-    for (int u = 0; u < dev::kLoadBatch; ++u) {
-      const int i = u * dev::kBlock + threadIdx.x;
-      if (i < n4) reinterpret_cast<float4 *>(gs)[i] = gv[u];
-    }
   } else {
     S::stage(smem, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
   }
-  const int oW4 = g.oW >> 2;
-  const int total = nOut * oW4;
   const int slot = n * g.tilesPerPlane + tile;
   const int lane = threadIdx.x % dev::kWave, wave = threadIdx.x / dev::kWave;
   for (int j = 0; j < nMul; ++j) {
@@ -596,10 +593,9 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
     float acc[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) acc[t] = 0.f;
-    for (int i = threadIdx.x; i < total; i += blockDim.x) {
+    auto item = [&](int i, const float4 gy4) {
       const int r = dev::fastDiv(i, g.magicOW4), b4 = i - r * oW4;
       const float *p = smem + r * ST * pitch;
-      const float4 gy4 = *reinterpret_cast<const float4 *>(gs + r * g.oW + b4 * 4);
       const float gy[4] = {gy4.x, gy4.y, gy4.z, gy4.w};
 #pragma unroll
       for (int kh = 0; kh < KS; ++kh) {
@@ -611,6 +607,15 @@ dwAccGradStrip(const float *__restrict__ in, const float *__restrict__ gradOut, 
           for (int q = 0; q < 4; ++q) acc[kh * KS + kw] = fmaf(gy[q], win[q * ST + kw], acc[kh * KS + kw]);
       }
       acc[T - 1] += (gy[0] + gy[1]) + (gy[2] + gy[3]);
+    };
+    if constexpr (ONE) {
+#pragma unroll
+      for (int u = 0; u < dev::kLoadBatch; ++u) {
+        const int i = u * dev::kBlock + (int)threadIdx.x;
+        if (i < total) item(i, gv[u]);
+      }
+    } else {
+      for (int i = threadIdx.x; i < total; i += blockDim.x) item(i, *reinterpret_cast<const float4 *>(gs + i * 4));
     }
     // rows of 16 lanes are folded on the VALU (4 DPP steps per sum), the 16 row sums of the workgroup through LDS
 #pragma unroll
@@ -1218,9 +1223,10 @@ void dwAccGradParameters(THCState *state, THCudaTensor *input, THCudaTensor *gra
       dim3 grid(g.nblk), block(dev::kBlock);
       g.magicTiles = dev::magicOf(g.tilesPerPlane), g.magicC = dev::magicOf(g.C);
       g.magicOW4 = dev::magicOf(g.oW / 4), g.magicW4 = dev::magicOf(g.W / 4);
-      if (g.M == 1 && staged(g.tileRows) <= (size_t)launch::kBatchFloats && aligned16(go.ptr()))
+      if (g.M == 1 && staged(g.tileRows) <= (size_t)launch::kBatchFloats && aligned16(go.ptr())) {
+        lds = stripFloats(g, (g.tileRows - 1) * g.dH + g.kH) * sizeof(float);  // gradOutput stays in registers
         DW_STRIP_DISPATCH1(dwAccGradStrip, true, in.ptr(), go.ptr(), partial, g);
-      else
+      } else
         DW_STRIP_DISPATCH1(dwAccGradStrip, false, in.ptr(), go.ptr(), partial, g);
     } else {
       if (ks == 3 && st == 1) launchAcc1<3, 1>(s, lds, vec, vecg, in.ptr(), go.ptr(), partial, g);

@@ -599,7 +599,7 @@ WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda
 
 
 PREROLL_SAMPLES = 12   # event samples per entry point collected before the timed region, whatever --warmup is
-COLD_SETS = 8          # buffer sets of the cache-cold ordering
+COLD_SETS = 6          # buffer sets of the cache-cold ordering
 COPY_LAUNCHES = 24     # launches of the copy kernel that give the in-run streaming ceiling
 
 
@@ -640,9 +640,12 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=F
     stride = max(1, ncold // len(names))
     cursor = [0]                         # buffer sets keep rotating across the phases below
 
-    def run(nsteps, bracket, cold=False):
-        """nsteps steps back to back; HIP events around the entry points named in `bracket`."""
+    def run(nsteps, bracket, cold=False, empty=False):
+        """nsteps steps back to back; HIP events around the entry points named in `bracket`; with `empty`, one more
+        event pair with nothing between them at the end of every step (what a bracket costs by itself)."""
         ev = {n: [(hip.event(), hip.event()) for _ in range(nsteps)] for n in bracket}
+        if empty:
+            ev[None] = [(hip.event(), hip.event()) for _ in range(nsteps)]
         hip.sync(stream)
         t0 = time.perf_counter()
         for i in range(nsteps):
@@ -656,10 +659,13 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=F
                     hip.record(ev[n][i][1], stream)
                 else:
                     fn()
+            if empty:
+                hip.record(ev[None][i][0], stream)
+                hip.record(ev[None][i][1], stream)
             cursor[0] += 1
         hip.sync(stream)
         wall = time.perf_counter() - t0
-        return wall, {n: [hip.elapsed_ms(a, b) for a, b in ev[n]] for n in bracket}
+        return wall, {n: [hip.elapsed_ms(a, b) for a, b in ev[n]] for n in ev}
 
     def table(per_kernel):
         kern = {}
@@ -703,7 +709,7 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=F
     # packets for the command processor, and the kernel behind a record starts later), so the pass that brackets
     # the dominant entry point for `roofline` is a second run of the same `steps` steps right behind the first.
     wall, _ = run(steps, [])
-    wall_ev, dom = run(steps, [dominant])
+    wall_ev, dom = run(steps, [dominant], empty=True)
     per_kernel[dominant] = dom[dominant]
     kern = table(per_kernel)
     ms_per_step = wall * 1e3 / steps
@@ -716,7 +722,8 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=F
                     median_launch_ms=round(d["median_ms"], 5), min_launch_ms=round(d["min_ms"], 5),
                     frac_median=round(d["frac_median"], 4), samples=d["samples"],
                     step_frac=step_frac(ms_per_step), algorithmic_per_step=step_work,
-                    ms_per_step_bracketed=round(wall_ev * 1e3 / steps, 5))
+                    ms_per_step_bracketed=round(wall_ev * 1e3 / steps, 5),
+                    empty_bracket_ms=round(float(np.median(dom[None])), 5))
     extra = 0
     if ncold > 1 and ncold >= 2 * len(names):
         # cache-cold variant, outside the timed steps: the same entry points, each on a buffer set that nothing has

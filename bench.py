@@ -709,8 +709,9 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=F
     # packets for the command processor, and the kernel behind a record starts later), so the pass that brackets
     # the dominant entry point for `roofline` is a second run of the same `steps` steps right behind the first.
     wall, _ = run(steps, [])
-    wall_ev, dom = run(steps, [dominant], empty=True)
+    wall_ev, dom = run(steps, [dominant])
     per_kernel[dominant] = dom[dominant]
+    _, emp = run(PREROLL_SAMPLES, [], empty=True)   # in a pass of its own: next to a real bracket it changes that bracket's reading
     kern = table(per_kernel)
     ms_per_step = wall * 1e3 / steps
     d = kern[dominant]
@@ -723,8 +724,8 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=F
                     frac_median=round(d["frac_median"], 4), samples=d["samples"],
                     step_frac=step_frac(ms_per_step), algorithmic_per_step=step_work,
                     ms_per_step_bracketed=round(wall_ev * 1e3 / steps, 5),
-                    empty_bracket_ms=round(float(np.median(dom[None])), 5))
-    extra = 0
+                    empty_bracket_ms=round(float(np.median(emp[None])), 5))
+    extra = PREROLL_SAMPLES
     if ncold > 1 and ncold >= 2 * len(names):
         # cache-cold variant, outside the timed steps: the same entry points, each on a buffer set that nothing has
         # touched for at least `stride` - 1 whole steps (more than 1 GB of traffic at cfg2)

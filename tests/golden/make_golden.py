@@ -87,6 +87,66 @@ def pool_case(rng, N, C, H, W, k, s, p, ceil):
     return out
 
 
+def dilpool_case(rng, N, C, H, W, k, s, p, dil, ceil):
+    x = (np.round(rng.uniform(-1, 1, (N, C, H, W)) * 16) / 16).astype(np.float32)   # ties
+    tx = T(x).requires_grad_()
+    y, idx = F.max_pool2d(tx, k, s, p, dilation=dil, ceil_mode=ceil, return_indices=True)
+    gy = rng.standard_normal(tuple(y.shape)).astype(np.float32)
+    y.backward(T(gy))
+    return dict(x=x, gy=gy, max_y=y.detach().numpy(), max_idx=idx.numpy() + 1, max_gx=tx.grad.numpy(),
+                geom=np.array([k, k, s, s, p, p, dil, dil, int(ceil)]))
+
+
+def dilconv_case(rng, N, Ci, Co, H, W, k, s, p, dil):
+    """SpatialDilatedConvolution: 4-D weight (Cout, Cin, kH, kW)."""
+    x = rng.standard_normal((N, Ci, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Co, Ci, k, k)) * 0.2).astype(np.float32)
+    b = rng.standard_normal(Co).astype(np.float32)
+    tx, tw, tb = T(x).requires_grad_(), T(w).requires_grad_(), T(b).requires_grad_()
+    y = F.conv2d(tx, tw, tb, stride=s, padding=p, dilation=dil)
+    gy = rng.standard_normal(tuple(y.shape)).astype(np.float32)
+    y.backward(T(gy))
+    return dict(x=x, w=w, b=b, gy=gy, y=y.detach().numpy(), gx=tx.grad.numpy(), gw=tw.grad.numpy(), gb=tb.grad.numpy(),
+                geom=np.array([k, k, s, s, p, p, dil, dil]))
+
+
+def fullconv_case(rng, N, Ci, Co, H, W, k, s, p, adj):
+    """SpatialFullConvolution: weight (Cin, Cout, kH, kW), output (H - 1) s - 2 p + k + adj."""
+    x = rng.standard_normal((N, Ci, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Ci, Co, k, k)) * 0.2).astype(np.float32)
+    b = rng.standard_normal(Co).astype(np.float32)
+    tx, tw, tb = T(x).requires_grad_(), T(w).requires_grad_(), T(b).requires_grad_()
+    y = F.conv_transpose2d(tx, tw, tb, stride=s, padding=p, output_padding=adj)
+    gy = rng.standard_normal(tuple(y.shape)).astype(np.float32)
+    y.backward(T(gy))
+    return dict(x=x, w=w, b=b, gy=gy, y=y.detach().numpy(), gx=tx.grad.numpy(), gw=tw.grad.numpy(), gb=tb.grad.numpy(),
+                geom=np.array([k, k, s, s, p, p, adj, adj]))
+
+
+def threshold_case(rng, shape, th, val):
+    """Threshold: y = x > th ? x : val; gradInput = x > th ? gradOutput : 0 (lib/THCUNN/Threshold.cu). Values
+    quantised so that some inputs equal the threshold exactly (the comparison is strict)."""
+    x = (np.round(rng.standard_normal(shape) * 4) / 4).astype(np.float32)
+    gy = rng.standard_normal(shape).astype(np.float32)
+    y = np.where(x > np.float32(th), x, np.float32(val)).astype(np.float32)
+    gx = np.where(x > np.float32(th), gy, np.float32(0)).astype(np.float32)
+    return dict(x=x, gy=gy, y=y, gx=gx, param=np.array([th, val], np.float32))
+
+
+def bnrelu_case(rng, shape):
+    """BatchNormalization (train) followed by Threshold(0, 0): activation, and the gradients of the pair."""
+    C = shape[1]
+    x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float32)
+    g = (rng.random(C) + 0.25).astype(np.float32)
+    b = rng.standard_normal(C).astype(np.float32)
+    rm, rv = torch.zeros(C, dtype=torch.float64), torch.ones(C, dtype=torch.float64)
+    tx, tg, tb = T(x).requires_grad_(), T(g).requires_grad_(), T(b).requires_grad_()
+    a = F.relu(F.batch_norm(tx, rm, rv, tg, tb, True, 0.1, 1e-5))
+    ga = rng.standard_normal(shape).astype(np.float32)
+    a.backward(T(ga))
+    return dict(x=x, g=g, b=b, ga=ga, a=a.detach().numpy(), gx=tx.grad.numpy(), gw=tg.grad.numpy(), gb=tb.grad.numpy())
+
+
 def main():
     rng = np.random.default_rng(20240601)
     cases = {
@@ -104,6 +164,15 @@ def main():
         # (lib/THCUNN/generic/SpatialDilatedMaxPooling.cu:56-64): 7 -> 4 and 9 -> 5 outputs instead of 5 and 6
         "pool_2s2p1_ceil_drop": pool_case(rng, 2, 3, 7, 9, 2, 2, 1, True),
     }
+    # cases added later draw from a generator of their own, so that the vectors above stay bit for bit what they were
+    rng2 = np.random.default_rng(20240602)
+    cases.update({
+        "pool_dil2": dilpool_case(rng2, 2, 3, 13, 14, 3, 2, 1, 2, False),
+        "dilconv_d2": dilconv_case(rng2, 2, 4, 6, 12, 11, 3, 1, 2, 2),
+        "fullconv_s2": fullconv_case(rng2, 2, 6, 4, 7, 8, 4, 2, 1, 0),
+        "thr": threshold_case(rng2, (3, 5, 7, 6), 0.25, -0.5),
+        "bnrelu_4d": bnrelu_case(rng2, (6, 5, 7, 9)),
+    })
     flat = {}
     for cname, d in cases.items():
         for k, v in d.items():

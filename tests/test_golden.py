@@ -170,3 +170,107 @@ def test_avgpool_reference_known_answer(backend):
     exc, _ = backend.avgpool({}, False, x=c["x"])
     assert exc[0, 0, 0, 0] == c["exclude_pad"] == 3.0
     assert inc[0, 0, 0, 0] == c["include_pad"] == 0.75
+
+
+# ---- vectors for the entry points next to the hot path: dilated max pooling, dilated and transposed convolution,
+# Threshold, and the fused BatchNormalization + ReLU pair ----------------------------------------------------------
+
+def _hip():
+    import cunn_amd
+    return cunn_amd.CudaTensor, cunn_amd.CudaLongTensor, cunn_amd.THNN
+
+
+def test_dilated_maxpool_golden(backend):
+    c = case("pool_dil2")
+    k, _, s, _, p, _, dil, _, ceil = [int(v) for v in c["geom"]]
+    if backend.name == "oracle":
+        y, idx = O.maxpool_updateOutput(c["x"], k, k, s, s, p, p, bool(ceil), dil, dil)
+        gx = O.maxpool_updateGradInput(c["x"].shape, c["gy"], idx, k, k, s, s, p, p, bool(ceil), dil, dil)
+    else:
+        CT, LT, THNN = _hip()
+        x, gy, ty, tidx, tgx = CT.from_numpy(c["x"]), CT.from_numpy(c["gy"]), CT(), LT(), CT()
+        THNN.SpatialDilatedMaxPooling_updateOutput(x, ty, tidx, k, k, s, s, p, p, dil, dil, bool(ceil))
+        THNN.SpatialDilatedMaxPooling_updateGradInput(x, gy, tgx, tidx, k, k, s, s, p, p, dil, dil, bool(ceil))
+        y, idx, gx = ty.numpy(), tidx.numpy(), tgx.numpy()
+    assert np.array_equal(y, c["max_y"]) and np.array_equal(idx, c["max_idx"])   # bit-exact
+    close(gx, c["max_gx"])
+
+
+def test_dilated_convolution_golden(backend):
+    c = case("dilconv_d2")
+    g = [int(v) for v in c["geom"]]
+    Co, K = c["w"].shape[0], int(np.prod(c["w"].shape[1:]))
+    if backend.name == "oracle":
+        y = O.dilconv_updateOutput(c["x"], c["w"], c["b"], *g)
+        gx = O.dilconv_updateGradInput(c["x"].shape, c["gy"], c["w"], *g)
+        gw, gb = O.dilconv_accGradParameters(c["x"], c["gy"], np.zeros((Co, K), np.float32), np.zeros_like(c["b"]), *g, 1.0)
+    else:
+        CT, _, THNN = _hip()
+        x, w, b, gy = (CT.from_numpy(c[k]) for k in ("x", "w", "b", "gy"))
+        ty, tgx, cols, gcols, ones = CT(), CT(), CT(), CT(), CT()
+        tgw, tgb = CT.from_numpy(np.zeros_like(c["w"])), CT.from_numpy(np.zeros_like(c["b"]))
+        THNN.SpatialDilatedConvolution_updateOutput(x, ty, w, b, cols, ones, *g)
+        THNN.SpatialDilatedConvolution_updateGradInput(x, gy, tgx, w, gcols, *g)
+        THNN.SpatialDilatedConvolution_accGradParameters(x, gy, tgw, tgb, cols, ones, *g, 1.0)
+        y, gx, gw, gb = ty.numpy(), tgx.numpy(), tgw.numpy(), tgb.numpy()
+    close(y, c["y"]); close(gx, c["gx"])
+    close(np.asarray(gw).reshape(c["gw"].shape), c["gw"], 1e-3, 1e-3); close(gb, c["gb"], 1e-3, 1e-3)
+
+
+def test_transposed_convolution_golden(backend):
+    c = case("fullconv_s2")
+    k, _, s, _, p, _, adj, _ = [int(v) for v in c["geom"]]
+    if backend.name == "oracle":
+        og = (k, k, s, s, p, p, 1, 1, adj, adj)
+        y = O.fullconv_updateOutput(c["x"], c["w"], c["b"], *og)
+        gx = O.fullconv_updateGradInput(c["x"].shape, c["gy"], c["w"], *og)
+        gw, gb = O.fullconv_accGradParameters(c["x"], c["gy"], np.zeros_like(c["w"]), np.zeros_like(c["b"]), *og, scale=1.0)
+    else:
+        CT, _, THNN = _hip()
+        g = (k, k, s, s, p, p, adj, adj)
+        x, w, b, gy = (CT.from_numpy(c[n]) for n in ("x", "w", "b", "gy"))
+        ty, tgx, cols, gcols, ones = CT(), CT(), CT(), CT(), CT()
+        tgw, tgb = CT.from_numpy(np.zeros_like(c["w"])), CT.from_numpy(np.zeros_like(c["b"]))
+        THNN.SpatialFullConvolution_updateOutput(x, ty, w, b, cols, ones, *g)
+        THNN.SpatialFullConvolution_updateGradInput(x, gy, tgx, w, gcols, *g)
+        THNN.SpatialFullConvolution_accGradParameters(x, gy, tgw, tgb, cols, ones, *g, 1.0)
+        y, gx, gw, gb = ty.numpy(), tgx.numpy(), tgw.numpy(), tgb.numpy()
+    close(y, c["y"]); close(gx, c["gx"])
+    close(np.asarray(gw).reshape(c["gw"].shape), c["gw"], 1e-3, 1e-3); close(gb, c["gb"], 1e-3, 1e-3)
+
+
+def test_threshold_golden(backend):
+    c = case("thr")
+    th, val = float(c["param"][0]), float(c["param"][1])
+    if backend.name == "oracle":
+        y, gx = O.threshold_updateOutput(c["x"], th, val), O.threshold_updateGradInput(c["x"], c["gy"], th)
+    else:
+        CT, _, THNN = _hip()
+        x, gy, ty, tgx = CT.from_numpy(c["x"]), CT.from_numpy(c["gy"]), CT(), CT()
+        THNN.Threshold_updateOutput(x, ty, th, val, False)
+        THNN.Threshold_updateGradInput(x, gy, tgx, th, val, False)
+        y, gx = ty.numpy(), tgx.numpy()
+    assert np.array_equal(y, c["y"]) and np.array_equal(gx, c["gx"])   # bit-exact: a select, no arithmetic
+
+
+def test_batchnorm_relu_golden(backend):
+    """The pair BatchNormalization (train) -> Threshold(0, 0): the oracle as the composition of its two functions, the
+    library through its fused entry points (include/THCUNN_fused.h)."""
+    c = case("bnrelu_4d")
+    C = c["g"].shape[0]
+    if backend.name == "oracle":
+        rm, rv = np.zeros(C, np.float32), np.ones(C, np.float32)
+        y, sm, ss = O.bn_updateOutput(c["x"], c["g"], c["b"], rm, rv, True, 0.1, 1e-5)
+        a = O.threshold_updateOutput(y, 0.0, 0.0)
+        gx, gw, gb = O.bn_backward(c["x"], O.threshold_updateGradInput(y, c["ga"], 0.0), c["g"], rm, rv, sm, ss, True, 1.0, 1e-5,
+                                   np.zeros(C, np.float32), np.zeros(C, np.float32))
+    else:
+        CT, _, THNN = _hip()
+        x, g, b, ga = (CT.from_numpy(c[k]) for k in ("x", "g", "b", "ga"))
+        rm, rv = CT.from_numpy(np.zeros(C, np.float32)), CT.from_numpy(np.ones(C, np.float32))
+        sm, ss, ta, tgx = CT.with_size(C), CT.with_size(C), CT(), CT.with_size(*c["x"].shape)
+        tgw, tgb = CT.from_numpy(np.zeros(C, np.float32)), CT.from_numpy(np.zeros(C, np.float32))
+        THNN.BatchNormalizationReLU_updateOutput(x, ta, g, b, rm, rv, sm, ss, True, 0.1, 1e-5)
+        THNN.BatchNormalizationReLU_backward(x, ga, tgx, tgw, tgb, g, b, rm, rv, sm, ss, True, 1.0, 1e-5)
+        a, gx, gw, gb = ta.numpy(), tgx.numpy(), tgw.numpy(), tgb.numpy()
+    close(a, c["a"], 1e-5, 1e-4); close(gx, c["gx"], 1e-5, 1e-4); close(gw, c["gw"], 1e-3, 1e-3); close(gb, c["gb"], 1e-3, 1e-3)

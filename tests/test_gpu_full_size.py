@@ -140,6 +140,17 @@ def test_cfg5_convmm(T):
     lhs = dot(yv - b[None, :, None, None], gy)
     assert abs(lhs - dot(x, gxv)) <= 1e-4 * abs(lhs) + 5.0
     assert abs(lhs - dot(w, gwv)) <= 1e-4 * abs(lhs) + 5.0
+    # gradWeight of the whole batch (the call that plans the many-way position split, its partial tiles and their
+    # fold), element by element against the same sum in float64: per image the im2col matrix as a strided view of
+    # the zero-padded image (2304 x 784) times gradOutput (256 x 784) transposed, 59 GFLOP of float64 BLAS
+    ref = np.zeros((Co, K))
+    xp = np.zeros((Ci, H + 2, H + 2))
+    for n in range(N):
+        xp[:, 1:-1, 1:-1] = x[n]
+        win = np.lib.stride_tricks.sliding_window_view(xp, (3, 3), axis=(1, 2))      # (Ci, H, H, 3, 3)
+        col = win.transpose(0, 3, 4, 1, 2).reshape(K, H * H)                        # row (c, kh, kw), column (oh, ow)
+        ref += gy[n].reshape(Co, H * H).astype(np.float64) @ col.T
+    np.testing.assert_allclose(gwv, ref, rtol=1e-3, atol=0.05)   # values are +-224 (50 176 terms of unit variance)
     # gradWeight against the oracle on the first four images (the full batch takes the CPU minutes)
     sub = slice(0, 4)
     gws = CT.from_numpy(np.zeros_like(w))

@@ -311,6 +311,37 @@ def test_bn_vs_torch_train_and_eval():
     assert np.array_equal(gi, gi2) and np.array_equal(gw, gw2) and np.array_equal(gb, gb2)
 
 
+def test_bn_eval_mode_parameter_gradients():
+    """Evaluation mode takes mean and 1/sigma from the running statistics for the parameter gradients too
+    (lib/THCUNN/BatchNormalization.cu:237-240, 272-282): gradWeight += scale * sum(gy * (x - runningMean)) /
+    sqrt(runningVar + eps), gradBias += scale * sum(gy), on top of what the tensors held. Checked against those
+    closed forms in float64 and against autograd through F.batch_norm(training=False), with running statistics
+    that differ from the batch's and from (0, 1), a scale that is not 1 and accumulators that are not 0."""
+    rng = np.random.default_rng(11)
+    shape, C, eps, scale = (5, 3, 6, 7), 3, 1e-3, 0.75
+    x = (rng.standard_normal(shape) * 1.5 - 0.3).astype(np.float32)
+    gy = rng.standard_normal(shape).astype(np.float32)
+    g = (rng.random(C) + 0.5).astype(np.float32)
+    rm = rng.standard_normal(C).astype(np.float32)
+    rv = (rng.random(C) * 2 + 0.25).astype(np.float32)
+    gw0, gb0 = rng.standard_normal(C).astype(np.float32), rng.standard_normal(C).astype(np.float32)
+    # saveMean / saveStd of some training step: must not enter the evaluation-mode formulas
+    sm, ss = np.full(C, 123.0, np.float32), np.full(C, 456.0, np.float32)
+    gi, gw, gb = O.bn_backward(x, gy, g, rm, rv, sm, ss, False, scale, eps, gw0.copy(), gb0.copy())
+    x64, gy64 = x.astype(np.float64), gy.astype(np.float64)
+    inv = 1.0 / np.sqrt(rv.astype(np.float64) + eps)
+    want_gw = gw0 + scale * (gy64 * (x64 - rm[None, :, None, None])).sum(axis=(0, 2, 3)) * inv
+    want_gb = gb0 + scale * gy64.sum(axis=(0, 2, 3))
+    close(gw, want_gw, 1e-5, 1e-5); close(gb, want_gb, 1e-5, 1e-5)
+    close(gi, gy64 * (g * inv)[None, :, None, None], 1e-5, 1e-6)
+    tx = torch.from_numpy(x).double().requires_grad_()
+    tg, tb = torch.from_numpy(g).double().requires_grad_(), torch.zeros(C, dtype=torch.float64, requires_grad=True)
+    F.batch_norm(tx, torch.from_numpy(rm).double(), torch.from_numpy(rv).double(), tg, tb, False, 0.1, eps).backward(
+        torch.from_numpy(gy).double())
+    close(gw, gw0 + scale * tg.grad.numpy(), 1e-5, 1e-5); close(gb, gb0 + scale * tb.grad.numpy(), 1e-5, 1e-5)
+    close(gi, tx.grad.numpy(), 1e-5, 1e-6)
+
+
 def test_bn_zero_variance_zero_eps():
     """invStd = 0 when varN == 0 and eps == 0 (lib/THCUNN/BatchNormalization.cu:188-191)."""
     x = np.full((2, 1, 3), 4.0, np.float32)

@@ -726,7 +726,7 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=F
                     ms_per_step_bracketed=round(wall_ev * 1e3 / steps, 5),
                     empty_bracket_ms=round(float(np.median(emp[None])), 5))
     extra = PREROLL_SAMPLES
-    if ncold > 1 and ncold >= 2 * len(names):
+    if ncold > len(names):
         # cache-cold variant, outside the timed steps: the same entry points, each on a buffer set that nothing has
         # touched for at least `stride` - 1 whole steps (more than 1 GB of traffic at cfg2)
         run(ncold, [], cold=True)

@@ -16,6 +16,7 @@
 #include "strip.h"
 #include "thc_internal.h"
 
+#include <atomic>
 #include <mutex>
 
 using namespace thc;
@@ -302,10 +303,12 @@ dwAccGradStage1(const float *__restrict__ in, const float *__restrict__ gradOut,
       if (lane == 0) red[wave][t] = v;
     }
     __syncthreads();
-    if (threadIdx.x < T) {
+    if (threadIdx.x < partialPitch(T)) {  // the whole run, padding included: stage 2 reads whole runs, also from scratch that is reused
       float v = 0.f;
+      if (threadIdx.x < T) {
 #pragma unroll
-      for (int w = 0; w < nWaves; ++w) v += red[w][threadIdx.x];
+        for (int w = 0; w < nWaves; ++w) v += red[w][threadIdx.x];
+      }
       partial[((long)slot * (g.C * g.M) + c * g.M + j) * partialPitch(T) + threadIdx.x] = v;
     }
   }
@@ -940,6 +943,7 @@ static __device__ __align__(256) float scratch[kNoAllocScratchFloats];
 constexpr int kMaxDevices = 64;
 std::mutex g_scratchMutex;
 float *g_scratchPtr[kMaxDevices];  // per device: that GPU's copy of `scratch`
+std::atomic<int> g_scratchBusy[kMaxDevices];  // per device: a host thread is inside the no-allocation entry point
 
 // Address of the current device's copy of the array; `device` must be the current device.
 float *noAllocScratch(int device) {
@@ -1282,6 +1286,20 @@ void THNN_CudaSpatialDepthWiseConvolution_accGradParameters_noAlloc(THCState *st
   DwScratch sc;
   sc.noAlloc = true;
   sc.fixed = noAllocScratch(device);  // looked up when the state was made; a table read here
+  // All calls on a GPU share that array. Two host threads inside this entry point for the same GPU at once are
+  // refused; calls that overlap only on the GPU (one thread, two streams) cannot be seen from here without a
+  // synchronising or allocating call and remain the caller's to order.
+  struct Busy {
+    std::atomic<int> &f;
+    bool mine;
+    explicit Busy(std::atomic<int> &flag) : f(flag), mine(flag.exchange(1) == 0) {}
+    ~Busy() {
+      if (mine) f.store(0);
+    }
+  } busy(g_scratchBusy[device]);
+  if (!busy.mine)
+    error("SpatialDepthWiseConvolution_accGradParameters_noAlloc: another thread is inside this entry point on "
+          "device %d; the calls share one scratch array per GPU and must not overlap", device);
   dwAccGradParameters(state, input, gradOutput, gradWeight, gradBias, sc, kW, kH, dW, dH, padW, padH, scale);
   THNN_LEAVE
 }

@@ -104,3 +104,65 @@ def test_no_alloc_refuses_what_would_allocate(T):
     THNN.SpatialDepthWiseConvolution_accGradParameters(xs, CT.from_numpy(gy), gw, gb, CT(), CT(), *g, 1.0)
     rgw, rgb = O.dwconv_accGradParameters(x, gy, np.zeros((1, 4, 3, 3), np.float32), np.zeros((1, 4), np.float32), *g, 1.0)
     np.testing.assert_allclose(gw.numpy(), rgw, rtol=WG_RTOL, atol=WG_ATOL)
+
+
+def test_no_alloc_two_host_threads_never_share_the_scratch_silently(T):
+    """All calls on a GPU share one scratch array. Two host threads that are inside the entry point at the same time
+    are told so (TH error, nothing launched) instead of folding each other's partial sums; a call that does go
+    through gives the regular entry point's bits. Both threads issue on the device's default stream, so the launches
+    of calls that did not overlap on the host do not overlap on the GPU either."""
+    import threading
+
+    from cunn_amd import tensor as TT
+    lib = T._lib.load()
+    CT, THNN = T.CudaTensor, T.THNN
+    g = (3, 3, 2, 2, 1, 1)
+    work = []
+    for seed, (N, C) in enumerate(((8, 32), (6, 24))):
+        rng = np.random.default_rng(40 + seed)
+        x, gy = rng.standard_normal((N, C, 56, 56)).astype(np.float32), rng.standard_normal((N, C, 28, 28)).astype(np.float32)
+        gw0, gb0 = rng.standard_normal((1, C, 3, 3)).astype(np.float32), rng.standard_normal((1, C)).astype(np.float32)
+        tx, tgy = CT.from_numpy(x), CT.from_numpy(gy)
+        ref_w, ref_b = CT.from_numpy(gw0), CT.from_numpy(gb0)
+        THNN.SpatialDepthWiseConvolution_accGradParameters(tx, tgy, ref_w, ref_b, CT(), CT(), *g, 1.0)
+        work.append(dict(x=tx, gy=tgy, gw0=gw0, gb0=gb0, ref_w=ref_w.numpy(), ref_b=ref_b.numpy(),
+                         gw=CT.from_numpy(gw0), gb=CT.from_numpy(gb0), done=0, refused=0, wrong=0))
+    TT.synchronize()
+    del TT._pending[:]
+    ROUNDS = 200
+
+    import ctypes as C
+
+    def put(st, t, a):      # the harness's own copy helpers raise on any pending TH error, also the other thread's
+        lib.THCudaTensor_copyFromHost(st, t.handle, a.ctypes.data_as(C.c_void_p))
+
+    def get(st, t, like):
+        out = np.empty_like(like)
+        lib.THCudaTensor_copyToHost(st, t.handle, out.ctypes.data_as(C.c_void_p))
+        return out
+
+    def run(w):
+        st = lib.THCState_alloc()
+        for _ in range(ROUNDS):
+            put(st, w["gw"], w["gw0"]), put(st, w["gb"], w["gb0"])
+            lib.THNN_CudaSpatialDepthWiseConvolution_accGradParameters_noAlloc(
+                st, w["x"].handle, w["gy"].handle, w["gw"].handle, w["gb"].handle, *g, 1.0)
+            lib.THCState_synchronize(st)
+            gw, gb = get(st, w["gw"], w["gw0"]), get(st, w["gb"], w["gb0"])
+            if np.array_equal(gw, w["ref_w"]) and np.array_equal(gb, w["ref_b"]):
+                w["done"] += 1
+            elif np.array_equal(gw, w["gw0"]) and np.array_equal(gb, w["gb0"]):
+                w["refused"] += 1
+            else:
+                w["wrong"] += 1
+        lib.THCState_free(st)
+
+    threads = [threading.Thread(target=run, args=(w,)) for w in work]
+    [t.start() for t in threads]
+    [t.join() for t in threads]
+    errors = list(TT._pending)
+    del TT._pending[:]
+    print("done", [w["done"] for w in work], "refused", [w["refused"] for w in work], flush=True)
+    assert all(w["wrong"] == 0 for w in work)
+    assert all(w["done"] > 0 for w in work)
+    assert len(errors) == sum(w["refused"] for w in work) and all("must not overlap" in e for e in errors)

@@ -898,8 +898,8 @@ void bnUpdateOutput(THCState *state, THCudaTensor *input_, THCudaTensor *output_
     return;
   }
   if (train) {
-    Temp partial(s, (size_t)g.C * g.chunks * 3 * sizeof(float));
-    float *p = (float *)partial.get();
+    // chunk statistics: BatchNormalization has no buffer argument, they live in the stream's scratch space
+    float *p = (float *)streamScratch(state, (size_t)g.C * g.chunks * 3 * sizeof(float));
 #define BN_FWD_TRAIN(MODE)                                                                                        \
   {                                                                                                               \
     bnStatsKernel<MODE><<<grid, block, 0, s>>>(in.ptr(), p, g);                                                   \
@@ -1013,11 +1013,9 @@ void bnBackward(THCState *state, THCudaTensor *input_, THCudaTensor *gradOutput_
     THC_HIP_CHECK(hipGetLastError());
     return;
   }
-  Temp partial;
   float *p = nullptr;
   if (needSums) {
-    partial = Temp(s, (size_t)g.C * g.chunks * 2 * sizeof(float));
-    p = (float *)partial.get();
+    p = (float *)streamScratch(state, (size_t)g.C * g.chunks * 2 * sizeof(float));
     if (v.mode == 1)
       bnGradSumsKernel<1><<<grid, block, 0, s>>>(in.ptr(), go.ptr(), p, meanSrc, g, rm);
     else if (v.mode == 2)

@@ -12,9 +12,18 @@
 
 #include "../../include/THCUNN.h"
 
-struct THCState {
-  int device;
+// Per stream: a block of device memory that entry points without a buffer argument use for their partial results
+// (cutorch keeps such a scratch space per device and stream as well). It grows on demand and lives as long as the state.
+struct StreamScratch {
   hipStream_t stream;
+  void *ptr;
+  size_t bytes;
+};
+
+struct THCState {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  std::vector<StreamScratch> scratch;
 };
 
 namespace thc {
@@ -118,6 +127,11 @@ inline long *data(const THCudaLongTensor *t) {
 
 // strided gather src(size,stride) -> dst contiguous (or the reverse scatter)
 void stridedCopy(hipStream_t stream, const Tensor *t, void *contig, size_t elemSize, bool toContig);
+
+// At least `bytes` of device memory that belongs to (state, current stream) and is reused by every call on that
+// stream: work that uses it is ordered by the stream. Allocates only when a call needs more than any earlier call
+// on the stream did (then the stream is drained before the smaller block is freed).
+void *streamScratch(THCState *state, size_t bytes);
 
 // Stream-ordered temporary: memory is returned to the pool after the work
 // queued so far on `stream` has drained, with no host synchronisation.

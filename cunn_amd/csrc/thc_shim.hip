@@ -86,6 +86,28 @@ static Switches switchesFromEnvironment() {
 }
 Switches g_switches = switchesFromEnvironment();  // read once, when the library is loaded
 
+// ------------------------------------------------------- per-stream scratch ----
+void *streamScratch(THCState *state, size_t bytes) {
+  StreamScratch *slot = nullptr;
+  for (StreamScratch &sc : state->scratch)
+    if (sc.stream == state->stream) slot = &sc;
+  if (!slot) {
+    state->scratch.push_back(StreamScratch{state->stream, nullptr, 0});
+    slot = &state->scratch.back();
+  }
+  if (slot->bytes < bytes) {
+    if (slot->ptr) {
+      THC_HIP_CHECK(hipStreamSynchronize(state->stream));
+      THC_HIP_CHECK(hipFree(slot->ptr));
+      slot->ptr = nullptr, slot->bytes = 0;
+    }
+    const size_t want = (bytes + 65535) / 65536 * 65536;
+    THC_HIP_CHECK(hipMalloc(&slot->ptr, want));
+    slot->bytes = want;
+  }
+  return slot->ptr;
+}
+
 // --------------------------------------------------------------- storage ----
 static Storage *storageNew(int device) {
   Storage *s = (Storage *)calloc(1, sizeof(Storage));
@@ -371,14 +393,19 @@ extern "C" {
 THCState *THCState_alloc(void) {
   THCState *s = nullptr;
   THNN_ENTER
-  s = (THCState *)calloc(1, sizeof(THCState));
+  s = new THCState();
   THC_HIP_CHECK(hipGetDevice(&s->device));
   s->stream = nullptr;  // the device's default stream
   dwNoAllocInit(s->device);
   THNN_LEAVE
   return s;
 }
-void THCState_free(THCState *state) { free(state); }
+void THCState_free(THCState *state) {
+  if (!state) return;
+  for (StreamScratch &sc : state->scratch)
+    if (sc.ptr) (void)hipFree(sc.ptr);  // waits for the device: nothing still reads the block
+  delete state;
+}
 void THCState_setCurrentStream(THCState *state, void *hipStream) { state->stream = (hipStream_t)hipStream; }
 void *THCState_getCurrentStream(THCState *state) { return (void *)state->stream; }
 void THCState_synchronize(THCState *state) {

@@ -3,7 +3,10 @@ allocates nor synchronises, so a caller may capture a sequence of calls on the s
 The captured sequence is replayed three times, with the program's own eager calls and synchronisations between
 the replays, and every replay has to give the eager results bit for bit. The depthwise weight gradient is
 captured through its no-allocation variant (the one meant for such callers) and through the regular entry point
-with the caller's scratch tensor already sized.
+with the caller's scratch tensor already sized. BatchNormalization, which has no buffer argument, is captured on
+both of its kernel families: 48 channels of 14 x 14 take the chunked two-pass kernels, whose chunk statistics
+live in the state's per-stream scratch space (sized by the eager calls before the capture), 96 channels of
+28 x 28 the kernels that keep a channel in registers.
 """
 import ctypes as C
 
@@ -29,11 +32,13 @@ def test_replays_of_a_captured_step_match_eager():
     cv = dict(x=CT.from_numpy(f(N, Ci, 28, 28)), w=CT.from_numpy(f(Co, Ci * 9) * 0.05), b=CT.from_numpy(f(Co)), gy=CT.from_numpy(f(N, Co, 28, 28)),
               y=CT(), gx=CT(), gw=CT.from_numpy(np.zeros((Co, Ci * 9), np.float32)), gb=CT.from_numpy(np.zeros(Co, np.float32)),
               cols=CT(), gcols=CT(), wcols=CT(), ones=CT())
-    Cb = 48
-    z = lambda: CT.from_numpy(np.zeros(Cb, np.float32))
-    bn = dict(x=CT.from_numpy(f(N, Cb, 14, 14)), gy=CT.from_numpy(f(N, Cb, 14, 14)), y=CT(), gx=CT.with_size(N, Cb, 14, 14),
-              g=CT.from_numpy(rng.random(Cb).astype(np.float32)), b=CT.from_numpy(f(Cb)), rm=z(), rv=CT.from_numpy(np.ones(Cb, np.float32)),
-              sm=CT.with_size(Cb), ss=CT.with_size(Cb), gw=z(), gb=z())
+    def make_bn(Cb, hw):
+        z = lambda: CT.from_numpy(np.zeros(Cb, np.float32))
+        return dict(x=CT.from_numpy(f(N, Cb, hw, hw)), gy=CT.from_numpy(f(N, Cb, hw, hw)), y=CT(), gx=CT.with_size(N, Cb, hw, hw),
+                    g=CT.from_numpy(rng.random(Cb).astype(np.float32)), b=CT.from_numpy(f(Cb)), rm=z(),
+                    rv=CT.from_numpy(np.ones(Cb, np.float32)), sm=CT.with_size(Cb), ss=CT.with_size(Cb), gw=z(), gb=z())
+
+    bn, bn2 = make_bn(48, 14), make_bn(96, 28)
     mp = dict(x=CT.from_numpy(f(N, 16, 57, 57)), y=CT(), idx=LT(), gy=CT.from_numpy(f(N, 16, 29, 29)), gx=CT())
     h = lambda t: None if t is None else t.handle
     st = state()
@@ -51,17 +56,19 @@ def test_replays_of_a_captured_step_match_eager():
         lib.THCudaTensor_fill(st, h(cv["gw"]), 0.0)
         lib.THCudaTensor_fill(st, h(cv["gb"]), 0.0)
         lib.THNN_CudaSpatialConvolutionMM_accGradParameters(st, h(cv["x"]), h(cv["gy"]), h(cv["gw"]), h(cv["gb"]), h(cv["wcols"]), h(cv["ones"]), *c, 1.0)
-        lib.THCudaTensor_fill(st, h(bn["rm"]), 0.0)
-        lib.THCudaTensor_fill(st, h(bn["rv"]), 1.0)
-        lib.THNN_CudaBatchNormalization_updateOutput(st, h(bn["x"]), h(bn["y"]), h(bn["g"]), h(bn["b"]), h(bn["rm"]), h(bn["rv"]), h(bn["sm"]), h(bn["ss"]), True, 0.1, 1e-5)
-        lib.THCudaTensor_fill(st, h(bn["gw"]), 0.0)
-        lib.THCudaTensor_fill(st, h(bn["gb"]), 0.0)
-        lib.THNN_CudaBatchNormalization_backward(st, h(bn["x"]), h(bn["gy"]), h(bn["gx"]), h(bn["gw"]), h(bn["gb"]), h(bn["g"]), h(bn["rm"]), h(bn["rv"]), h(bn["sm"]), h(bn["ss"]), True, 1.0, 1e-5)
+        for b_ in (bn, bn2):
+            lib.THCudaTensor_fill(st, h(b_["rm"]), 0.0)
+            lib.THCudaTensor_fill(st, h(b_["rv"]), 1.0)
+            lib.THNN_CudaBatchNormalization_updateOutput(st, h(b_["x"]), h(b_["y"]), h(b_["g"]), h(b_["b"]), h(b_["rm"]), h(b_["rv"]), h(b_["sm"]), h(b_["ss"]), True, 0.1, 1e-5)
+            lib.THCudaTensor_fill(st, h(b_["gw"]), 0.0)
+            lib.THCudaTensor_fill(st, h(b_["gb"]), 0.0)
+            lib.THNN_CudaBatchNormalization_backward(st, h(b_["x"]), h(b_["gy"]), h(b_["gx"]), h(b_["gw"]), h(b_["gb"]), h(b_["g"]), h(b_["rm"]), h(b_["rv"]), h(b_["sm"]), h(b_["ss"]), True, 1.0, 1e-5)
         lib.THNN_CudaSpatialMaxPooling_updateOutput(st, h(mp["x"]), h(mp["y"]), h(mp["idx"]), 3, 3, 2, 2, 1, 1, False)
         lib.THNN_CudaSpatialMaxPooling_updateGradInput(st, h(mp["x"]), h(mp["gy"]), h(mp["gx"]), h(mp["idx"]), 3, 3, 2, 2, 1, 1, False)
 
     outs = [dw["y"], dw["gx"], dw["gw"], dw["gb"], dw["gw2"], dw["gb2"], cv["y"], cv["gx"], cv["gw"], cv["gb"], bn["y"], bn["gx"], bn["gw"],
-            bn["gb"], bn["rm"], bn["rv"], bn["sm"], bn["ss"], mp["y"], mp["idx"], mp["gx"]]
+            bn["gb"], bn["rm"], bn["rv"], bn["sm"], bn["ss"], bn2["y"], bn2["gx"], bn2["gw"], bn2["gb"], bn2["sm"], bn2["ss"],
+            mp["y"], mp["idx"], mp["gx"]]
     results = lambda: [t.numpy().copy() for t in outs]
 
     def scribble():

@@ -572,6 +572,108 @@ def wl_convrelu(nsets, fused=True):
                      + ("fused entry point" if fused else "two separate calls"))
 
 
+def wl_mbv1_block(nsets):
+    """Beyond the five configurations: one MobileNet-v1 block at the shape of the metric's layer, forward then backward
+    in network order - depthwise 3x3 stride 2 (128 planes, 56x56 -> 28x28) -> BatchNormalization + ReLU -> 1x1
+    convolution 128 -> 128 -> BatchNormalization + ReLU, and back. All five module families of the path and the fused
+    entry points in one stream: the forward and the backward pass of a layer are eight to nine launches apart, so no
+    backward kernel finds its operands where the forward kernel left them."""
+    from cunn_amd import CudaTensor as CT, THNN
+    from oracle import oracle as O
+    N, Cc, H, oH = 64, 128, 56, 28
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((N, Cc, H, H)).astype(np.float32)
+    wd = _kaiming_uniform(rng, (1, Cc, 3, 3), 9)
+    bd = rng.uniform(-1 / 3, 1 / 3, (1, Cc)).astype(np.float32)
+    wp = (rng.standard_normal((Cc, Cc)) * np.sqrt(2.0 / Cc)).astype(np.float32)
+    bp = rng.uniform(-0.02, 0.02, Cc).astype(np.float32)
+    g1, b1 = (rng.random(Cc) + 0.5).astype(np.float32), (rng.standard_normal(Cc) * 0.1).astype(np.float32)
+    g2, b2 = (rng.random(Cc) + 0.5).astype(np.float32), (rng.standard_normal(Cc) * 0.1).astype(np.float32)
+    ga2 = rng.standard_normal((N, Cc, oH, oH)).astype(np.float32)      # gradient arriving from the next block
+    z = lambda n=Cc: CT.from_numpy(np.zeros(n, np.float32))
+    one = lambda: CT.from_numpy(np.ones(Cc, np.float32))
+    sets = []
+    for _ in range(nsets):
+        sets.append(dict(
+            x=CT.from_numpy(x), wd=CT.from_numpy(wd), bd=CT.from_numpy(bd), wp=CT.from_numpy(wp), bp=CT.from_numpy(bp),
+            g1=CT.from_numpy(g1), b1=CT.from_numpy(b1), g2=CT.from_numpy(g2), b2=CT.from_numpy(b2), ga2=CT.from_numpy(ga2),
+            y1=CT(), a1=CT(), y2=CT(), a2=CT(), gy2=CT.with_size(N, Cc, oH, oH), ga1=CT(), gy1=CT.with_size(N, Cc, oH, oH), gx=CT(),
+            rm1=z(), rv1=one(), sm1=CT.with_size(Cc), ss1=CT.with_size(Cc), rm2=z(), rv2=one(), sm2=CT.with_size(Cc), ss2=CT.with_size(Cc),
+            gg1=z(), gb1=z(), gg2=z(), gb2=z(), gwd=CT.from_numpy(np.zeros_like(wd)), gbd=CT.from_numpy(np.zeros_like(bd)),
+            gwp=CT.from_numpy(np.zeros_like(wp)), gbp=z(), cd=CT(), od=CT(), cp=CT(), gcp=CT(), wcp=CT(), op=CT()))
+    gd, gp = (3, 3, 2, 2, 1, 1), (1, 1, 1, 1, 0, 0)
+
+    def calls(i):
+        t = sets[i]
+        return [
+            ("dw_updateOutput", lambda: THNN.SpatialDepthWiseConvolution_updateOutput(t["x"], t["y1"], t["wd"], t["bd"], t["cd"], t["od"], *gd)),
+            ("bnrelu1_updateOutput", lambda: THNN.BatchNormalizationReLU_updateOutput(
+                t["y1"], t["a1"], t["g1"], t["b1"], t["rm1"], t["rv1"], t["sm1"], t["ss1"], True, 0.1, 1e-5)),
+            ("pw_updateOutput", lambda: THNN.SpatialConvolutionMM_updateOutput(t["a1"], t["y2"], t["wp"], t["bp"], t["cp"], t["op"], *gp)),
+            ("bnrelu2_updateOutput", lambda: THNN.BatchNormalizationReLU_updateOutput(
+                t["y2"], t["a2"], t["g2"], t["b2"], t["rm2"], t["rv2"], t["sm2"], t["ss2"], True, 0.1, 1e-5)),
+            ("bnrelu2_backward", lambda: THNN.BatchNormalizationReLU_backward(
+                t["y2"], t["ga2"], t["gy2"], t["gg2"], t["gb2"], t["g2"], t["b2"], t["rm2"], t["rv2"], t["sm2"], t["ss2"], True, 1.0, 1e-5)),
+            ("pw_updateGradInput", lambda: THNN.SpatialConvolutionMM_updateGradInput(t["a1"], t["gy2"], t["ga1"], t["wp"], t["gcp"], t["op"], *gp)),
+            ("pw_accGradParameters", lambda: THNN.SpatialConvolutionMM_accGradParameters(
+                t["a1"], t["gy2"], t["gwp"], t["gbp"], t["wcp"], t["op"], *gp, 1.0)),
+            ("bnrelu1_backward", lambda: THNN.BatchNormalizationReLU_backward(
+                t["y1"], t["ga1"], t["gy1"], t["gg1"], t["gb1"], t["g1"], t["b1"], t["rm1"], t["rv1"], t["sm1"], t["ss1"], True, 1.0, 1e-5)),
+            ("dw_updateGradInput", lambda: THNN.SpatialDepthWiseConvolution_updateGradInput(t["x"], t["gy1"], t["gx"], t["wd"], t["cd"], t["od"], *gd)),
+            ("dw_accGradParameters", lambda: THNN.SpatialDepthWiseConvolution_accGradParameters(
+                t["x"], t["gy1"], t["gwd"], t["gbd"], t["cd"], t["od"], *gd, 1.0)),
+        ]
+
+    xb, yb = x.nbytes, ga2.nbytes
+    # algorithmic bytes, every tensor of an entry point once; the 1x1 convolution with 128-term sums moves 2 x 25.7 MB for
+    # 1.64 GFLOP (10 us of the matrix pipe): bound by memory like the rest of the block
+    work = {"dw_updateOutput": (xb + yb, "bytes"), "bnrelu1_updateOutput": (2 * yb, "bytes"), "pw_updateOutput": (2 * yb, "bytes"),
+            "bnrelu2_updateOutput": (2 * yb, "bytes"), "bnrelu2_backward": (3 * yb, "bytes"), "pw_updateGradInput": (2 * yb, "bytes"),
+            "pw_accGradParameters": (2 * yb, "bytes"), "bnrelu1_backward": (3 * yb, "bytes"), "dw_updateGradInput": (xb + yb, "bytes"),
+            "dw_accGradParameters": (xb + yb, "bytes")}
+
+    def oracle_forward():
+        y1 = O.dwconv_updateOutput(x, wd, bd, *gd)
+        n1, sm1, ss1 = O.bn_updateOutput(y1, g1, b1, np.zeros(Cc, np.float32), np.ones(Cc, np.float32), True, 0.1, 1e-5)
+        a1 = O.threshold_updateOutput(n1, 0.0, 0.0)
+        y2 = O.convmm_updateOutput(a1, wp, bp, *gp)
+        n2, sm2, ss2 = O.bn_updateOutput(y2, g2, b2, np.zeros(Cc, np.float32), np.ones(Cc, np.float32), True, 0.1, 1e-5)
+        return dict(y1=y1, n1=n1, a1=a1, y2=y2, n2=n2, a2=O.threshold_updateOutput(n2, 0.0, 0.0), sm1=sm1, ss1=ss1, sm2=sm2, ss2=ss2)
+
+    def cpu(reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            f = oracle_forward()
+            rm, rv = np.zeros(Cc, np.float32), np.ones(Cc, np.float32)
+            gy2, _, _ = O.bn_backward(f["y2"], O.threshold_updateGradInput(f["n2"], ga2, 0.0), g2, rm, rv, f["sm2"], f["ss2"], True, 1.0,
+                                      1e-5, np.zeros(Cc, np.float32), np.zeros(Cc, np.float32))
+            ga1 = O.convmm_updateGradInput(f["a1"].shape, gy2, wp, *gp)
+            O.convmm_accGradParameters(f["a1"], gy2, np.zeros_like(wp), np.zeros_like(bp), *gp, 1.0)
+            gy1, _, _ = O.bn_backward(f["y1"], O.threshold_updateGradInput(f["n1"], ga1, 0.0), g1, rm, rv, f["sm1"], f["ss1"], True, 1.0,
+                                      1e-5, np.zeros(Cc, np.float32), np.zeros(Cc, np.float32))
+            O.dwconv_updateGradInput(x.shape, gy1, wd, *gd)
+            O.dwconv_accGradParameters(x, gy1, np.zeros_like(wd), np.zeros_like(bd), *gd, 1.0)
+        return time.perf_counter() - t0, reps * N, f"{reps} full forward + backward passes of the block ({N} images each)"
+
+    def verify():
+        t = sets[0]
+        for _, fn in calls(0):
+            fn()
+        f = oracle_forward()
+        np.testing.assert_allclose(t["a1"].numpy(), f["a1"], rtol=1e-5, atol=1e-4)
+        # the second normalisation divides by the spread of a 128-term sum: deviations of the first stage pass through scaled
+        np.testing.assert_allclose(t["a2"].numpy(), f["a2"], rtol=1e-4, atol=1e-4)
+        for k in ("gg1", "gb1", "gg2", "gb2", "gwd", "gbd", "gwp", "gbp"):
+            t[k].fill(0.0)
+        for k in ("rm1", "rm2"):
+            t[k].fill(0.0)
+        for k in ("rv1", "rv2"):
+            t[k].fill(1.0)
+
+    return dict(calls=calls, work=work, images=N, cpu=cpu, verify=verify, bound="hbm",
+                desc=f"MobileNet-v1 block fwd+bwd fp32 N={N}: depthwise 3x3 s2 {Cc}x{H}x{H} -> BN+ReLU -> 1x1 {Cc}->{Cc} at {oH}x{oH} -> BN+ReLU")
+
+
 def wl_copy(nsets):
     """Calibration: plain device-to-device copy of 128 MB (2 x 128 MB of HBM traffic per launch)."""
     from cunn_amd import CudaTensor as CT
@@ -595,7 +697,7 @@ WORKLOADS = {"copy": wl_copy, "cfg1": lambda n: wl_dw("cfg1", n), "cfg2": lambda
              "dw147": lambda n: wl_dw("dw147", n), "dw14": lambda n: wl_dw("dw14", n), "pool71": lambda n: wl_pool(n, odd=True),
              "cfg5": wl_conv, "pw128": lambda n: wl_conv(n, pointwise=True), "conv1": lambda n: wl_conv(n, first=True), "dilconv": wl_dilconv, "fullconv": wl_fullconv, "relu": wl_relu,
              "bnrelu": wl_bnrelu, "bnrelu_unfused": lambda n: wl_bnrelu(n, fused=False),
-             "convrelu": wl_convrelu, "convrelu_unfused": lambda n: wl_convrelu(n, fused=False)}
+             "convrelu": wl_convrelu, "convrelu_unfused": lambda n: wl_convrelu(n, fused=False), "mbv1_block": wl_mbv1_block}
 
 
 PREROLL_SAMPLES = 12   # event samples per entry point collected before the timed region, whatever --warmup is

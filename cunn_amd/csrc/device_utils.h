@@ -103,6 +103,12 @@ __device__ __forceinline__ void bufStoreStream4(__amdgpu_buffer_rsrc_t r, int by
   __builtin_amdgcn_raw_buffer_store_b128(v, r, byteOff, 0, 2 | 16);
 }
 
+// two 64-bit values as one streaming 16-byte store
+__device__ __forceinline__ void bufStoreStream2L(__amdgpu_buffer_rsrc_t r, int byteOff, long a, long b) {
+  u32x4 v = {(unsigned)a, (unsigned)((unsigned long)a >> 32), (unsigned)b, (unsigned)((unsigned long)b >> 32)};
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, byteOff, 0, 2 | 16);
+}
+
 __device__ __forceinline__ int ceilDivPos(int a, int b) {  // ceil(a / b) for b > 0, any sign of a
   return (a >= 0) ? (a + b - 1) / b : -((-a) / b);
 }

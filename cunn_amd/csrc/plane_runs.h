@@ -127,10 +127,11 @@ __device__ __forceinline__ void smallZero(float *__restrict__ xs, int floats) { 
 __device__ __forceinline__ void smallStoreRun(float *__restrict__ tensor, long first, const float *__restrict__ os, int count) {
   const int lead = (int)(first & 3);
   float *base = tensor + (first - lead);
+  const __amdgpu_buffer_rsrc_t br = dev::makeRsrc(base, (long)(lead + count) * 4);
   for (int i = threadIdx.x; i * 4 < lead + count; i += dev::kBlock) {
     const int e = i * 4;
     if (e >= lead && e + 4 <= lead + count) {
-      dev::storeStream4(base + e, reinterpret_cast<const float4 *>(os)[i]);
+      dev::bufStoreStream4(br, e * 4, reinterpret_cast<const float4 *>(os)[i]);
     } else {
       for (int k = max(e, lead); k < min(e + 4, lead + count); ++k) base[k] = os[k];
     }
@@ -172,11 +173,12 @@ __device__ __forceinline__ void smallIssueIdx(SmallIdxRun &r, const long *__rest
 __device__ __forceinline__ void smallStoreIdxRun(long *__restrict__ tensor, long first, const int *__restrict__ is, int count) {
   const int lead = (int)(first & 1);
   long *base = tensor + (first - lead);
+  const __amdgpu_buffer_rsrc_t br = dev::makeRsrc(base, (long)(lead + count) * 8);
   for (int i = threadIdx.x; i * 2 < lead + count; i += dev::kBlock) {
     const int e = i * 2;
     if (e >= lead && e + 2 <= lead + count) {
       const int2 v = reinterpret_cast<const int2 *>(is)[i];
-      dev::storeStream2(base + e, (long)v.x, (long)v.y);
+      dev::bufStoreStream2L(br, e * 8, (long)v.x, (long)v.y);
     } else {
       for (int k = max(e, lead); k < min(e + 2, lead + count); ++k) base[k] = is[k];
     }

@@ -664,7 +664,7 @@ poolBwdStrip(const float *__restrict__ gradOut, const long *__restrict__ indices
   // kh = dy + PAD - qh*ST lies inside the window; dy is a run-time value. For max pooling the argmax
   // test alone decides (a window that does not cover the element cannot point at it).
   const int total = nRows * W4;
-  float *o = gradIn + ((long)plane * g.H + h0) * g.W;
+  const __amdgpu_buffer_rsrc_t orr = dev::makeRsrc(gradIn + ((long)plane * g.H + h0) * g.W, (long)total * 16);
   for (int i = threadIdx.x; i < total; i += blockDim.x) {
     const int hl = dev::fastDiv(i, magicW4), b = i - hl * W4;
     const int a = ST == 1 ? hl : hl / ST, dy = hl - a * ST;
@@ -695,7 +695,7 @@ poolBwdStrip(const float *__restrict__ gradOut, const long *__restrict__ indices
           }
         }
     }
-    dev::storeStream4(o + (long)i * 4, make_float4(acc[0], acc[1], acc[2], acc[3]));
+    dev::bufStoreStream4(orr, i * 16, make_float4(acc[0], acc[1], acc[2], acc[3]));
   }
 }
 

@@ -22,7 +22,7 @@
 #pragma once
 
 struct PwArgs {
-  const float *w;     // (M x K) row-major, 16-byte aligned
+  const float *w;     // (M x K) row-major, 16-byte aligned; TRANS kernels: (K x M) row-major, read as its transpose
   const float *x;     // (N, K, L), 16-byte aligned, L % 4 == 0
   float *out;         // (N, M, L), 16-byte aligned
   const float *bias;  // M or null
@@ -32,6 +32,13 @@ struct PwArgs {
   unsigned magicL;    // dev::magicOf(L)
   int xBytes, outBytes;  // < 2^31
 };
+
+// LDS floats of a workgroup: the two chunk buffers, or the slab of weights that passes through them first
+constexpr int pwLdsFloats(int K, int MR, int WR, int CT) {
+  const int ksl = K < 128 ? K : 128, rows = 32 * MR * WR;
+  const int chunks = 2 * K * 32 * CT, slab = rows * (ksl + 4), slabT = ksl * (rows + 4);
+  return chunks > slab ? (chunks > slabT ? chunks : slabT) : (slab > slabT ? slab : slabT);
+}
 
 // What a job (the MFMAs of JP column tiles x MR row tiles) leaves behind: its accumulators and, per tile and
 // group of 8 rows, the lane's byte offset into out (position part; the row part is a scalar offset), out of
@@ -47,8 +54,9 @@ struct PwDone {
 // NW = 8 is one workgroup per CU, two waves per SIMD that take turns on the matrix pipe and meet at every chunk's
 // barrier: they advance together. (Two independent workgroups of 4 waves per CU do not - the SIMD favours the
 // older wave, one workgroup of each pair finishes at 60 % of the time and the other runs the rest alone.)
-// RELU: the stored value is v > 0 ? v : 0.
-template <int K, int MR, int WR, int CT, int NW, bool RELU = false>
+// RELU: the stored value is v > 0 ? v : 0. TRANS: the weights are given as (K x M) and used as their transpose -
+// the gradInput pass of a 1x1 convolution (gradInput = W^T gradOutput) reads the layer's own weight tensor.
+template <int K, int MR, int WR, int CT, int NW, bool RELU = false, bool TRANS = false>
 __global__ void __launch_bounds__(64 * NW, 2)
 convPointwiseKernel(PwArgs p) {
   constexpr int BLK = 64 * NW;
@@ -114,30 +122,54 @@ convPointwiseKernel(PwArgs p) {
     constexpr int WP = KSL + 4;              // LDS row pitch in floats
     constexpr int C4 = KSL / 4;              // 16-byte groups per row of a slab
     constexpr int NW4 = ROWS * C4;           // 16-byte groups of a slab
-    static_assert(ROWS * WP <= 2 * K * CP, "the slab fits the chunk buffers");
+    static_assert(ROWS * WP <= pwLdsFloats(K, MR, WR, CT), "the slab fits the LDS the host asks for");
     const int rowW0 = (int)blockIdx.y * ROWS;
 #pragma unroll
     for (int slab = 0; slab < K / KSL; ++slab) {
       if (slab > 0) __syncthreads();  // the previous slab has been read
+      if constexpr (!TRANS) {
 #pragma unroll
-      for (int u = 0; u < (NW4 + BLK - 1) / BLK; ++u) {
-        const int i = u * BLK + t;
-        if (i < NW4) {
-          const int row = i / C4, c4 = i - row * C4;
-          const int grow = min(rowW0 + row, p.M - 1);  // rows past M are computed from row M - 1 and never stored
-          *reinterpret_cast<float4 *>(Bs + row * WP + c4 * 4) =
-              *reinterpret_cast<const float4 *>(p.w + (long)grow * K + slab * KSL + c4 * 4);
+        for (int u = 0; u < (NW4 + BLK - 1) / BLK; ++u) {
+          const int i = u * BLK + t;
+          if (i < NW4) {
+            const int row = i / C4, c4 = i - row * C4;
+            const int grow = min(rowW0 + row, p.M - 1);  // rows past M are computed from row M - 1 and never stored
+            *reinterpret_cast<float4 *>(Bs + row * WP + c4 * 4) =
+                *reinterpret_cast<const float4 *>(p.w + (long)grow * K + slab * KSL + c4 * 4);
+          }
         }
-      }
-      __syncthreads();
+        __syncthreads();
 #pragma unroll
-      for (int r = 0; r < MR; ++r) {
-        const float *wrow = Bs + (wr * (32 * MR) + 32 * r + idx) * WP;
+        for (int r = 0; r < MR; ++r) {
+          const float *wrow = Bs + (wr * (32 * MR) + 32 * r + idx) * WP;
 #pragma unroll
-        for (int j = 0; j < C4; ++j) {
-          const float4 q = *reinterpret_cast<const float4 *>(wrow + 4 * j);
-          a[r][slab * (KSL / 2) + 2 * j] = grp ? q.y : q.x;
-          a[r][slab * (KSL / 2) + 2 * j + 1] = grp ? q.w : q.z;
+          for (int j = 0; j < C4; ++j) {
+            const float4 q = *reinterpret_cast<const float4 *>(wrow + 4 * j);
+            a[r][slab * (KSL / 2) + 2 * j] = grp ? q.y : q.x;
+            a[r][slab * (KSL / 2) + 2 * j + 1] = grp ? q.w : q.z;
+          }
+        }
+      } else {
+        // the slab as memory holds it: KSL rows (k) of the workgroup's ROWS consecutive columns (m), coalesced along
+        // m; a lane then picks its operands column-wise (consecutive lanes read consecutive floats)
+        constexpr int WPT = ROWS + 4, R4 = ROWS / 4, NT4 = KSL * R4;
+        static_assert(KSL * WPT <= pwLdsFloats(K, MR, WR, CT), "the transposed slab fits the LDS the host asks for");
+#pragma unroll
+        for (int u = 0; u < (NT4 + BLK - 1) / BLK; ++u) {
+          const int i = u * BLK + t;
+          if (i < NT4) {
+            const int k = i / R4, j4 = i - k * R4;
+            const int m = min(rowW0 + 4 * j4, p.M - 4);  // M % 8 == 0; columns past M repeat the last ones, never stored
+            *reinterpret_cast<float4 *>(Bs + k * WPT + 4 * j4) =
+                *reinterpret_cast<const float4 *>(p.w + (long)(slab * KSL + k) * p.M + m);
+          }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+          const float *wcol = Bs + grp * WPT + (wr * (32 * MR) + 32 * r + idx);
+#pragma unroll
+          for (int j = 0; j < KSL / 2; ++j) a[r][slab * (KSL / 2) + j] = wcol[2 * j * WPT];
         }
       }
     }

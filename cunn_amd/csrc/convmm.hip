@@ -1893,10 +1893,10 @@ bool pwShape(int M, int K, PwShape *sh) {
   return true;
 }
 
-template <int K, int MR, int WR, int CT, int NW, bool RELU>
+template <int K, int MR, int WR, int CT, int NW, bool RELU, bool TRANS>
 void launchPointwiseShape(hipStream_t s, PwArgs p, int device) {
-  constexpr size_t lds = 2 * (size_t)K * 32 * CT * sizeof(float);
-  auto kernel = convPointwiseKernel<K, MR, WR, CT, NW, RELU>;
+  constexpr size_t lds = (size_t)pwLdsFloats(K, MR, WR, CT) * sizeof(float);
+  auto kernel = convPointwiseKernel<K, MR, WR, CT, NW, RELU, TRANS>;
   if (lds > 64 * 1024) {  // once per kernel instance and device: allow more than 64 KB of dynamic LDS
     static std::atomic<bool> raised[64];
     if (!raised[device].load()) {
@@ -1915,14 +1915,24 @@ void launchPointwiseShape(hipStream_t s, PwArgs p, int device) {
   THC_HIP_CHECK(hipGetLastError());
 }
 
-// out(N, M, L) = bias + W(M x K) x(N, K, L) on the weight-stationary kernel; false: the shape is not one of its
+// out(N, M, L) = bias + W(M x K) x(N, K, L) on the weight-stationary kernel; false: the shape is not one of its.
+// transW: w holds (K x M) and its transpose is what multiplies (the gradInput pass hands over the layer's weights).
 bool convPointwise(THCState *state, const ConvGeom &g, const float *x, const float *w, const float *bias, float *out,
-                   bool relu = false) {
+                   bool relu = false, bool transW = false) {
   if (forceGeneric() || g_switches.convPointwise == 0) return false;
   if (g.kH != 1 || g.kW != 1 || g.dH != 1 || g.dW != 1 || g.padH != 0 || g.padW != 0) return false;
   const long P = (long)g.N * g.L;
   PwShape sh;
   if (g.L % 4 != 0 || g.Cout % 8 != 0 || P < 32 || !pwShape(g.Cout, g.K, &sh)) return false;
+  // Short runs: with fewer than three chunks per workgroup the pipeline (chunk c multiplied, c + 1 in registers,
+  // c + 2 in flight) never fills; chunks of half the size do better there (128 -> 128 at 28 x 28, N = 64, 7 column
+  // tiles per workgroup: 28.2 -> 24.7 us, the tiled GEMM 25.8; at 56 x 56, 25 tiles per workgroup: 70 -> 76 us).
+  if (g.K == 128 && sh.wr == 4) {
+    const int rowBlocks = launch::ceilDiv(g.Cout, 32 * sh.mr * sh.wr);
+    const int slots = std::max(1, residentSlots(nullptr) / rowBlocks);
+    const long perWg = (((P + 31) / 32) + slots - 1) / slots;
+    if (perWg < 5 * sh.ct) sh.ct = 2;
+  }
   if (!launch::aligned16(x) || !launch::aligned16(w) || !launch::aligned16(out)) return false;
   // 32-bit byte offsets into x and out; the reciprocal division of a position by L is exact while P * L < 2^32
   if (P * g.K * 4 >= 0x7fffffffL || P * g.Cout * 4 >= 0x7fffffffL || P * g.L >= 0xffffffffL) return false;
@@ -1938,15 +1948,17 @@ bool convPointwise(THCState *state, const ConvGeom &g, const float *x, const flo
   hipStream_t s = state->stream;
 #define PW_CASE(KK, MRR, WRR, CTT, NWW)                                              \
   if (g.K == KK && sh.mr == MRR && sh.wr == WRR && sh.ct == CTT && sh.nw == NWW) {   \
-    if (relu)                                                                        \
-      launchPointwiseShape<KK, MRR, WRR, CTT, NWW, true>(s, p, device);              \
+    if (transW)                                                                      \
+      launchPointwiseShape<KK, MRR, WRR, CTT, NWW, false, true>(s, p, device);       \
+    else if (relu)                                                                   \
+      launchPointwiseShape<KK, MRR, WRR, CTT, NWW, true, false>(s, p, device);       \
     else                                                                             \
-      launchPointwiseShape<KK, MRR, WRR, CTT, NWW, false>(s, p, device);             \
+      launchPointwiseShape<KK, MRR, WRR, CTT, NWW, false, false>(s, p, device);      \
     return true;                                                                     \
   }
   PW_CASE(32, 2, 4, 16, 8) PW_CASE(32, 1, 4, 16, 8) PW_CASE(32, 1, 2, 16, 8)
   PW_CASE(64, 2, 4, 8, 8) PW_CASE(64, 1, 4, 8, 8) PW_CASE(64, 1, 2, 8, 8)
-  PW_CASE(128, 1, 4, 4, 8) PW_CASE(128, 1, 2, 4, 8)
+  PW_CASE(128, 1, 4, 4, 8) PW_CASE(128, 1, 2, 4, 8) PW_CASE(128, 1, 4, 2, 8)
 #undef PW_CASE
   return false;
 }
@@ -2325,13 +2337,14 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
     FwdPlan pl = planFwdImplicit(t.Cout, std::min(group, g.N), t);
     long need = pl.scratchFloats;
     if (g.N % group != 0) need = std::max(need, planFwdImplicit(t.Cout, g.N % group, t).scratchFloats);
+    // 1x1: gradInput = W^T gradOutput, a pointwise pass itself, which reads the weights as they are
+    if (convPointwise(state, t, gy, w, bias, gi, false, true)) return;
     const long wfFloats = ((long)g.Cout * g.K + 3) / 4 * 4;
     Temp tmp;
     float *buf = scratchFloats(state, scratchBuf, wfFloats + need, tmp, bufName);
     flipWeightKernel<<<launch::directGrid((long)g.Cout * g.K, dev::kBlock), dev::kBlock, 0, s>>>(w, buf, g.Cout, g.Cin,
                                                                                                 g.kH, g.kW);
     THC_HIP_CHECK(hipGetLastError());
-    if (convPointwise(state, t, gy, buf, bias, gi)) return;  // 1x1: gradInput = W^T gradOutput, a pointwise pass itself
     for (int n0 = 0; n0 < g.N; n0 += group) {
       int cnt = std::min(group, g.N - n0);
       if (cnt != std::min(group, g.N)) pl = planFwdImplicit(t.Cout, cnt, t);

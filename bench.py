@@ -732,8 +732,10 @@ def copy_ceiling(hip, stream):
                 copy_bytes_per_launch=nbytes, copy_launches=COPY_LAUNCHES)
 
 
-def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=False, cold_sets=COLD_SETS):
+def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=False, cold_sets=COLD_SETS, order="step"):
     ncold = cold_sets if nsets > 1 and name != "copy" else nsets
+    if order == "cold":                  # every pass in the cache-cold ordering (for profiles of that ordering)
+        ncold = max(ncold, 2)
     wl = WORKLOADS[name](max(nsets, ncold))
     wl["verify"]()                       # parity against the oracle in this very run
     names = [n for n, _ in wl["calls"](0)]
@@ -742,7 +744,7 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=F
     stride = max(1, ncold // len(names))
     cursor = [0]                         # buffer sets keep rotating across the phases below
 
-    def run(nsteps, bracket, cold=False, empty=False):
+    def run(nsteps, bracket, cold=(order == "cold"), empty=False):
         """nsteps steps back to back; HIP events around the entry points named in `bracket`; with `empty`, one more
         event pair with nothing between them at the end of every step (what a bracket costs by itself)."""
         ev = {n: [(hip.event(), hip.event()) for _ in range(nsteps)] for n in bracket}
@@ -828,7 +830,7 @@ def run_workload(name, steps, warmup, hip, stream, nsets, cpu_seconds, ceiling=F
                     ms_per_step_bracketed=round(wall_ev * 1e3 / steps, 5),
                     empty_bracket_ms=round(float(np.median(emp[None])), 5))
     extra = PREROLL_SAMPLES
-    if ncold > len(names):
+    if ncold > len(names) and order != "cold":
         # cache-cold variant, outside the timed steps: the same entry points, each on a buffer set that nothing has
         # touched for at least `stride` - 1 whole steps (more than 1 GB of traffic at cfg2)
         run(ncold, [], cold=True)
@@ -870,6 +872,8 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time the other four configurations")
     ap.add_argument("--sets", type=int, default=4, help="buffer sets rotated between steps (1 = cache-warm variant)")
     ap.add_argument("--cold-sets", type=int, default=COLD_SETS, help="buffer sets of the cache-cold ordering (0 = skip it)")
+    ap.add_argument("--order", default="step", choices=["step", "cold"],
+                    help="cold: the timed steps themselves run in the cache-cold ordering (config.order says so)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU time budget of the oracle baseline (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -885,12 +889,13 @@ def main():
     hip = Hip()
 
     main_res = run_workload(args.workload, args.steps, args.warmup, hip, stream, args.sets, args.cpu_seconds, ceiling=True,
-                            cold_sets=args.cold_sets)
+                            cold_sets=args.cold_sets, order=args.order)
     out = {
         "metric": METRIC, "value": round(main_res["images_per_s"], 1), "unit": "images/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(main_res["ms_per_step"], 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {main_res['workload']}", "buffer_sets": args.sets,
+        "config": {"workload": f"{args.workload}: {main_res['workload']}", "buffer_sets": args.sets if args.order == "step" else args.cold_sets,
+                   "order": "every entry point of a step on the same buffer set" if args.order == "step" else "cache-cold: entry points of a step on different buffer sets",
                    "entry": "C ABI libTHCUNN.so (THNN_Cuda*) via ctypes"},
         "device_ms_per_step": round(main_res["device_ms_per_step"], 5),
         "preroll_steps": main_res["preroll_steps"],

@@ -1028,6 +1028,13 @@ convFwdPaddedBatchKernel(FwdBatch b) {
   fwdPaddedBody<WM>(it.p, it.g, blockIdx.x, blockIdx.y, it.p.nSplit <= 1);
 }
 
+// 16-byte load of data that is read exactly once (non-temporal hint: it does not displace what the caches hold)
+__device__ __forceinline__ float4 loadOnce4(const float4 *p) {
+  typedef float f32x4v __attribute__((ext_vector_type(4)));
+  const f32x4v v = __builtin_nontemporal_load(reinterpret_cast<const f32x4v *>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+
 // out tile = bias + sum over the nSplit partial tiles (ascending split order).
 // grid = (tail tiles, BM*BN / 1024): a workgroup folds 1024 consecutive tile elements, 4 per lane.
 __device__ __forceinline__ void fwdTailFixupBody(const FwdArgs &p, const ConvGeom &g) {
@@ -1043,7 +1050,7 @@ __device__ __forceinline__ void fwdTailFixupBody(const FwdArgs &p, const ConvGeo
     constexpr int NQ = decltype(nc)::value;
     float4 q[NQ];
 #pragma unroll
-    for (int i = 0; i < NQ; ++i) q[i] = *reinterpret_cast<const float4 *>(src + (long)(sp + i) * (BM * BN) + e);
+    for (int i = 0; i < NQ; ++i) q[i] = loadOnce4(reinterpret_cast<const float4 *>(src + (long)(sp + i) * (BM * BN) + e));
 #pragma unroll
     for (int i = 0; i < NQ; ++i) v.x += q[i].x, v.y += q[i].y, v.z += q[i].z, v.w += q[i].w;
     sp += NQ;
@@ -1403,12 +1410,12 @@ foldPartials4Kernel(const float *__restrict__ partial, float *__restrict__ dst, 
     for (; s + 3 * G < splits; s += 4 * G) {
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const float4 v = p[(long)(s + G * u) * count4];
+        const float4 v = loadOnce4(p + (long)(s + G * u) * count4);  // the partials' only reader
         a[u].x += v.x, a[u].y += v.y, a[u].z += v.z, a[u].w += v.w;
       }
     }
     for (; s < splits; s += G) {
-      const float4 v = p[(long)s * count4];
+      const float4 v = loadOnce4(p + (long)s * count4);
       a[0].x += v.x, a[0].y += v.y, a[0].z += v.z, a[0].w += v.w;
     }
   }

@@ -515,6 +515,27 @@ padRowsKernel(const float *__restrict__ w, float *__restrict__ wp, int rows, int
   }
 }
 
+// Wf[c][(o, kh', kw')] = W[o][(c, kH-1-kh', kW-1-kw')]: with these weights the stride-1 gradInput is a plain forward
+// convolution of gradOutput (padding k-1-pad). The job rides along with the bordered copy of gradOutput (a few more
+// workgroups of that launch) instead of costing a launch of its own: both are short, and their latencies would add.
+__global__ void flipWeightKernel(const float *__restrict__ w, float *__restrict__ wf, int Cout, int Cin, int kH, int kW);
+struct FlipJob {
+  const float *w;
+  float *wf;
+  int Cout, Cin, kH, kW;
+};
+constexpr int kFlipBlocks = 4096;  // a lane per element up to a million weights: a lane that walks several is bound by their latencies
+__device__ __forceinline__ void flipWeights(const FlipJob &f, int block, int blocks) {
+  const int KK = f.kH * f.kW;
+  const long total = (long)f.Cout * f.Cin * KK;
+  for (long i = (long)block * dev::kBlock + threadIdx.x; i < total; i += (long)blocks * dev::kBlock) {
+    const int t = (int)(i % KK);
+    const long r = i / KK;
+    const int o = (int)(r % f.Cout), c = (int)(r / f.Cout);
+    f.wf[i] = f.w[((long)o * f.Cin + c) * KK + (KK - 1 - t)];
+  }
+}
+
 // xp(nc, Hp, Wp) = x(nc, H, W) at row padTop, column padLeft inside zeros. grid = (planes, chunks of a plane);
 // VEC: a lane produces 4 consecutive floats of the bordered plane with one 16-byte store
 // (plane size a multiple of 4 floats, 16-byte aligned destination).
@@ -550,9 +571,13 @@ padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int 
 template <bool ANY>
 __global__ void __launch_bounds__(dev::kBlock)
 padPlanesFlatKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int padTop, int padLeft, int Hp, int Wp,
-                    long total4, int copyBlocks, int *taps, int tapEntries, ConvGeom tg) {
+                    long total4, int copyBlocks, int *taps, int tapEntries, ConvGeom tg, int tapBlocks, FlipJob flip) {
+  if ((int)blockIdx.x >= copyBlocks + tapBlocks) {  // the weights of the convolution that follows, flipped
+    flipWeights(flip, blockIdx.x - copyBlocks - tapBlocks, gridDim.x - copyBlocks - tapBlocks);
+    return;
+  }
   if ((int)blockIdx.x >= copyBlocks) {
-    for (int k = (blockIdx.x - copyBlocks) * dev::kBlock + threadIdx.x; k < tapEntries; k += (gridDim.x - copyBlocks) * dev::kBlock)
+    for (int k = (blockIdx.x - copyBlocks) * dev::kBlock + threadIdx.x; k < tapEntries; k += tapBlocks * dev::kBlock)
       taps[k] = tapOffset(k, tg);
     return;
   }
@@ -594,9 +619,17 @@ padPlanesFlatKernel(const float *__restrict__ x, float *__restrict__ xp, int H, 
 }
 
 // taps != nullptr: the same launch also builds the tap table (tapEntries entries) of geometry tg
+// flip != nullptr: and flips the weights of *flip (the flat kernels take the job along; otherwise a launch of its own)
 void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int H, int W, int padTop, int padLeft, int Hp,
-                     int Wp, int *taps = nullptr, int tapEntries = 0, const ConvGeom *tg = nullptr) {
+                     int Wp, int *taps = nullptr, int tapEntries = 0, const ConvGeom *tg = nullptr, const FlipJob *flip = nullptr) {
   const int plane = Hp * Wp;
+  const FlipJob fj = flip ? *flip : FlipJob{};
+  const int flipBlocks = flip ? (int)std::min<long>(kFlipBlocks, ((long)fj.Cout * fj.Cin * fj.kH * fj.kW + dev::kBlock - 1) / dev::kBlock) : 0;
+  auto flipAlone = [&]() {
+    if (!flip) return;
+    flipWeightKernel<<<launch::directGrid((long)fj.Cout * fj.Cin * fj.kH * fj.kW, dev::kBlock), dev::kBlock, 0, s>>>(
+        fj.w, fj.wf, fj.Cout, fj.Cin, fj.kH, fj.kW);
+  };
   if (launch::ceilDiv(plane, dev::kBlock) > 65535) error("SpatialConvolutionMM: image plane too large");
   const unsigned gx = (unsigned)planes + (taps ? 1 : 0);
   const ConvGeom g = tg ? *tg : ConvGeom{};
@@ -605,26 +638,29 @@ void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int 
   if (plane % 4 == 0 && plane < 4096 && launch::aligned16(xp) && total4 * (plane / 4) < 0xffffffffL) {
     const int copyBlocks = (int)std::min<long>((total4 + dev::kBlock - 1) / dev::kBlock, 16384);
     const int tapBlocks = taps ? std::max(1, std::min(16, launch::ceilDiv(tapEntries, dev::kBlock))) : 0;
-    padPlanesFlatKernel<false><<<copyBlocks + tapBlocks, dev::kBlock, 0, s>>>(x, xp, H, W, padTop, padLeft, Hp, Wp, total4,
-                                                                             copyBlocks, taps, tapEntries, g);
+    padPlanesFlatKernel<false><<<copyBlocks + tapBlocks + flipBlocks, dev::kBlock, 0, s>>>(
+        x, xp, H, W, padTop, padLeft, Hp, Wp, total4, copyBlocks, taps, tapEntries, g, tapBlocks, fj);
   } else if (plane < 1024 && launch::aligned16(xp) && planes * plane * (long)plane < 0xffffffffL) {
     // small planes of any size (a bordered 7x7 or 13x13 plane): a workgroup per plane would leave most of its lanes idle
     const long total = planes * plane;
     const int copyBlocks = (int)std::min<long>(((total + 3) / 4 + dev::kBlock - 1) / dev::kBlock, 16384);
     const int tapBlocks = taps ? std::max(1, std::min(16, launch::ceilDiv(tapEntries, dev::kBlock))) : 0;
-    padPlanesFlatKernel<true><<<copyBlocks + tapBlocks, dev::kBlock, 0, s>>>(x, xp, H, W, padTop, padLeft, Hp, Wp, total,
-                                                                            copyBlocks, taps, tapEntries, g);
-  } else if (plane % 4 == 0 && launch::aligned16(xp))
+    padPlanesFlatKernel<true><<<copyBlocks + tapBlocks + flipBlocks, dev::kBlock, 0, s>>>(
+        x, xp, H, W, padTop, padLeft, Hp, Wp, total, copyBlocks, taps, tapEntries, g, tapBlocks, fj);
+  } else if (plane % 4 == 0 && launch::aligned16(xp)) {
+    flipAlone();
     padPlanesKernel<true><<<dim3(gx, launch::ceilDiv(plane / 4, dev::kBlock)), dev::kBlock, 0, s>>>(
         x, xp, H, W, padTop, padLeft, Hp, Wp, (int)planes, taps, tapEntries, g);
-  else
+  } else {
+    flipAlone();
     padPlanesKernel<false><<<dim3(gx, launch::ceilDiv(plane, dev::kBlock)), dev::kBlock, 0, s>>>(
         x, xp, H, W, padTop, padLeft, Hp, Wp, (int)planes, taps, tapEntries, g);
+  }
   THC_HIP_CHECK(hipGetLastError());
 }
 inline void launchPadPlanes(hipStream_t s, const float *x, float *xp, long planes, int H, int W, int padH, int padW,
-                            int *taps = nullptr, int tapEntries = 0, const ConvGeom *tg = nullptr) {
-  launchPadPlanes(s, x, xp, planes, H, W, padH, padW, H + 2 * padH, W + 2 * padW, taps, tapEntries, tg);
+                            int *taps = nullptr, int tapEntries = 0, const ConvGeom *tg = nullptr, const FlipJob *flip = nullptr) {
+  launchPadPlanes(s, x, xp, planes, H, W, padH, padW, H + 2 * padH, W + 2 * padW, taps, tapEntries, tg, flip);
 }
 
 // ---- gradInput by output phase ------------------------------------------------------------------
@@ -1806,8 +1842,14 @@ struct OutMap {
 
 void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const float *w, const float *x, float *out,
                        const float *bias, int M, int nImages, const ConvGeom &g, bool relu = false,
-                       const OutMap *om = nullptr) {
+                       const OutMap *om = nullptr, const FlipJob *flip = nullptr) {
   const bool fast = pl.tapEntries > 0;
+  if (flip && !(fast && pl.paddedFloats > 0)) {  // no bordered copy to ride along with
+    flipWeightKernel<<<launch::directGrid((long)flip->Cout * flip->Cin * flip->kH * flip->kW, dev::kBlock), dev::kBlock, 0, s>>>(
+        flip->w, flip->wf, flip->Cout, flip->Cin, flip->kH, flip->kW);
+    THC_HIP_CHECK(hipGetLastError());
+    flip = nullptr;
+  }
   if (fast && !(launch::aligned16(scratch) && (pl.weightFloats > 0 || launch::aligned16(w))))
     error("SpatialConvolutionMM: internal error, convolution scratch or weights not 16-byte aligned");
   float *partial = scratch + pl.tapEntries;
@@ -1821,7 +1863,7 @@ void launchFwdImplicit(hipStream_t s, const FwdPlan &pl, float *scratch, const f
     const bool linear = g.kH == 1 && g.kW == 1 && g.K % BK == 0;
     if (pl.paddedFloats > 0) {  // the copy into the bordered layout builds the tap table on the side
       launchPadPlanes(s, x, xp, (long)nImages * g.Cin, g.H, g.W, g.padH, g.padW, linear ? nullptr : reinterpret_cast<int *>(scratch),
-                      pl.tapEntries, &gk);
+                      pl.tapEntries, &gk, flip);
       p.x = xp;
     }
     if (linear) {
@@ -2349,14 +2391,12 @@ void convGradInput(THCState *state, const ConvGeom &g, const float *gy, const fl
     const long wfFloats = ((long)g.Cout * g.K + 3) / 4 * 4;
     Temp tmp;
     float *buf = scratchFloats(state, scratchBuf, wfFloats + need, tmp, bufName);
-    flipWeightKernel<<<launch::directGrid((long)g.Cout * g.K, dev::kBlock), dev::kBlock, 0, s>>>(w, buf, g.Cout, g.Cin,
-                                                                                                g.kH, g.kW);
-    THC_HIP_CHECK(hipGetLastError());
+    const FlipJob flip{w, buf, g.Cout, g.Cin, g.kH, g.kW};  // done by the first group's bordered copy, or by a launch of its own
     for (int n0 = 0; n0 < g.N; n0 += group) {
       int cnt = std::min(group, g.N - n0);
       if (cnt != std::min(group, g.N)) pl = planFwdImplicit(t.Cout, cnt, t);
       launchFwdImplicit(s, pl, buf + wfFloats, buf, gy + (long)n0 * g.Cout * g.L, gi + (long)n0 * g.Cin * g.H * g.W,
-                        bias, t.Cout, cnt, t);
+                        bias, t.Cout, cnt, t, false, nullptr, n0 == 0 ? &flip : nullptr);
     }
     return;
   }

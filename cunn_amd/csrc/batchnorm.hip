@@ -408,9 +408,14 @@ __device__ __forceinline__ float blockSum1024(float v, float *red) {
 // host checks that the tensor is smaller than 2 GiB).
 struct ResWalker {
   int off, l4, stepOff, stepL, L4, wrapOff;
-  __device__ ResWalker(int L, int C) : L4(L >> 2) {
-    const int n = threadIdx.x / L4;
-    l4 = threadIdx.x - n * L4;
+  // fresh: the walk is derived again from a lane index the compiler cannot relate to an earlier walk, so
+  // that it recomputes the offsets (one add and a compare per step) instead of keeping one register per
+  // step of the earlier walk alive.
+  __device__ ResWalker(int L, int C, bool fresh = false) : L4(L >> 2) {
+    int tid = threadIdx.x;
+    if (fresh) __asm__ volatile("" : "+v"(tid));
+    const int n = tid / L4;
+    l4 = tid - n * L4;
     const int stepN = kResBlock / L4;
     stepL = kResBlock - stepN * L4;
     off = (n * C * L + (l4 << 2)) * 4;
@@ -488,17 +493,20 @@ bnFwdResident(const float *__restrict__ x, float *__restrict__ y, const float *_
 }
 
 // Backward with gradOutput resident in registers. KEEPX: (x - mean) stays in
-// registers as well (2R float4 per lane); otherwise x is read a second time in
-// the apply phase - it was streamed by this CU a moment ago, so the re-read is
-// served by the L2 / Infinity Cache rather than HBM.
-template <int R, bool TRAIN, bool KEEPX>
+// registers as well (2R float4 per lane). Otherwise x is consumed in batches; XL > 0: the first XL float4
+// of x per lane wait in LDS for the apply phase and the other R - XL in registers, so that x crosses HBM
+// once as well; XL == 0: nothing of x is kept (no apply phase, or one that does not need x).
+template <int R, bool TRAIN, bool KEEPX, int XL = 0>
 __global__ void __launch_bounds__(kResBlock)
 bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
               float *__restrict__ gradWeight, float *__restrict__ gradBias, const float *__restrict__ weight,
               const float *__restrict__ meanSrc, const float *__restrict__ stdSrc, int N, int C, int L, float scale,
-              float eps, int xlds, ReluMask rm) {
+              float eps, ReluMask rm) {
   __shared__ float red[kResWaves];
-  extern __shared__ float4 xpark[];  // !KEEPX: the first xlds (a multiple of 4) float4 of x per lane wait here for the apply phase
+  extern __shared__ float4 xpark[];  // XL float4 of x per lane
+  constexpr int XK = XL > 0 ? R - XL : 0;
+  static_assert(!KEEPX || XL == 0, "either everything of x in registers or the split");
+  float4 xk[XK > 0 ? XK : 1];
   const int ch = blockIdx.x;
   const int total4 = N * (L >> 2);
   const float mean = meanSrc[ch];
@@ -508,7 +516,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
   const long span = ((long)(N - 1) * C * L + L) * 4;
   const __amdgpu_buffer_rsrc_t xr = dev::makeRsrc(x + (long)ch * L, span), gr = dev::makeRsrc(gy + (long)ch * L, span);
   const __amdgpu_buffer_rsrc_t or_ = dev::makeRsrc(gx ? gx + (long)ch * L : x, gx ? span : 0);
-  constexpr int XB = R > 8 ? 8 : 4;  // x float4 per lane requested together when x is not kept in registers
+  constexpr int XB = (R > 8 && XL == 0) ? 8 : 4;  // x float4 per lane requested together when x is not kept in registers
   float4 d[R], xc[KEEPX ? R : 1];
   float s0 = 0.f, s1 = 0.f;
   {
@@ -553,11 +561,14 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
             wx.next();
           }
         }
-        if (u0 < xlds) {
 #pragma unroll
-          for (int k = 0; k < XB; ++k)
-            if (u0 + k < R) xpark[(u0 + k) * kResBlock + threadIdx.x] = q[k];
-        }
+        for (int k = 0; k < XB; ++k)
+          if (u0 + k < R) {
+            if (u0 + k < XL)
+              xpark[(u0 + k) * kResBlock + threadIdx.x] = q[k];
+            else if (XL > 0)
+              xk[XK > 0 ? u0 + k - XL : 0] = q[k];
+          }
 #pragma unroll
         for (int k = 0; k < XB; ++k)
           if (u0 + k < R) {
@@ -577,7 +588,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
   const float projScale = dotP * norm * stdVal * stdVal;
   const float gradScale = stdVal * weightVal;
   if (gx) {
-    ResWalker wk(L, C);
+    ResWalker wk(L, C, XL > 0);
     if (KEEPX || !TRAIN) {
 #pragma unroll
       for (int u = 0; u < R; ++u) {
@@ -608,7 +619,12 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
           if (u0 + k < R) {
             if ((u0 + k) * kResBlock + (int)threadIdx.x < total4) {
               off[k] = wk.offset();
-              q[k] = u0 < xlds ? xpark[(u0 + k) * kResBlock + threadIdx.x] : dev::bufLoad4(xr, off[k]);
+              if (XL == 0)
+                q[k] = dev::bufLoad4(xr, off[k]);
+              else if (u0 + k < XL)
+                q[k] = xpark[(u0 + k) * kResBlock + threadIdx.x];
+              else
+                q[k] = xk[XK > 0 ? u0 + k - XL : 0];
             }
             wk.next();
           }
@@ -968,25 +984,31 @@ void bnBackward(THCState *state, THCudaTensor *input_, THCudaTensor *gradOutput_
     float *gxp = gradInput_ ? data(gradInput_) : nullptr;
 #define BN_BWD_RES(RR)                                                                                             \
   if (R == RR) {                                                                                                   \
-    /* x parked in LDS between the two phases: 8 of the up to 13 float4 per lane (128 KB of the CU's 160 KB) */   \
-    const int xlds = (RR > 8 && train && gxp) ? 8 : 0;                                                             \
-    const size_t lds = (size_t)xlds * kResBlock * sizeof(float4);                                                  \
-    if (train) {                                                                                                   \
+    /* x between the two phases: 9 of the up to 13 float4 per lane in LDS (144 KB of the CU's 160 KB), the rest   \
+       in registers */                                                                                             \
+    constexpr int XL = RR > 8 ? 9 : 0;                                                                             \
+    constexpr size_t lds = (size_t)XL * kResBlock * sizeof(float4);                                                \
+    if (train && gxp && XL > 0) {                                                                                  \
       /* once per kernel instance and device: allow more than 64 KB of dynamic LDS */                             \
       static std::atomic<bool> ldsRaised[kMaxDevices];                                                             \
       const int dv = currentDevice();                                                                              \
-      if (lds && !ldsRaised[dv].load()) {                                                                          \
-        THC_HIP_CHECK(hipFuncSetAttribute((const void *)bnBwdResident<RR, true, (RR <= 8)>,                        \
+      if (!ldsRaised[dv].load()) {                                                                                 \
+        THC_HIP_CHECK(hipFuncSetAttribute((const void *)bnBwdResident<RR, true, false, XL>,                        \
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                  \
         ldsRaised[dv].store(true);                                                                                 \
       }                                                                                                            \
-      bnBwdResident<RR, true, (RR <= 8)><<<g.C, kResBlock, lds, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_), \
+      bnBwdResident<RR, true, false, XL><<<g.C, kResBlock, lds, s>>>(in.ptr(), go.ptr(), gxp,                      \
+                                                        dataOrNull(gradWeight_), dataOrNull(gradBias_),            \
+                                                        dataOrNull(weight_), meanSrc, stdSrc, g.N, g.C, g.L,       \
+                                                        (float)scale, (float)eps, rm);                             \
+    } else if (train) {                                                                                            \
+      bnBwdResident<RR, true, (RR <= 8)><<<g.C, kResBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_), \
                                                         dataOrNull(gradBias_), dataOrNull(weight_), meanSrc,       \
-                                                        stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, xlds, rm); \
+                                                        stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, rm);      \
     } else {                                                                                                       \
       bnBwdResident<RR, false, (RR <= 8)><<<g.C, kResBlock, 0, s>>>(in.ptr(), go.ptr(), gxp, dataOrNull(gradWeight_), \
                                                          dataOrNull(gradBias_), dataOrNull(weight_), meanSrc,      \
-                                                         stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, 0, rm);  \
+                                                         stdSrc, g.N, g.C, g.L, (float)scale, (float)eps, rm);     \
     }                                                                                                              \
   }
     BN_BWD_RES(2) BN_BWD_RES(4) BN_BWD_RES(8) BN_BWD_RES(12) BN_BWD_RES(13)

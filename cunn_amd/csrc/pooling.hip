@@ -588,19 +588,30 @@ avgPoolFwdFlat(const float *__restrict__ in, float *__restrict__ out, int oW4, u
                                                     acc[2] / (float)(KS * KS), acc[3] / (float)(KS * KS)));
 }
 
-// total = gradInput float4s; a lane writes float4 i of gradInput (memory order: a wave's store is one
-// contiguous run) from the up to 4 gradOutput values above it.
+// total = float4s of every KS-th gradInput row; a lane reads the up to 4 gradOutput values above float4 b of
+// the KS gradInput rows under one gradOutput row once and writes that float4 to each of the rows (a wave's
+// store is one contiguous run; KS stores in flight per lane, gradOutput crosses the memory system once).
 template <int KS>
 __global__ void __launch_bounds__(dev::kBlock)
 avgPoolBwdFlat(const float *__restrict__ gradOut, float *__restrict__ gradIn, int W4, unsigned magicW4, int oW, unsigned total) {
   const unsigned i = blockIdx.x * dev::kBlock + threadIdx.x;
   if (i >= total) return;
-  const unsigned R = dev::fastDiv((int)i, magicW4), b = i - R * W4;  // row of the tall gradInput image, float4 within it
-  const float *gp = gradOut + (size_t)(R / KS) * oW;
+  const unsigned R = dev::fastDiv((int)i, magicW4), b = i - R * W4;  // row of the tall gradOutput image, float4 within the rows under it
+  const float *gp = gradOut + (size_t)R * oW;
   float v[4];
+  if constexpr (KS == 2) {
+    typedef float f32x2v __attribute__((ext_vector_type(2)));
+    const f32x2v g2 = __builtin_nontemporal_load(reinterpret_cast<const f32x2v *>(gp) + b);
+    v[0] = v[1] = g2.x / 4.f, v[2] = v[3] = g2.y / 4.f;
+  } else if constexpr (KS == 4) {
+    v[0] = v[1] = v[2] = v[3] = __builtin_nontemporal_load(gp + b) / 16.f;
+  } else {
 #pragma unroll
-  for (int q = 0; q < 4; ++q) v[q] = gp[(b * 4 + q) / KS] / (float)(KS * KS);
-  dev::storeStream4(gradIn + (size_t)i * 4, make_float4(v[0], v[1], v[2], v[3]));
+    for (int q = 0; q < 4; ++q) v[q] = gp[(b * 4 + q) / KS] / (float)(KS * KS);
+  }
+  float *o = gradIn + ((size_t)R * KS * W4 + b) * 4;
+#pragma unroll
+  for (int k = 0; k < KS; ++k) dev::storeStream4(o + (size_t)k * W4 * 4, make_float4(v[0], v[1], v[2], v[3]));
 }
 
 // Backward gathers. MAX: gradOutput and the argmax (narrowed to int32, base
@@ -1303,7 +1314,7 @@ void THNN_CudaSpatialAveragePooling_updateGradInput(THCState *state, THCudaTenso
     avgPoolGlobalBwd<<<launch::directGrid(total, dev::kBlock), dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), total,
                                                                                     g.H * g.W, dev::magicOf(g.H * g.W));
   } else if (avgFlatOk(g, planes) && vec && aligned16(data(gradInput)) && planes * g.H * (g.W / 4) * (g.W / 4) < 0xffffffffL) {
-    const unsigned total = (unsigned)(planes * g.H * (g.W / 4));
+    const unsigned total = (unsigned)(planes * g.oH * (g.W / 4));
     const unsigned grid = (total + dev::kBlock - 1) / dev::kBlock;
     const unsigned magic = dev::magicOf(g.W / 4);
     if (g.kH == 2) avgPoolBwdFlat<2><<<grid, dev::kBlock, 0, s>>>(go.ptr(), data(gradInput), g.W / 4, magic, g.oW, total);

@@ -431,7 +431,12 @@ dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strid
   const int nIn = (nOut - 1) * ST + KS;
   const int pitch = S::pitch(g.W);
   typename S::InFlight fl;
-  if (ONE) S::issue(fl, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
+  // Stride 2 reads four bytes for every byte it writes, and its input is read with the non-temporal hint: after a
+  // kernel that has just written that input the pass measures 22 us with the hint and 23-28 us without
+  // (N 64, 128 x 56 x 56); only a caller that runs this pass again on an input still resident in the Infinity
+  // Cache, or the weight-gradient pass right behind it, would gain from plain loads. At stride 1 the two forms
+  // measure the same behind a producer, and plain loads keep a resident input resident.
+  if (ONE) S::template issue<(ST == 2)>(fl, in + (long)plane * g.H * g.W, g.H, g.W, oh0 * ST - PAD, nIn);
   float w[KS * KS];
   loadTaps<KS>(weight, ws, 0, c, w);
   float b = bias ? bias[c * bs.s1] : 0.f;

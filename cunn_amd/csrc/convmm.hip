@@ -1044,24 +1044,39 @@ convFwdPaddedKernel(FwdArgs p, ConvGeom g) {
   fwdPaddedBody<WM, LINEAR>(p, g, bx, by, whole);
 }
 
-// Several independent GEMMs of the same tile shape in one launch (the phases of a strided gradInput):
-// grid = (most tiles of an item, most splits of an item, items); workgroups beyond an item's own extent leave.
+// Several independent GEMMs of the same tile shape in one launch (the phases of a strided gradInput). An item's
+// first p.full tiles are reduced by one workgroup each, its other p.tail tiles by p.nSplit workgroups. One flat
+// grid: the whole tiles of all items in item order, then the splits of all items (split-major within an item) -
+// the splits fill the slots that the last whole tiles free.
 struct FwdBatchItem {
   FwdArgs p;
   ConvGeom g;
-  int tiles;  // p.mTiles * column tiles
+  int wholeEnd, splitEnd;  // running totals of p.full and of p.tail * p.nSplit up to and including this item
 };
 constexpr int kMaxBatch = 16;
 struct FwdBatch {
   FwdBatchItem item[kMaxBatch];
+  int count, wholeTotal;
 };
+static_assert(sizeof(FwdBatch) <= 4096, "kernel arguments are limited to 4 KB");
 
 template <int WM>
 __global__ void __launch_bounds__(dev::kBlock, 3)
 convFwdPaddedBatchKernel(FwdBatch b) {
-  const FwdBatchItem &it = b.item[blockIdx.z];
-  if ((int)blockIdx.x >= it.tiles || (int)blockIdx.y >= it.p.nSplit) return;
-  fwdPaddedBody<WM>(it.p, it.g, blockIdx.x, blockIdx.y, it.p.nSplit <= 1);
+  int bx = blockIdx.x, by = 0, i = 0;
+  const bool whole = bx < b.wholeTotal;
+  if (whole) {
+    while (i + 1 < b.count && bx >= b.item[i].wholeEnd) ++i;
+    bx -= i > 0 ? b.item[i - 1].wholeEnd : 0;
+  } else {
+    bx -= b.wholeTotal;
+    while (i + 1 < b.count && bx >= b.item[i].splitEnd) ++i;
+    bx -= i > 0 ? b.item[i - 1].splitEnd : 0;
+    const int tail = b.item[i].p.tail;
+    by = bx / tail;
+    bx -= by * tail;
+  }
+  fwdPaddedBody<WM>(b.item[i].p, b.item[i].g, bx, by, whole);
 }
 
 // 16-byte load of data that is read exactly once (non-temporal hint: it does not displace what the caches hold)
@@ -1147,11 +1162,11 @@ fwdTailFixupKernel(FwdArgs p, ConvGeom g) {
   fwdTailFixupBody(p, g);
 }
 
-// the fold for the split items of a batch; grid = (most tiles of an item, BM*BN / 1024, items)
+// the fold for the split tiles of a batch; grid = (most split tiles of an item, BM*BN / 1024, items)
 __global__ void __launch_bounds__(dev::kBlock)
 fwdTailFixupBatchKernel(FwdBatch b) {
   const FwdBatchItem &it = b.item[blockIdx.z];
-  if ((int)blockIdx.x >= it.tiles || it.p.nSplit <= 1) return;
+  if ((int)blockIdx.x >= it.p.tail) return;
   fwdTailFixupBody(it.p, it.g);
 }
 
@@ -2135,26 +2150,62 @@ bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const
   const int bm = low ? 32 : wide ? 64 : BM, bn = low || wide ? 256 : BN;
   const int mTiles = (int)tiles(g.Cin, bm);
   struct Split {
-    int tiles, nSplit, ktPerSplit;
+    int tiles, tail, nSplit, ktPerSplit;  // the last `tail` of the item's tiles are split nSplit ways
     long partialOfs;
   } split[kMaxPhases];
   long partialTotal = 0;
   auto planAll = [&](int cnt) {
-    long units = 0;
+    const int cus = residentSlots(nullptr);
+    long units = 0, wgs = 0;
     for (int i = 0; i < set.count; ++i) {
       const Phase &P = set.ph[i];
       split[i].tiles = mTiles * (int)tiles((long)cnt * P.h.n * P.w.n, bn);
       units += (long)split[i].tiles * (P.Kp / BK);
     }
-    const long target = std::max<long>(4, units / (2L * residentSlots(nullptr)));  // k-tiles per workgroup
-    long total = 0;
+    const long target = std::max<long>(4, units / (2L * cus));  // k-tiles per workgroup
+    bool anySplit = false;
     for (int i = 0; i < set.count; ++i) {
       const int nkt = set.ph[i].Kp / BK;
       const int n = (int)std::max<long>(1, std::min<long>(nkt / 4, (nkt + target / 2) / target));
       split[i].ktPerSplit = launch::ceilDiv(nkt, n);
       split[i].nSplit = launch::ceilDiv(nkt, split[i].ktPerSplit);
+      split[i].tail = split[i].nSplit > 1 ? split[i].tiles : 0;
+      anySplit = anySplit || split[i].nSplit > 1;
+      wgs += split[i].tiles;
+    }
+    // No phase is heavy enough to be split by that rule, and the whole tiles fill the CUs once or more with a
+    // partial round left over (4 equal phases of a 4x4 stride-2 layer: 392 tiles on 256 CUs): the tiles of that
+    // last round - the end of the launch order - are split along K like the tail of a single forward pass
+    // (planTiles: same cost model, the k-tiles of the heaviest phase in the tail).
+    const int q = (int)(wgs / cus), r = (int)(wgs % cus);
+    if (!anySplit && q > 0 && r > 0) {
+      int first = set.count - 1;  // first item with tiles in the tail
+      for (int left = r; first > 0 && left > split[first].tiles; --first) left -= split[first].tiles;
+      const int nktTail = set.ph[first].Kp / BK, nktHead = set.ph[0].Kp / BK;
+      auto perWg = [&](int nkt, int S) { return (double)launch::ceilDiv(nkt, S) + 4.0; };
+      double best = 0.95 * (q + 1) * perWg(nktHead, 1);
+      int S = 1;
+      for (int c = 2; c <= std::max(1, std::min(nktTail / 4, 16)); ++c) {
+        if (launch::ceilDiv(nktTail, launch::ceilDiv(nktTail, c)) != c) continue;
+        const double t = q * perWg(nktHead, 1) + launch::ceilDiv(r * c, cus) * perWg(nktTail, c) + 0.006 * r * c;
+        if (t < best) best = t, S = c;
+      }
+      if (S > 1) {
+        int left = r;
+        for (int i = set.count - 1; i >= 0 && left > 0; --i) {
+          const int nkt = set.ph[i].Kp / BK;
+          split[i].tail = std::min(left, split[i].tiles);
+          left -= split[i].tail;
+          split[i].ktPerSplit = launch::ceilDiv(nkt, std::min(S, std::max(1, nkt / 4)));
+          split[i].nSplit = launch::ceilDiv(nkt, split[i].ktPerSplit);
+          if (split[i].nSplit <= 1) split[i].tail = 0;
+        }
+      }
+    }
+    long total = 0;
+    for (int i = 0; i < set.count; ++i) {
       split[i].partialOfs = total;
-      if (split[i].nSplit > 1) total += (long)split[i].tiles * split[i].nSplit * BM * BN;
+      total += (long)split[i].tail * split[i].nSplit * BM * BN;
     }
     partialTotal = std::max(partialTotal, total);
   };
@@ -2185,7 +2236,8 @@ bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const
       src = gyp;
     }
     FwdBatch batch{};
-    int maxTiles = 0, maxSplit = 1;
+    batch.count = set.count;
+    int maxTail = 0, wholeTotal = 0, splitTotal = 0;
     for (int i = 0; i < set.count; ++i) {
       const Phase &P = set.ph[i];
       FwdBatchItem &it = batch.item[i];
@@ -2214,13 +2266,17 @@ bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const
       a.wBytes = (int)((long)g.Cin * P.Kp * 4);
       a.vecA = true;
       a.mTiles = mTiles, a.bm = bm, a.bn = bn;
-      a.tile0 = 0;
-      a.nSplit = split[i].nSplit, a.ktPerSplit = split[i].ktPerSplit;
+      a.tail = split[i].tail, a.full = split[i].tiles - split[i].tail;
+      a.tile0 = a.full;
+      a.nSplit = a.tail > 0 ? split[i].nSplit : 1;
+      a.ktPerSplit = a.tail > 0 ? split[i].ktPerSplit : P.Kp / BK;
       a.partial = partial + split[i].partialOfs;
-      it.tiles = split[i].tiles;
-      maxTiles = std::max(maxTiles, it.tiles), maxSplit = std::max(maxSplit, a.nSplit);
+      wholeTotal += a.full, splitTotal += a.tail * a.nSplit;
+      it.wholeEnd = wholeTotal, it.splitEnd = splitTotal;
+      maxTail = std::max(maxTail, a.tail);
     }
-    const dim3 grid(maxTiles, maxSplit, set.count);
+    batch.wholeTotal = wholeTotal;
+    const dim3 grid(wholeTotal + splitTotal);
     if (low)
       convFwdPaddedBatchKernel<0><<<grid, dev::kBlock, 0, s>>>(batch);
     else if (wide)
@@ -2228,8 +2284,8 @@ bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const
     else
       convFwdPaddedBatchKernel<2><<<grid, dev::kBlock, 0, s>>>(batch);
     THC_HIP_CHECK(hipGetLastError());
-    if (maxSplit > 1) {
-      fwdTailFixupBatchKernel<<<dim3(maxTiles, BM * BN / (4 * dev::kBlock), set.count), dev::kBlock, 0, s>>>(batch);
+    if (maxTail > 0) {
+      fwdTailFixupBatchKernel<<<dim3(maxTail, BM * BN / (4 * dev::kBlock), set.count), dev::kBlock, 0, s>>>(batch);
       THC_HIP_CHECK(hipGetLastError());
     }
   }

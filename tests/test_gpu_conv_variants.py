@@ -205,6 +205,25 @@ def test_full_convolution(T, case):
     _full_run(T, case)
 
 
+def test_full_convolution_phases_with_split_last_round(T):
+    """The four phases of a 4x4 stride-2 transposed convolution run as one batched launch; with 392 tiles of
+    128 x 128 and 48 k-tiles each on 256 CUs, the tiles past the first full round (the last images of the last
+    two phases) are split along K and folded. First and last images against the oracle."""
+    THNN, CT = T.THNN, T.CudaTensor
+    N, Cin, Cout, H, k = 64, 192, 128, 14, 4
+    rng = np.random.default_rng(92)
+    x = rng.standard_normal((N, Cin, H, H)).astype(np.float32)
+    w = (rng.standard_normal((Cin, Cout, k, k)) * np.sqrt(2.0 / (Cin * k * k))).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    out = CT()
+    THNN.SpatialFullConvolution_updateOutput(CT.from_numpy(x), out, CT.from_numpy(w), CT.from_numpy(b), CT(), CT(),
+                                             k, k, 2, 2, 1, 1, 0, 0)
+    y = out.numpy()
+    assert y.shape == (N, Cout, 2 * H, 2 * H)
+    for n in (0, 1, 31, 32, 62, 63):
+        close(y[n:n + 1], O.fullconv_updateOutput(x[n:n + 1], w, b, k, k, 2, 2, 1, 1, 1, 1, 0, 0))
+
+
 def test_full_convolution_variants(T):
     rng = np.random.default_rng(91)
     _full_run(T, FULL_CASES[0], bias=False, scale=0.5, dilated_entry=False)

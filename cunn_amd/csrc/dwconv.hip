@@ -467,7 +467,14 @@ dwFwdStrip(const float *__restrict__ in, const float *__restrict__ weight, Strid
 #pragma unroll
           for (int q = 0; q < 4; ++q) acc[q] = fmaf(win[q * ST + kw], w[kh * KS + kw], acc[q]);
       }
-      dev::bufStoreStream4(orr, i * 16, make_float4(acc[0], acc[1], acc[2], acc[3]));  // r * oW + b4 * 4 = 4 i
+      // Stride 2 writes a fifth of what it moves: plain stores cost this pass nothing (a 4:1 stream measures the
+      // same with either kind), and they leave the output in the Infinity Cache for the layer that reads it next
+      // (BatchNormalization behind this pass: 11.8 -> 10.0 us at N 64, 128 x 28 x 28). At stride 1 half of the
+      // traffic is stores and streaming stores are 8 % faster.
+      if (ST == 2)
+        dev::bufStore4(orr, i * 16, make_float4(acc[0], acc[1], acc[2], acc[3]));
+      else
+        dev::bufStoreStream4(orr, i * 16, make_float4(acc[0], acc[1], acc[2], acc[3]));  // r * oW + b4 * 4 = 4 i
     }
   }
 }

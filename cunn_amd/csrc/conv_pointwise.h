@@ -199,7 +199,10 @@ convPointwiseKernel(PwArgs p) {
     float o = d.acc[q][r][v];
     // one instruction between the MFMAs: max(v, 0) is v > 0 ? v : 0 for every input (a NaN gives 0, -0 gives +0)
     if (RELU) asm volatile("v_max_f32 %0, 0, %1" : "=v"(o) : "v"(o));
-    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(o), outr, d.voff[q][r][v >> 2], rowBase * p.L * 4, 0);
+    // K >= 64: streaming stores (the nt policy bit). Measured at N = 64: 64 -> 128 at 56 x 56 54.2 -> 43.6 us, 64 -> 64
+    // 33.7 -> 27.1 us, 128 -> 128 at 56 x 56 77.2 -> 73.5 us, at 28 x 28 24.2 -> 22.4 us; at K = 32 plain stores are level
+    // or better (32 -> 64 at 112 x 112: 44.9 against 46.1 us).
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(o), outr, d.voff[q][r][v >> 2], rowBase * p.L * 4, K >= 64 ? 2 : 0);
   };
   // second operand of MFMA s of column tile ct: lane (j = lane % 32, kk = lane / 32) holds x[2s + kk][position j]
   auto bAddr = [&](int buf, int ct) {

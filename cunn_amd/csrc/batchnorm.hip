@@ -496,6 +496,8 @@ bnFwdResident(const float *__restrict__ x, float *__restrict__ y, const float *_
 // registers as well (2R float4 per lane). Otherwise x is consumed in batches; XL > 0: the first XL float4
 // of x per lane wait in LDS for the apply phase and the other R - XL in registers, so that x crosses HBM
 // once as well; XL == 0: nothing of x is kept (no apply phase, or one that does not need x).
+// x and gradOutput are read with the non-temporal hint: the backward pass is the last reader of both in a training
+// step (cfg3, N 64, 256 x 28 x 28: 27.0 -> 25.9 us per call, forward + backward step 46.0 -> 44.5 us).
 template <int R, bool TRAIN, bool KEEPX, int XL = 0>
 __global__ void __launch_bounds__(kResBlock)
 bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *__restrict__ gx,
@@ -528,8 +530,8 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
         xc[KEEPX ? u : 0] = make_float4(mean, mean, mean, mean);
         if (u * kResBlock + (int)threadIdx.x < total4) {
           const int off = wk.offset();
-          d[u] = dev::bufLoad4(gr, off);
-          xc[KEEPX ? u : 0] = dev::bufLoad4(xr, off);
+          d[u] = dev::bufLoadStream4(gr, off);
+          xc[KEEPX ? u : 0] = dev::bufLoadStream4(xr, off);
         }
         wk.next();
       }
@@ -547,7 +549,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
 #pragma unroll
       for (int u = 0; u < R; ++u) {
         d[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (u * kResBlock + (int)threadIdx.x < total4) d[u] = dev::bufLoad4(gr, wk.offset());
+        if (u * kResBlock + (int)threadIdx.x < total4) d[u] = dev::bufLoadStream4(gr, wk.offset());
         wk.next();
       }
 #pragma unroll
@@ -557,7 +559,7 @@ bnBwdResident(const float *__restrict__ x, const float *__restrict__ gy, float *
         for (int k = 0; k < XB; ++k) {
           q[k] = make_float4(mean, mean, mean, mean);
           if (u0 + k < R) {
-            if ((u0 + k) * kResBlock + (int)threadIdx.x < total4) q[k] = dev::bufLoad4(xr, wx.offset());
+            if ((u0 + k) * kResBlock + (int)threadIdx.x < total4) q[k] = dev::bufLoadStream4(xr, wx.offset());
             wx.next();
           }
         }

@@ -20,10 +20,16 @@ __global__ void __launch_bounds__(dev::kBlock)
 thresholdKernel4(const float *x, const float *other, float *out, long n4, float thr, float val) {
   const long i = (long)blockIdx.x * dev::kBlock + threadIdx.x;
   if (i >= n4) return;
-  const float4 a = reinterpret_cast<const float4 *>(x)[i];
+  // the backward pass is the last reader of the layer's input and of gradOutput: non-temporal loads
+  typedef float f32x4v __attribute__((ext_vector_type(4)));
+  auto loadOnce = [](const float *p, long at) {
+    const f32x4v v = __builtin_nontemporal_load(reinterpret_cast<const f32x4v *>(p) + at);
+    return make_float4(v.x, v.y, v.z, v.w);
+  };
+  const float4 a = GRAD ? loadOnce(x, i) : reinterpret_cast<const float4 *>(x)[i];
   float4 r;
   if (GRAD) {
-    const float4 g = reinterpret_cast<const float4 *>(other)[i];
+    const float4 g = loadOnce(other, i);
     r = make_float4(a.x > thr ? g.x : 0.f, a.y > thr ? g.y : 0.f, a.z > thr ? g.z : 0.f, a.w > thr ? g.w : 0.f);
   } else {
     r = make_float4(a.x > thr ? a.x : val, a.y > thr ? a.y : val, a.z > thr ? a.z : val, a.w > thr ? a.w : val);

@@ -568,6 +568,26 @@ padPlanesKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int 
 // 16-byte group of the whole destination. Workgroups past copyBlocks build the tap table.
 // ANY: planes of any size (9x9 = a bordered 7x7 plane): a group may straddle two planes and the last elements of
 // the destination may not fill a group.
+// The copy of padPlanesFlatKernel for planes of a multiple of 4 floats: workgroups 0 .. copyBlocks - 1 of a launch, a
+// lane per 16-byte group of the bordered planes.
+__device__ __forceinline__ void padFlatVecBody(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int padTop,
+                                               int padLeft, int Hp, int Wp, long total4, int copyBlocks) {
+  const int plane4 = (Hp * Wp) >> 2;
+  const unsigned magicPlane = dev::magicOf(plane4), magicW = dev::magicOf(Wp);
+  for (long i = (long)blockIdx.x * dev::kBlock + threadIdx.x; i < total4; i += (long)copyBlocks * dev::kBlock) {
+    const int pl = dev::fastDiv((int)i, magicPlane), j = ((int)i - pl * plane4) * 4;
+    const float *src = x + (long)pl * H * W;
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int hp = dev::fastDiv(j + k, magicW), wp = j + k - hp * Wp;
+      const int h = hp - padTop, w = wp - padLeft;
+      v[k] = (((unsigned)h < (unsigned)H) & ((unsigned)w < (unsigned)W)) ? src[h * W + w] : 0.f;
+    }
+    reinterpret_cast<float4 *>(xp)[i] = make_float4(v[0], v[1], v[2], v[3]);
+  }
+}
+
 template <bool ANY>
 __global__ void __launch_bounds__(dev::kBlock)
 padPlanesFlatKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int padTop, int padLeft, int Hp, int Wp,
@@ -602,20 +622,7 @@ padPlanesFlatKernel(const float *__restrict__ x, float *__restrict__ xp, int H, 
     }
     return;
   }
-  const int plane4 = (Hp * Wp) >> 2;
-  const unsigned magicPlane = dev::magicOf(plane4), magicW = dev::magicOf(Wp);
-  for (long i = (long)blockIdx.x * dev::kBlock + threadIdx.x; i < total4; i += (long)copyBlocks * dev::kBlock) {
-    const int pl = dev::fastDiv((int)i, magicPlane), j = ((int)i - pl * plane4) * 4;
-    const float *src = x + (long)pl * H * W;
-    float v[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int hp = dev::fastDiv(j + k, magicW), wp = j + k - hp * Wp;
-      const int h = hp - padTop, w = wp - padLeft;
-      v[k] = (((unsigned)h < (unsigned)H) & ((unsigned)w < (unsigned)W)) ? src[h * W + w] : 0.f;
-    }
-    reinterpret_cast<float4 *>(xp)[i] = make_float4(v[0], v[1], v[2], v[3]);
-  }
+  padFlatVecBody(x, xp, H, W, padTop, padLeft, Hp, Wp, total4, copyBlocks);
 }
 
 // taps != nullptr: the same launch also builds the tap table (tapEntries entries) of geometry tg
@@ -690,17 +697,18 @@ struct PhaseSet {
 // tap table of each phase: entry k = (o, a, b) is the byte offset of gy element (o, q0h - a*qStepH, q0w - b*qStepW) of
 // the bordered image, 0 from K on.
 // grid = (chunks of a weight row, Cin + 1, phases): blocks with blockIdx.y == Cin write the tap table.
-__global__ void __launch_bounds__(dev::kBlock)
-phaseSetupKernel(const float *__restrict__ w, float *__restrict__ dst, int *__restrict__ taps, PhaseSet set, int Cin, int kH,
-                 int kW, int Hp, int Wp, int top, int left) {
-  const Phase &P = set.ph[blockIdx.z];
+// (bx of gx, by, bz) = the workgroup's position in that grid
+__device__ __forceinline__ void phaseSetupBody(const float *__restrict__ w, float *__restrict__ dst, int *__restrict__ taps,
+                                               const PhaseSet &set, int Cin, int kH, int kW, int Hp, int Wp, int top, int left,
+                                               int bx, int gx, int by, int bz) {
+  const Phase &P = set.ph[bz];
   const int tp = P.h.nk * P.w.nk;
   const unsigned magicTp = dev::magicOf(tp), magicNk = dev::magicOf(P.w.nk);
-  const int c = blockIdx.y;
+  const int c = by;
   if (c == Cin) {
     const int entries = P.Kp + 2 * BK;
     int *d = taps + P.tapOfs;
-    for (int k = blockIdx.x * dev::kBlock + threadIdx.x; k < entries; k += gridDim.x * dev::kBlock) {
+    for (int k = bx * dev::kBlock + threadIdx.x; k < entries; k += gx * dev::kBlock) {
       int v = 0;
       if (k < P.K) {
         const int o = dev::fastDiv(k, magicTp), r = k - o * tp;
@@ -714,7 +722,7 @@ phaseSetupKernel(const float *__restrict__ w, float *__restrict__ dst, int *__re
   float *d = dst + P.wOfs + (long)c * P.Kp;
   const long oStride = (long)Cin * kH * kW;
   const float *src = w + ((long)c * kH + P.h.k0) * kW + P.w.k0;
-  for (int k = blockIdx.x * dev::kBlock + threadIdx.x; k < P.Kp; k += gridDim.x * dev::kBlock) {
+  for (int k = bx * dev::kBlock + threadIdx.x; k < P.Kp; k += gx * dev::kBlock) {
     float v = 0.f;
     if (k < P.K) {
       const int o = dev::fastDiv(k, magicTp), r = k - o * tp;
@@ -723,6 +731,29 @@ phaseSetupKernel(const float *__restrict__ w, float *__restrict__ dst, int *__re
     }
     d[k] = v;
   }
+}
+
+__global__ void __launch_bounds__(dev::kBlock)
+phaseSetupKernel(const float *__restrict__ w, float *__restrict__ dst, int *__restrict__ taps, PhaseSet set, int Cin, int kH,
+                 int kW, int Hp, int Wp, int top, int left) {
+  phaseSetupBody(w, dst, taps, set, Cin, kH, kW, Hp, Wp, top, left, blockIdx.x, gridDim.x, blockIdx.y, blockIdx.z);
+}
+
+// The bordered copy of gradOutput and the phase set-up in one launch (both are short: as two launches their latencies
+// add): workgroups 0 .. copyBlocks - 1 copy (planes of a multiple of 4 floats), the others are the set-up's grid
+// (chunks, Cin + 1, phases) laid out flat.
+__global__ void __launch_bounds__(dev::kBlock)
+padPlanesPhaseSetupKernel(const float *__restrict__ x, float *__restrict__ xp, int H, int W, int Hp, int Wp, int top, int left,
+                          long total4, int copyBlocks, const float *__restrict__ w, float *__restrict__ dst,
+                          int *__restrict__ taps, PhaseSet set, int Cin, int kH, int kW, int chunks) {
+  if ((int)blockIdx.x < copyBlocks) {
+    padFlatVecBody(x, xp, H, W, top, left, Hp, Wp, total4, copyBlocks);
+    return;
+  }
+  const int l = blockIdx.x - copyBlocks;
+  const int r = l / chunks, bx = l - r * chunks;
+  const int bz = r / (Cin + 1), by = r - bz * (Cin + 1);
+  phaseSetupBody(w, dst, taps, set, Cin, kH, kW, Hp, Wp, top, left, bx, chunks, by, bz);
 }
 
 // Generic forward kernel: any K, any alignment; taps and bounds resolved in the loop.
@@ -2218,20 +2249,31 @@ bool gradInputByPhase(THCState *state, const ConvGeom &g, const float *gy, const
   float *wph = buf + tapTotal;
   float *partial = wph + wTotal;
   float *gyp = partial + partialTotal;
-  {
-    int maxKp = 0;
-    for (int i = 0; i < set.count; ++i) maxKp = std::max(maxKp, set.ph[i].Kp);
-    if (g.Cin + 1 > 65535) return false;
-    const int chunks = std::max(1, std::min(8, launch::ceilDiv(maxKp + 2 * BK, 4 * dev::kBlock)));
+  int maxKp = 0;
+  for (int i = 0; i < set.count; ++i) maxKp = std::max(maxKp, set.ph[i].Kp);
+  if (g.Cin + 1 > 65535) return false;
+  const int chunks = std::max(1, std::min(8, launch::ceilDiv(maxKp + 2 * BK, 4 * dev::kBlock)));
+  // the set-up rides along with the first group's bordered copy when that copy has the flat 16-byte form
+  const long plane = Hp * Wp, firstTotal4 = (long)std::min(group, g.N) * g.Cout * (plane / 4);
+  const long setupBlocks = (long)chunks * (g.Cin + 1) * set.count;
+  const bool together = copy && plane % 4 == 0 && plane < 4096 && launch::aligned16(gyp) &&
+                        firstTotal4 * (plane / 4) < 0xffffffffL && setupBlocks < (1L << 24);
+  if (!together) {
     phaseSetupKernel<<<dim3(chunks, g.Cin + 1, set.count), dev::kBlock, 0, s>>>(w, wph, taps, set, g.Cin, g.kH, g.kW, (int)Hp,
                                                                               (int)Wp, top, left);
+    THC_HIP_CHECK(hipGetLastError());
   }
-  THC_HIP_CHECK(hipGetLastError());
   for (int n0 = 0; n0 < g.N; n0 += group) {
     const int cnt = std::min(group, g.N - n0);
     if (cnt != std::min(group, g.N)) planAll(cnt);
     const float *src = gy + (long)n0 * g.Cout * g.L;
-    if (copy) {
+    if (copy && together && n0 == 0) {
+      const int copyBlocks = (int)std::min<long>((firstTotal4 + dev::kBlock - 1) / dev::kBlock, 16384);
+      padPlanesPhaseSetupKernel<<<(unsigned)(copyBlocks + setupBlocks), dev::kBlock, 0, s>>>(
+          src, gyp, g.oH, g.oW, (int)Hp, (int)Wp, top, left, firstTotal4, copyBlocks, w, wph, taps, set, g.Cin, g.kH, g.kW, chunks);
+      THC_HIP_CHECK(hipGetLastError());
+      src = gyp;
+    } else if (copy) {
       launchPadPlanes(s, src, gyp, (long)cnt * g.Cout, g.oH, g.oW, top, left, (int)Hp, (int)Wp);
       src = gyp;
     }
